@@ -1,0 +1,167 @@
+// Builtin data-movement kernels: replicate, iota, copy and the batched 2-D
+// transpose.  They stand where the reference keeps builtin#replicate_* /
+// builtin#iota_* (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:1274-1436) and
+// map_transpose_{1,2,4,8}b (rts/opencl/transpose.cl, dispatch rts/c/gpu.h:333-461).
+#include "dispatch.hip.h"
+
+namespace fa {
+
+template <class T>
+__global__ __launch_bounds__(256) void replicate_kernel(T *dst, int64_t n, T v) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) dst[i] = v;
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void iota_kernel(T *dst, int64_t n, T start, T step) {
+  using U = typename std::make_unsigned<T>::type;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+    dst[i] = (T)((U)start + (U)i * (U)step);
+}
+
+// 16 bytes per lane per access, four accesses in flight.
+__global__ __launch_bounds__(256) void copy_kernel(uint4 *__restrict__ dst,
+                                                   const uint4 *__restrict__ src, int64_t nvec) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  for (; i + 3 * stride < nvec; i += 4 * stride) {
+    uint4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+    dst[i] = a;
+    dst[i + stride] = b;
+    dst[i + 2 * stride] = c;
+    dst[i + 3 * stride] = d;
+  }
+  for (; i < nvec; i += stride) dst[i] = src[i];
+}
+
+__global__ void copy_tail_kernel(uint8_t *dst, const uint8_t *src, int64_t from, int64_t n) {
+  const int64_t i = from + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+// dst[b][j][i] = src[b][i][j].  A 64x64 tile goes through LDS; rows are padded
+// by one element so that the column reads fall on distinct banks.  Both the
+// global reads and the global writes of a wave touch 64 consecutive elements.
+template <class T>
+__global__ __launch_bounds__(256) void transpose_kernel(T *__restrict__ dst,
+                                                        const T *__restrict__ src, int64_t rows,
+                                                        int64_t cols) {
+  constexpr int TS = 64;
+  __shared__ T tile[TS][TS + 1];
+  const int64_t b = blockIdx.z;
+  const int64_t r0 = (int64_t)blockIdx.y * TS, c0 = (int64_t)blockIdx.x * TS;
+  const T *s = src + b * rows * cols;
+  T *d = dst + b * rows * cols;
+  const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;  // 64 x 4
+#pragma unroll 4
+  for (int i = ty; i < TS; i += 4) {
+    const int64_t r = r0 + i, c = c0 + tx;
+    if (r < rows && c < cols) tile[i][tx] = s[r * cols + c];
+  }
+  __syncthreads();
+#pragma unroll 4
+  for (int i = ty; i < TS; i += 4) {
+    const int64_t c = c0 + i, r = r0 + tx;
+    if (r < rows && c < cols) d[c * rows + r] = tile[tx][i];
+  }
+}
+
+static int grid_for(int64_t n, int per_block) {
+  int64_t g = ceil_div(n, per_block);
+  if (g < 1) g = 1;
+  if (g > 256 * 16) g = 256 * 16;
+  return (int)g;
+}
+
+template <class T>
+static int launch_transpose(hipStream_t s, void *dst, const void *src, int64_t batch,
+                            int64_t rows, int64_t cols) {
+  const int64_t gx = ceil_div(cols, 64), gy = ceil_div(rows, 64);
+  if (gx > INT32_MAX || gy > 65535 || batch > 65535) return FA_EINVAL;
+  hipLaunchKernelGGL((transpose_kernel<T>), dim3((unsigned)gx, (unsigned)gy, (unsigned)batch),
+                     dim3(256), 0, s, (T *)dst, (const T *)src, rows, cols);
+  return launch_status();
+}
+
+}  // namespace fa
+
+extern "C" int fa_replicate(fa_stream_t stream, int elem_bytes, void *dst, int64_t n,
+                            uint64_t pattern) {
+  if (n < 0 || (n > 0 && dst == nullptr)) return FA_EINVAL;
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int g = grid_for(n, 256 * 4);
+  switch (elem_bytes) {
+    case 1: hipLaunchKernelGGL((replicate_kernel<uint8_t>), dim3(g), dim3(256), 0, s, (uint8_t *)dst, n, (uint8_t)pattern); break;
+    case 2: hipLaunchKernelGGL((replicate_kernel<uint16_t>), dim3(g), dim3(256), 0, s, (uint16_t *)dst, n, (uint16_t)pattern); break;
+    case 4: hipLaunchKernelGGL((replicate_kernel<uint32_t>), dim3(g), dim3(256), 0, s, (uint32_t *)dst, n, (uint32_t)pattern); break;
+    case 8: hipLaunchKernelGGL((replicate_kernel<uint64_t>), dim3(g), dim3(256), 0, s, (uint64_t *)dst, n, (uint64_t)pattern); break;
+    default: return FA_ENOTSUP;
+  }
+  return launch_status();
+}
+
+extern "C" int fa_iota(fa_stream_t stream, fa_dtype t, void *dst, int64_t n, int64_t start,
+                       int64_t step) {
+  if (n < 0 || (n > 0 && dst == nullptr)) return FA_EINVAL;
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int g = grid_for(n, 256 * 4);
+  switch (t) {
+    case FA_I32: case FA_U32:
+      hipLaunchKernelGGL((iota_kernel<int32_t>), dim3(g), dim3(256), 0, s, (int32_t *)dst, n, (int32_t)start, (int32_t)step);
+      break;
+    case FA_I64: case FA_U64:
+      hipLaunchKernelGGL((iota_kernel<int64_t>), dim3(g), dim3(256), 0, s, (int64_t *)dst, n, start, step);
+      break;
+    default: return FA_ENOTSUP;
+  }
+  return launch_status();
+}
+
+extern "C" int fa_copy(fa_stream_t stream, void *dst, const void *src, size_t bytes) {
+  if (bytes > 0 && (dst == nullptr || src == nullptr)) return FA_EINVAL;
+  if (bytes == 0) return 0;
+  if (!is_aligned(dst, 16) || !is_aligned(src, 16)) return FA_EALIGN;
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t nvec = (int64_t)(bytes / 16);
+  if (nvec > 0) {
+    hipLaunchKernelGGL(copy_kernel, dim3(grid_for(nvec, 256 * 4)), dim3(256), 0, s, (uint4 *)dst,
+                       (const uint4 *)src, nvec);
+  }
+  if (bytes % 16) {
+    hipLaunchKernelGGL(copy_tail_kernel, dim3(1), dim3(16), 0, s, (uint8_t *)dst,
+                       (const uint8_t *)src, nvec * 16, (int64_t)bytes);
+  }
+  return launch_status();
+}
+
+extern "C" int fa_map_transpose(fa_stream_t stream, int elem_bytes, void *dst, const void *src,
+                                int64_t batch, int64_t rows, int64_t cols) {
+  if (batch < 0 || rows < 0 || cols < 0) return FA_EINVAL;
+  if (batch * rows * cols == 0) return 0;
+  if (dst == nullptr || src == nullptr) return FA_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (elem_bytes) {
+    case 1: return launch_transpose<uint8_t>(s, dst, src, batch, rows, cols);
+    case 2: return launch_transpose<uint16_t>(s, dst, src, batch, rows, cols);
+    case 4: return launch_transpose<uint32_t>(s, dst, src, batch, rows, cols);
+    case 8: return launch_transpose<uint64_t>(s, dst, src, batch, rows, cols);
+    default: return FA_ENOTSUP;
+  }
+}
+
+extern "C" int fa_version(void) { return 1000; }
+
+extern "C" const char *fa_strerror(int code) {
+  if (code == 0) return "success";
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  switch (code) {
+    case FA_EINVAL: return "invalid argument";
+    case FA_ENOTSUP: return "element type / operator combination not supported";
+    case FA_ESCRATCH: return "scratch buffer too small";
+    case FA_EALIGN: return "pointer not sufficiently aligned";
+    default: return "unknown error";
+  }
+}

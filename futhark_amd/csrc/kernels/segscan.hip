@@ -1,0 +1,464 @@
+// SegScan for gfx950: single-pass scan with decoupled look-back, plus the
+// irregular segmented reduction that shares its machinery.
+//
+// What is computed follows src/Futhark/CodeGen/ImpGen/GPU/SegScan/SinglePass.hs
+// (dynamic tile ids :443-461, tile aggregate/prefix publication with status
+// X/A/P :128-131,625-777) and, for segments, the flag-tuple operator of
+// src/Futhark/Pass/Flatten/Builtins.hs:374-393.  How it is computed is native
+// to CDNA4:
+//   * every wave owns a contiguous chunk; each load/store instruction of a wave
+//     covers 1 KiB of consecutive bytes (128 bits per lane), so no LDS
+//     transpose is needed to coalesce;
+//   * scans inside a wave use DPP row shifts and broadcasts over all 64 lanes;
+//   * a tile descriptor is a 64-bit word {value bits, epoch, segment flag,
+//     status} written and read with single relaxed agent-scope accesses, so no
+//     fence separates value and status.  8-byte element types use two such
+//     words (low and high half), accepted only when both carry the same status;
+//   * descriptors carry a launch epoch, so no kernel clears them between calls;
+//   * the look-back window is a full 64-lane wave.
+#include "dispatch.hip.h"
+
+namespace fa {
+
+constexpr int SCAN_ROWS = 4;
+constexpr int SCAN_WAVES = 4;
+constexpr int SCAN_BLOCK = SCAN_WAVES * WAVE;
+static_assert(SCAN_WAVES >= 4, "the irregular reduction runs four searches on four waves");
+
+constexpr uint32_t ST_X = 0;  // nothing published
+constexpr uint32_t ST_A = 1;  // aggregate of the tile
+constexpr uint32_t ST_P = 2;  // inclusive prefix up to the end of the tile
+
+constexpr size_t SCAN_HEADER_BYTES = 256;  // ticket counter, padded
+constexpr size_t SCAN_DESC_BYTES = 16;     // per tile
+
+template <class T> constexpr int scan_tile_elems() {
+  return SCAN_BLOCK * SCAN_ROWS * Vec16<T>::N;
+}
+
+__device__ __forceinline__ uint32_t desc_meta(uint32_t epoch, uint32_t flag, uint32_t status) {
+  return (epoch << 3) | ((flag & 1u) << 2) | status;
+}
+
+template <class T>
+__device__ __forceinline__ void desc_publish(uint64_t *desc, int64_t tile, uint32_t epoch,
+                                             uint32_t status, uint32_t flag, T v) {
+  const uint32_t meta = desc_meta(epoch, flag, status);
+  if constexpr (sizeof(T) == 4) {
+    st_relaxed_u64(desc + 2 * tile, ((uint64_t)bit_cast<uint32_t>(v) << 32) | meta);
+  } else {
+    const uint64_t b = bit_cast<uint64_t>(v);
+    st_relaxed_u64(desc + 2 * tile, ((b & 0xffffffffull) << 32) | meta);
+    st_relaxed_u64(desc + 2 * tile + 1, ((b >> 32) << 32) | meta);
+  }
+}
+
+// Returns false while the tile has published nothing (for this epoch), or
+// while the two halves of an 8-byte value belong to different publications.
+template <class T>
+__device__ __forceinline__ bool desc_read(const uint64_t *desc, int64_t tile, uint32_t epoch,
+                                          uint32_t &status, uint32_t &flag, T &v) {
+  const uint64_t w0 = ld_relaxed_u64(desc + 2 * tile);
+  const uint32_t m0 = (uint32_t)w0;
+  if ((m0 >> 3) != epoch || (m0 & 3u) == ST_X) return false;
+  if constexpr (sizeof(T) == 4) {
+    v = bit_cast<T>((uint32_t)(w0 >> 32));
+  } else {
+    const uint64_t w1 = ld_relaxed_u64(desc + 2 * tile + 1);
+    if ((uint32_t)w1 != m0) return false;
+    v = bit_cast<T>((w0 >> 32) | ((w1 >> 32) << 32));
+  }
+  status = m0 & 3u;
+  flag = (m0 >> 2) & 1u;
+  return true;
+}
+
+// First index i in [0,m] for which pred(i) holds, pred monotone (false..true);
+// a 64-ary search run by one whole wave.
+template <class Pred>
+__device__ __forceinline__ int64_t wave_search_first(int64_t m, int lane, Pred pred) {
+  int64_t lo = 0, hi = m;
+  while (hi > lo) {
+    const int64_t span = hi - lo;
+    const int64_t step = (span + WAVE - 1) / WAVE;
+    const int64_t p = lo + (int64_t)lane * step;
+    const bool t = (p < hi) ? pred(p) : true;
+    const uint64_t mask = __ballot(t);
+    const int L = mask ? __builtin_ctzll(mask) : WAVE;
+    if (L == 0) return lo;
+    const int64_t nhi = lo + (int64_t)L * step;
+    lo = lo + (int64_t)(L - 1) * step + 1;
+    hi = nhi < hi ? nhi : hi;
+  }
+  return lo;
+}
+
+enum { MODE_SCAN = 0, MODE_SEGRED = 1 };
+
+// MODE_SCAN  : out[n], flags optional (SEG), EXCL selects the exclusive form.
+// MODE_SEGRED: flags are derived from `offsets`; out[m] receives the scanned
+//              value at the last element of each segment (ne for empty ones).
+template <class T, class Op, bool SEG, bool EXCL, int MODE>
+__global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
+    const T *__restrict__ xs, const uint8_t *__restrict__ flags, int64_t n, T *__restrict__ out,
+    uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles,
+    const int64_t *__restrict__ offsets, const int64_t *__restrict__ lens, int64_t m) {
+  constexpr int VEC = Vec16<T>::N;
+  constexpr int WCHUNK = SCAN_ROWS * WAVE * VEC;
+  constexpr int TILE = SCAN_WAVES * WCHUNK;
+  using Pair = SegPair<T>;
+
+  __shared__ int64_t s_tile;
+  __shared__ T s_wv[SCAN_WAVES];
+  __shared__ uint32_t s_wf[SCAN_WAVES];
+  __shared__ T s_pv;
+  __shared__ uint32_t s_pf;
+  __shared__ uint32_t s_bits[MODE == MODE_SEGRED ? TILE / 32 : 1];
+  __shared__ int64_t s_bounds[4];
+  __shared__ T s_vals[MODE == MODE_SEGRED ? TILE : 1];
+
+  if (threadIdx.x == 0) {
+    const uint32_t t = atomicAdd(ticket, 1u);
+    s_tile = (int64_t)t;
+    // The last ticket of this launch has been drawn: rearm for the next one.
+    if ((int64_t)t == num_tiles - 1) st_relaxed_u32(ticket, 0u);
+  }
+  if constexpr (MODE == MODE_SEGRED) {
+    for (int i = threadIdx.x; i < TILE / 32; i += SCAN_BLOCK) s_bits[i] = 0u;
+  }
+  __syncthreads();
+  // Tile and wave numbers are the same in all lanes; say so to the compiler.
+  const int64_t tile = (int64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile);
+  const int lane = lane_id();
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / WAVE));
+  const int64_t t0 = tile * TILE;
+  const int64_t wbase = t0 + (int64_t)wave * WCHUNK;
+
+  // ---- load: row r of a wave is 64 lanes x 16 bytes of consecutive memory.
+  T x[SCAN_ROWS][VEC];
+  uint32_t fm[SCAN_ROWS];
+#pragma unroll
+  for (int r = 0; r < SCAN_ROWS; r++) {
+    const int64_t idx = wbase + (int64_t)(r * WAVE + lane) * VEC;
+    fm[r] = 0u;
+    if (idx + VEC <= n) {
+      Vec16<T> v = load_vec16_nt(xs + idx);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) x[r][e] = v.e[e];
+      if constexpr (SEG && MODE == MODE_SCAN) {
+        if constexpr (VEC == 4) {
+          const uint32_t w = *reinterpret_cast<const uint32_t *>(flags + idx);
+#pragma unroll
+          for (int e = 0; e < 4; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+        } else {
+          const uint32_t w = *reinterpret_cast<const uint16_t *>(flags + idx);
+#pragma unroll
+          for (int e = 0; e < 2; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; e++) {
+        const bool in = idx + e < n;
+        x[r][e] = in ? xs[idx + e] : Op::identity();
+        if constexpr (SEG && MODE == MODE_SCAN) {
+          if (in && flags[idx + e] != 0) fm[r] |= 1u << e;
+        }
+      }
+    }
+  }
+
+  // ---- irregular reduction: find the segments that start / end in this tile
+  //      and turn their start offsets into flag bits.
+  int64_t e_first = 0, e_last = 0;
+  if constexpr (MODE == MODE_SEGRED) {
+    const int64_t t1 = (t0 + TILE < n) ? t0 + TILE : n;
+    int64_t r;
+    if (wave == 0) {
+      r = wave_search_first(m, lane, [&](int64_t i) { return offsets[i] >= t0; });
+    } else if (wave == 1) {
+      r = wave_search_first(m, lane, [&](int64_t i) { return offsets[i] >= t1; });
+    } else if (wave == 2) {
+      r = (tile == 0) ? 0
+                      : wave_search_first(
+                            m, lane, [&](int64_t i) { return offsets[i] + lens[i] > t0; });
+    } else if (wave == 3) {
+      r = wave_search_first(m, lane, [&](int64_t i) { return offsets[i] + lens[i] > t1; });
+    } else {
+      r = 0;
+    }
+    if (lane == 0 && wave < 4) s_bounds[wave] = r;
+    __syncthreads();
+    const int64_t s_first = s_bounds[0], s_last = s_bounds[1];
+    e_first = s_bounds[2];
+    e_last = s_bounds[3];
+    for (int64_t i = s_first + threadIdx.x; i < s_last; i += SCAN_BLOCK) {
+      const int64_t p = offsets[i] - t0;
+      if ((uint64_t)p < (uint64_t)TILE) atomicOr(&s_bits[p >> 5], 1u << (p & 31));
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r2 = 0; r2 < SCAN_ROWS; r2++) {
+      const int p = wave * WCHUNK + (r2 * WAVE + lane) * VEC;
+      fm[r2] = (s_bits[p >> 5] >> (p & 31)) & ((1u << VEC) - 1u);
+    }
+  }
+
+  // ---- scan inside each thread's VEC consecutive elements.
+#pragma unroll
+  for (int r = 0; r < SCAN_ROWS; r++) {
+#pragma unroll
+    for (int e = 1; e < VEC; e++) {
+      if constexpr (SEG) {
+        x[r][e] = ((fm[r] >> e) & 1u) ? x[r][e] : Op::apply(x[r][e - 1], x[r][e]);
+      } else {
+        x[r][e] = Op::apply(x[r][e - 1], x[r][e]);
+      }
+    }
+  }
+
+  // ---- scan across lanes per row, then chain the rows of the wave.
+  Pair pre[SCAN_ROWS];  // what precedes this lane's elements inside the wave
+  Pair carry = {Op::identity(), 0u};
+#pragma unroll
+  for (int r = 0; r < SCAN_ROWS; r++) {
+    Pair incl, excl;
+    if constexpr (SEG) {
+      Pair tot = {x[r][VEC - 1], fm[r] ? 1u : 0u};
+      incl = wave_incl_scan_seg<T, Op>(tot);
+      excl.v = wave_shift_up1<T, Op>(incl.v);
+      excl.f = dpp_move<DPP_WAVE_SHR1, 0xf>(0u, incl.f);
+      pre[r] = seg_apply<T, Op>(carry, excl);
+      Pair rowtot = {read_lane(incl.v, 63), read_lane(incl.f, 63)};
+      carry = seg_apply<T, Op>(carry, rowtot);
+    } else {
+      incl.v = wave_incl_scan<T, Op>(x[r][VEC - 1]);
+      excl.v = wave_shift_up1<T, Op>(incl.v);
+      pre[r].v = Op::apply(carry.v, excl.v);
+      pre[r].f = 0u;
+      carry.v = Op::apply(carry.v, read_lane(incl.v, 63));
+    }
+  }
+  if (lane == 63) {
+    s_wv[wave] = carry.v;
+    s_wf[wave] = carry.f;
+  }
+  __syncthreads();
+
+  Pair wp = {Op::identity(), 0u};  // what precedes this wave inside the tile
+  Pair bt = {Op::identity(), 0u};  // tile aggregate
+#pragma unroll
+  for (int w = 0; w < SCAN_WAVES; w++) {
+    if (w == wave) wp = bt;
+    Pair t = {s_wv[w], SEG ? s_wf[w] : 0u};
+    if constexpr (SEG) bt = seg_apply<T, Op>(bt, t);
+    else bt.v = Op::apply(bt.v, t.v);
+  }
+
+  // ---- publish the aggregate, look back for the exclusive prefix of the tile.
+  if (wave == 0) {
+    Pair acc = {Op::identity(), 0u};
+    if (tile == 0) {
+      if (lane == 0) desc_publish<T>(desc, tile, epoch, ST_P, bt.f, bt.v);
+    } else {
+      // A tile that contains a segment start already knows its inclusive
+      // prefix: nothing before the start can reach past it.
+      const bool self_contained = SEG && bt.f;
+      if (lane == 0)
+        desc_publish<T>(desc, tile, epoch, self_contained ? ST_P : ST_A, bt.f, bt.v);
+      int64_t j = tile - 1;
+      while (true) {
+        const int64_t idx = j - (WAVE - 1) + lane;
+        uint32_t st = ST_P, fl = 0u;
+        T v = Op::identity();
+        if (idx >= 0) {
+          while (!desc_read<T>(desc, idx, epoch, st, fl, v)) __builtin_amdgcn_s_sleep(1);
+        }
+        const bool term = (st == ST_P) || (SEG && fl);
+        const uint64_t mask = __ballot(term);
+        Pair mine = {v, SEG ? fl : 0u};
+        if (mask) {
+          const int first = 63 - __builtin_clzll(mask);
+          if (lane < first) {
+            mine.v = Op::identity();
+            mine.f = 0u;
+          }
+        }
+        Pair win;
+        if constexpr (SEG) {
+          Pair sc = wave_incl_scan_seg<T, Op>(mine);
+          win.v = read_lane(sc.v, 63);
+          win.f = read_lane(sc.f, 63);
+          acc = seg_apply<T, Op>(win, acc);
+        } else {
+          win.v = read_lane(wave_incl_scan<T, Op>(mine.v), 63);
+          acc.v = Op::apply(win.v, acc.v);
+        }
+        if (mask) break;
+        j -= WAVE;
+      }
+      if (lane == 0 && !self_contained) {
+        Pair inc;
+        if constexpr (SEG) inc = seg_apply<T, Op>(acc, bt);
+        else { inc.v = Op::apply(acc.v, bt.v); inc.f = 0u; }
+        desc_publish<T>(desc, tile, epoch, ST_P, inc.f, inc.v);
+      }
+    }
+    if (lane == 0) {
+      s_pv = acc.v;
+      s_pf = acc.f;
+    }
+  }
+  __syncthreads();
+
+  Pair base = {s_pv, SEG ? s_pf : 0u};
+  if constexpr (SEG) base = seg_apply<T, Op>(base, wp);
+  else base.v = Op::apply(base.v, wp.v);
+
+  // ---- apply the prefix and write.
+#pragma unroll
+  for (int r = 0; r < SCAN_ROWS; r++) {
+    T pv;
+    if constexpr (SEG) pv = seg_apply<T, Op>(base, pre[r]).v;
+    else pv = Op::apply(base.v, pre[r].v);
+
+    Vec16<T> o;
+    uint32_t seen = 0u;
+    T prev = pv;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+      const uint32_t fbit = SEG ? ((fm[r] >> e) & 1u) : 0u;
+      seen |= fbit;
+      const T incl = (SEG && seen) ? x[r][e] : Op::apply(pv, x[r][e]);
+      if constexpr (EXCL) o.e[e] = fbit ? Op::identity() : prev;
+      else o.e[e] = incl;
+      prev = incl;
+    }
+
+    if constexpr (MODE == MODE_SCAN) {
+      const int64_t idx = wbase + (int64_t)(r * WAVE + lane) * VEC;
+      if (idx + VEC <= n) {
+        store_vec16_nt(out + idx, o);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+          if (idx + e < n) out[idx + e] = o.e[e];
+      }
+    } else {
+      const int p = wave * WCHUNK + (r * WAVE + lane) * VEC;
+#pragma unroll
+      for (int e = 0; e < VEC; e++) s_vals[p + e] = o.e[e];
+    }
+  }
+
+  if constexpr (MODE == MODE_SEGRED) {
+    __syncthreads();
+    for (int64_t i = e_first + threadIdx.x; i < e_last; i += SCAN_BLOCK) {
+      const int64_t len = lens[i];
+      const int64_t p = offsets[i] + len - 1 - t0;
+      out[i] = (len == 0 || (uint64_t)p >= (uint64_t)TILE) ? Op::identity() : s_vals[p];
+    }
+  }
+}
+
+template <class T> static int64_t scan_num_tiles(int64_t n) {
+  return ceil_div(n, (int64_t)scan_tile_elems<T>());
+}
+
+template <class T, class Op>
+static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int64_t n,
+                       int exclusive, void *out, void *scratch, size_t scratch_bytes,
+                       uint32_t epoch) {
+  if (n == 0) return 0;
+  const int64_t tiles = scan_num_tiles<T>(n);
+  if (scratch_bytes < SCAN_HEADER_BYTES + (size_t)tiles * SCAN_DESC_BYTES) return FA_ESCRATCH;
+  if (!is_aligned(xs, 16) || !is_aligned(out, 16) || !is_aligned(scratch, 16) ||
+      (flags && !is_aligned(flags, 4)))
+    return FA_EALIGN;
+  if (tiles > INT32_MAX) return FA_EINVAL;
+  uint32_t *ticket = (uint32_t *)scratch;
+  uint64_t *desc = (uint64_t *)((char *)scratch + SCAN_HEADER_BYTES);
+  const dim3 grid((unsigned)tiles), block(SCAN_BLOCK);
+#define FA_LAUNCH(SEGV, EXV)                                                              \
+  hipLaunchKernelGGL((segscan_kernel<T, Op, SEGV, EXV, MODE_SCAN>), grid, block, 0, s,   \
+                     (const T *)xs, flags, n, (T *)out, ticket, desc, epoch, tiles,       \
+                     (const int64_t *)nullptr, (const int64_t *)nullptr, (int64_t)0)
+  if (flags) {
+    if (exclusive) FA_LAUNCH(true, true);
+    else FA_LAUNCH(true, false);
+  } else {
+    if (exclusive) FA_LAUNCH(false, true);
+    else FA_LAUNCH(false, false);
+  }
+#undef FA_LAUNCH
+  return launch_status();
+}
+
+template <class T>
+__global__ void fill_kernel(T *dst, int64_t n, T v) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (int64_t)gridDim.x * blockDim.x)
+    dst[i] = v;
+}
+
+template <class T, class Op>
+static int launch_segred_irregular(hipStream_t s, const void *vs, int64_t n,
+                                   const int64_t *offsets, const int64_t *lens, int64_t m,
+                                   void *out, void *scratch, size_t scratch_bytes,
+                                   uint32_t epoch) {
+  if (m == 0) return 0;
+  if (n == 0) {
+    // Every segment is empty.
+    int grid = (int)(ceil_div(m, 256) < 4096 ? ceil_div(m, 256) : 4096);
+    hipLaunchKernelGGL((fill_kernel<T>), dim3(grid), dim3(256), 0, s, (T *)out, m,
+                       Op::identity());
+    return launch_status();
+  }
+  const int64_t tiles = scan_num_tiles<T>(n);
+  if (scratch_bytes < SCAN_HEADER_BYTES + (size_t)tiles * SCAN_DESC_BYTES) return FA_ESCRATCH;
+  if (!is_aligned(vs, 16) || !is_aligned(scratch, 16) || !is_aligned(offsets, 8) ||
+      !is_aligned(lens, 8))
+    return FA_EALIGN;
+  if (tiles > INT32_MAX) return FA_EINVAL;
+  uint32_t *ticket = (uint32_t *)scratch;
+  uint64_t *desc = (uint64_t *)((char *)scratch + SCAN_HEADER_BYTES);
+  hipLaunchKernelGGL((segscan_kernel<T, Op, true, false, MODE_SEGRED>), dim3((unsigned)tiles),
+                     dim3(SCAN_BLOCK), 0, s, (const T *)vs, (const uint8_t *)nullptr, n,
+                     (T *)out, ticket, desc, epoch, tiles, offsets, lens, m);
+  return launch_status();
+}
+
+}  // namespace fa
+
+extern "C" size_t fa_segscan_scratch_bytes(fa_dtype t, int64_t n) {
+  const size_t es = dtype_size(t);
+  if (es != 4 && es != 8) return 0;
+  if (n < 0) n = 0;
+  const int64_t tile = (es == 4) ? scan_tile_elems<int32_t>() : scan_tile_elems<int64_t>();
+  const int64_t tiles = ceil_div(n, tile);
+  return SCAN_HEADER_BYTES + (size_t)(tiles < 1 ? 1 : tiles) * SCAN_DESC_BYTES;
+}
+
+extern "C" int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op, const void *xs,
+                          const uint8_t *flags, int64_t n, int exclusive, void *out,
+                          void *scratch, size_t scratch_bytes, uint32_t epoch) {
+  if (n < 0 || (n > 0 && (xs == nullptr || out == nullptr || scratch == nullptr)))
+    return FA_EINVAL;
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xs, flags, n, exclusive, out, scratch,
+                      scratch_bytes, epoch);
+}
+
+extern "C" int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op, const void *vs,
+                                   int64_t n, const int64_t *offsets, const int64_t *lens,
+                                   int64_t m, void *out, void *scratch, size_t scratch_bytes,
+                                   uint32_t epoch) {
+  if (n < 0 || m < 0 || (m > 0 && (offsets == nullptr || lens == nullptr || out == nullptr)) ||
+      (n > 0 && m > 0 && (vs == nullptr || scratch == nullptr)))
+    return FA_EINVAL;
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  FA_DISPATCH_TYPE_OP(launch_segred_irregular, t, op, s, vs, n, offsets, lens, m, out, scratch,
+                      scratch_bytes, epoch);
+}

@@ -1,0 +1,664 @@
+/*
+ * segops.c -- the `segops` program: array types and entry points of the public
+ * API in include/segops.h, written the way the Futhark C backends generate
+ * them (array functions: src/Futhark/CodeGen/Backends/GenericC/Types.hs:177-240;
+ * entry-point wrapper with lock, size checks and output packing:
+ * GenericC/EntryPoints.hs:133-208), with each SegOp handed to the gfx950
+ * kernel library instead of to a `gpu_kernel_*` launch wrapper.
+ */
+#define _POSIX_C_SOURCE 200809L
+#include <stdlib.h>
+#include <string.h>
+
+#include "../rts/rts.h"
+#include "futhark_amd_kernels.h"
+#include "segops.h"
+
+/* ---------------------------------------------------------- tuning params
+ * Named like the reference names them, `<entry>.<description>`
+ * (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:118-120). */
+static const char *const tuning_names[] = {
+    "segops.hist_lds_bins_max",
+    "segops.segred_small_threshold",
+};
+static const char *const tuning_classes[] = {"shared_memory", "threshold"};
+static const int64_t tuning_defaults[] = {0, 0};
+
+const struct rts_program futhark_program = {
+    "segops", 2, tuning_names, tuning_classes, tuning_defaults,
+};
+
+/* ------------------------------------------------------------------ arrays */
+
+struct fut_array {
+  struct memblock_device mem;
+  int64_t shape[3];
+};
+
+static int64_t shape_elems(int rank, const int64_t *shape) {
+  int64_t n = 1;
+  for (int i = 0; i < rank; i++) n *= shape[i];
+  return n;
+}
+
+static struct fut_array *array_new(struct futhark_context *ctx, const void *data, size_t elem,
+                                   int rank, const int64_t *dims, const char *desc) {
+  struct fut_array *arr = (struct fut_array *)calloc(1, sizeof(struct fut_array));
+  if (arr == NULL) return NULL;
+  int err = 0;
+  pthread_mutex_lock(&ctx->lock);
+  for (int i = 0; i < rank; i++) {
+    arr->shape[i] = dims[i];
+    if (dims[i] < 0) err = 1;
+  }
+  if (err) {
+    rts_set_error(ctx, strdup("Negative array dimension.\n"));
+  } else {
+    const int64_t bytes = shape_elems(rank, dims) * (int64_t)elem;
+    err = rts_memblock_alloc(ctx, &arr->mem, bytes, desc);
+    if (err == 0) {
+      err = rts_copy_h2d(ctx, arr->mem.mem, data, (size_t)bytes);
+      if (err != 0) rts_memblock_unref(ctx, &arr->mem, desc);
+    }
+  }
+  pthread_mutex_unlock(&ctx->lock);
+  if (err != 0) {
+    free(arr);
+    return NULL;
+  }
+  return arr;
+}
+
+static struct fut_array *array_new_raw(struct futhark_context *ctx, void *data, size_t elem,
+                                       int rank, const int64_t *dims) {
+  (void)ctx;
+  struct fut_array *arr = (struct fut_array *)calloc(1, sizeof(struct fut_array));
+  if (arr == NULL) return NULL;
+  for (int i = 0; i < rank; i++) arr->shape[i] = dims[i];
+  arr->mem.references = NULL;
+  arr->mem.mem = data;
+  arr->mem.size = shape_elems(rank, dims) * (int64_t)elem;
+  arr->mem.desc = "raw";
+  return arr;
+}
+
+static int array_free(struct futhark_context *ctx, struct fut_array *arr, const char *desc) {
+  pthread_mutex_lock(&ctx->lock);
+  int err = rts_memblock_unref(ctx, &arr->mem, desc);
+  pthread_mutex_unlock(&ctx->lock);
+  free(arr);
+  return err;
+}
+
+static int array_values(struct futhark_context *ctx, struct fut_array *arr, void *out,
+                        size_t elem, int rank) {
+  pthread_mutex_lock(&ctx->lock);
+  int err =
+      rts_copy_d2h(ctx, out, arr->mem.mem, (size_t)shape_elems(rank, arr->shape) * elem);
+  pthread_mutex_unlock(&ctx->lock);
+  return err;
+}
+
+static int array_index(struct futhark_context *ctx, void *out, struct fut_array *arr,
+                       size_t elem, int rank, const int64_t *idx) {
+  int64_t flat = 0;
+  for (int i = 0; i < rank; i++) {
+    if (idx[i] < 0 || idx[i] >= arr->shape[i]) {
+      rts_set_error(ctx, strdup("Index out of bounds."));
+      return 1;
+    }
+    flat = flat * arr->shape[i] + idx[i];
+  }
+  pthread_mutex_lock(&ctx->lock);
+  int err = rts_copy_d2h(ctx, out, (const char *)arr->mem.mem + flat * (int64_t)elem, elem);
+  pthread_mutex_unlock(&ctx->lock);
+  return err;
+}
+
+#define DIMS_PARAMS_1 int64_t dim0
+#define DIMS_PARAMS_2 int64_t dim0, int64_t dim1
+#define DIMS_PARAMS_3 int64_t dim0, int64_t dim1, int64_t dim2
+#define DIMS_ARGS_1 {dim0}
+#define DIMS_ARGS_2 {dim0, dim1}
+#define DIMS_ARGS_3 {dim0, dim1, dim2}
+#define IDX_PARAMS_1 int64_t i0
+#define IDX_PARAMS_2 int64_t i0, int64_t i1
+#define IDX_PARAMS_3 int64_t i0, int64_t i1, int64_t i2
+#define IDX_ARGS_1 {i0}
+#define IDX_ARGS_2 {i0, i1}
+#define IDX_ARGS_3 {i0, i1, i2}
+
+#define DEFINE_ARRAY(NAME, CT, R)                                                              \
+  struct futhark_##NAME##_##R##d {                                                             \
+    struct fut_array a;                                                                        \
+  };                                                                                           \
+  struct futhark_##NAME##_##R##d *futhark_new_##NAME##_##R##d(struct futhark_context *ctx,     \
+                                                              const CT *data,                  \
+                                                              DIMS_PARAMS_##R) {               \
+    const int64_t dims[3] = DIMS_ARGS_##R;                                                     \
+    return (struct futhark_##NAME##_##R##d *)array_new(ctx, data, sizeof(CT), R, dims,         \
+                                                       "arr->mem");                            \
+  }                                                                                            \
+  struct futhark_##NAME##_##R##d *futhark_new_raw_##NAME##_##R##d(                             \
+      struct futhark_context *ctx, futhark_device_ptr data, DIMS_PARAMS_##R) {                 \
+    const int64_t dims[3] = DIMS_ARGS_##R;                                                     \
+    return (struct futhark_##NAME##_##R##d *)array_new_raw(ctx, data, sizeof(CT), R, dims);    \
+  }                                                                                            \
+  int futhark_free_##NAME##_##R##d(struct futhark_context *ctx,                                \
+                                   struct futhark_##NAME##_##R##d *arr) {                      \
+    return array_free(ctx, &arr->a, "arr->mem");                                               \
+  }                                                                                            \
+  int futhark_values_##NAME##_##R##d(struct futhark_context *ctx,                              \
+                                     struct futhark_##NAME##_##R##d *arr, CT *data) {          \
+    return array_values(ctx, &arr->a, data, sizeof(CT), R);                                    \
+  }                                                                                            \
+  int futhark_index_##NAME##_##R##d(struct futhark_context *ctx, CT *out,                      \
+                                    struct futhark_##NAME##_##R##d *arr, IDX_PARAMS_##R) {     \
+    const int64_t idx[3] = IDX_ARGS_##R;                                                       \
+    return array_index(ctx, out, &arr->a, sizeof(CT), R, idx);                                 \
+  }                                                                                            \
+  futhark_device_ptr futhark_values_raw_##NAME##_##R##d(struct futhark_context *ctx,           \
+                                                        struct futhark_##NAME##_##R##d *arr) { \
+    (void)ctx;                                                                                 \
+    return arr->a.mem.mem;                                                                     \
+  }                                                                                            \
+  const int64_t *futhark_shape_##NAME##_##R##d(struct futhark_context *ctx,                    \
+                                               struct futhark_##NAME##_##R##d *arr) {          \
+    (void)ctx;                                                                                 \
+    return arr->a.shape;                                                                       \
+  }
+
+DEFINE_ARRAY(i32, int32_t, 1)
+DEFINE_ARRAY(i64, int64_t, 1)
+DEFINE_ARRAY(u8, uint8_t, 1)
+DEFINE_ARRAY(u32, uint32_t, 1)
+DEFINE_ARRAY(u64, uint64_t, 1)
+DEFINE_ARRAY(f32, float, 1)
+DEFINE_ARRAY(f64, double, 1)
+DEFINE_ARRAY(i32, int32_t, 2)
+DEFINE_ARRAY(i64, int64_t, 2)
+DEFINE_ARRAY(f32, float, 2)
+DEFINE_ARRAY(f64, double, 2)
+DEFINE_ARRAY(f32, float, 3)
+DEFINE_ARRAY(f16, uint16_t, 3)
+DEFINE_ARRAY(u16, uint16_t, 3)
+
+/* ------------------------------------------------------ entry-point helpers */
+
+/* A fresh output array of `rank` dims over a new block of `bytes` bytes. */
+static struct fut_array *out_array(struct futhark_context *ctx, int64_t bytes, int rank,
+                                   const int64_t *dims, const char *desc) {
+  struct fut_array *arr = (struct fut_array *)calloc(1, sizeof(struct fut_array));
+  if (arr == NULL) return NULL;
+  if (rts_memblock_alloc(ctx, &arr->mem, bytes, desc) != 0) {
+    free(arr);
+    return NULL;
+  }
+  for (int i = 0; i < rank; i++) arr->shape[i] = dims[i];
+  return arr;
+}
+
+static void drop_array(struct futhark_context *ctx, struct fut_array *arr) {
+  if (arr != NULL) {
+    rts_memblock_unref(ctx, &arr->mem, "out");
+    free(arr);
+  }
+}
+
+static int bad_sizes(struct futhark_context *ctx, const char *entry) {
+  rts_set_error(ctx, rts_msgprintf("Error: entry point arguments have invalid sizes.\n"
+                                   "Entry point: %s\n", entry));
+  return 1;
+}
+
+static const fa_dtype DT_i32 = FA_I32, DT_i64 = FA_I64, DT_f32 = FA_F32, DT_f64 = FA_F64;
+static const fa_op OP_add = FA_ADD, OP_max = FA_MAX, OP_min = FA_MIN;
+
+static int do_reduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es, void *out,
+                     const struct fut_array *in) {
+  const int64_t n = in->shape[0];
+  void *scratch = rts_red_scratch(ctx, fa_segred_scratch_bytes(t));
+  if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
+  struct memblock_device res = {0};
+  int err = rts_memblock_alloc(ctx, &res, (int64_t)es, "reduce.res");
+  if (err != 0) return err;
+  struct rts_event *ev = rts_kernel_begin(
+      ctx, "segred_nonseg", rts_msgprintf("{\"n\":%lld,\"bytes\":%lld}", (long long)n,
+                                          (long long)(n * (int64_t)es)));
+  int code = fa_segred_nonseg(ctx->stream, t, op, in->mem.mem, n, res.mem, scratch,
+                              ctx->red_scratch_bytes);
+  err = rts_kernel_end(ctx, ev, "segred_nonseg", code);
+  if (err == 0) err = rts_copy_d2h(ctx, out, res.mem, es);
+  rts_memblock_unref(ctx, &res, "reduce.res");
+  return err;
+}
+
+static int do_scan(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                   struct fut_array **out, const struct fut_array *flags,
+                   const struct fut_array *in, int exclusive, const char *entry) {
+  const int64_t n = in->shape[0];
+  if (flags != NULL && flags->shape[0] != n) return bad_sizes(ctx, entry);
+  uint32_t epoch = 0;
+  const size_t sbytes = fa_segscan_scratch_bytes(t, n);
+  void *scratch = rts_scan_scratch(ctx, sbytes, &epoch);
+  if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
+  struct fut_array *res = out_array(ctx, n * (int64_t)es, 1, &n, "scan.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  struct rts_event *ev = rts_kernel_begin(
+      ctx, "segscan", rts_msgprintf("{\"n\":%lld,\"segmented\":%d,\"exclusive\":%d}",
+                                    (long long)n, flags != NULL, exclusive));
+  int code = fa_segscan(ctx->stream, t, op, in->mem.mem,
+                        flags ? (const uint8_t *)flags->mem.mem : NULL, n, exclusive,
+                        res->mem.mem, scratch, ctx->scan_scratch_bytes, epoch);
+  int err = rts_kernel_end(ctx, ev, "segscan", code);
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
+static int do_segred(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                     struct fut_array **out, const struct fut_array *offsets,
+                     const struct fut_array *lens, const struct fut_array *vs,
+                     const char *entry) {
+  const int64_t m = offsets->shape[0], n = vs->shape[0];
+  if (lens->shape[0] != m) return bad_sizes(ctx, entry);
+  uint32_t epoch = 0;
+  void *scratch = rts_scan_scratch(ctx, fa_segscan_scratch_bytes(t, n), &epoch);
+  if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
+  struct fut_array *res = out_array(ctx, m * (int64_t)es, 1, &m, "segred.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  struct rts_event *ev = rts_kernel_begin(
+      ctx, "segred_irregular",
+      rts_msgprintf("{\"n\":%lld,\"segments\":%lld}", (long long)n, (long long)m));
+  int code = fa_segred_irregular(ctx->stream, t, op, vs->mem.mem, n,
+                                 (const int64_t *)offsets->mem.mem,
+                                 (const int64_t *)lens->mem.mem, m, res->mem.mem, scratch,
+                                 ctx->scan_scratch_bytes, epoch);
+  int err = rts_kernel_end(ctx, ev, "segred_irregular", code);
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
+static int do_segreduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                        struct fut_array **out, const struct fut_array *in) {
+  const int64_t m = in->shape[0], k = in->shape[1];
+  struct fut_array *res = out_array(ctx, m * (int64_t)es, 1, &m, "segreduce.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  struct rts_event *ev = rts_kernel_begin(
+      ctx, "segred_regular",
+      rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)k));
+  int code = fa_segred_regular(ctx->stream, t, op, in->mem.mem, m, k, res->mem.mem);
+  int err = rts_kernel_end(ctx, ev, "segred_regular", code);
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
+static uint64_t neutral_bits(fa_dtype t, fa_op op) {
+  union { int32_t i; float f; uint32_t u; } b32;
+  union { int64_t i; double f; uint64_t u; } b64;
+  switch (t) {
+    case FA_I32:
+      b32.i = op == FA_ADD ? 0 : (op == FA_MAX ? INT32_MIN : INT32_MAX);
+      return b32.u;
+    case FA_F32:
+      b32.f = op == FA_ADD ? 0.0f : (op == FA_MAX ? -__builtin_inff() : __builtin_inff());
+      return b32.u;
+    case FA_I64:
+      b64.i = op == FA_ADD ? 0 : (op == FA_MAX ? INT64_MIN : INT64_MAX);
+      return b64.u;
+    default:
+      b64.f = op == FA_ADD ? 0.0 : (op == FA_MAX ? -__builtin_inf() : __builtin_inf());
+      return b64.u;
+  }
+}
+
+/* dest_in == NULL: histogram into a fresh array of k neutral elements. */
+static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                   struct fut_array **out, int64_t k, const struct fut_array *dest_in,
+                   const struct fut_array *is, const struct fut_array *vs, const char *entry) {
+  const int64_t n = is->shape[0];
+  if (vs->shape[0] != n) return bad_sizes(ctx, entry);
+  if (dest_in != NULL) k = dest_in->shape[0];
+  if (k < 0) {
+    rts_set_error(ctx, rts_msgprintf("Error: negative histogram size %lld.\n", (long long)k));
+    return FUTHARK_PROGRAM_ERROR;
+  }
+  struct fut_array *res = out_array(ctx, k * (int64_t)es, 1, &k, "hist.dest");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  int err = 0;
+  if (dest_in != NULL) {
+    err = rts_copy_d2d(ctx, res->mem.mem, dest_in->mem.mem, (size_t)k * es);
+  } else if (k > 0) {
+    int code = fa_replicate(ctx->stream, (int)es, res->mem.mem, k, neutral_bits(t, op));
+    err = rts_kernel_end(ctx, NULL, "replicate", code);
+  }
+  struct memblock_device scratch = {0};
+  if (err == 0) {
+    err = rts_memblock_alloc(ctx, &scratch, (int64_t)fa_seghist_scratch_bytes(t, k),
+                             "hist.scratch");
+  }
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "seghist", rts_msgprintf("{\"n\":%lld,\"bins\":%lld}", (long long)n, (long long)k));
+    int code = fa_seghist(ctx->stream, t, op, is->mem.mem, 0, vs->mem.mem, n, res->mem.mem, k,
+                          scratch.mem, (size_t)scratch.size);
+    err = rts_kernel_end(ctx, ev, "seghist", code);
+  }
+  rts_memblock_unref(ctx, &scratch, "hist.scratch");
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
+#define ENTER(ctx) pthread_mutex_lock(&(ctx)->lock)
+#define LEAVE(ctx) pthread_mutex_unlock(&(ctx)->lock)
+
+#define DEFINE_SEGOP_ENTRIES(OP, T, CT)                                                       \
+  int futhark_entry_reduce_##OP##_##T(struct futhark_context *ctx, CT *out0,                  \
+                                      const struct futhark_##T##_1d *in0) {                   \
+    ENTER(ctx);                                                                               \
+    int ret = do_reduce(ctx, DT_##T, OP_##OP, sizeof(CT), out0, &in0->a);                     \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_scan_##OP##_##T(struct futhark_context *ctx,                              \
+                                    struct futhark_##T##_1d **out0,                           \
+                                    const struct futhark_##T##_1d *in0) {                     \
+    ENTER(ctx);                                                                               \
+    int ret = do_scan(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, NULL,      \
+                      &in0->a, 0, "scan_" #OP "_" #T);                                        \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_exscan_##OP##_##T(struct futhark_context *ctx,                            \
+                                      struct futhark_##T##_1d **out0,                         \
+                                      const struct futhark_##T##_1d *in0) {                   \
+    ENTER(ctx);                                                                               \
+    int ret = do_scan(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, NULL,      \
+                      &in0->a, 1, "exscan_" #OP "_" #T);                                      \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_segscan_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_1d **out0,                        \
+                                       const struct futhark_u8_1d *in0,                       \
+                                       const struct futhark_##T##_1d *in1) {                  \
+    ENTER(ctx);                                                                               \
+    int ret = do_scan(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a,   \
+                      &in1->a, 0, "segscan_" #OP "_" #T);                                     \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_segred_##OP##_##T(struct futhark_context *ctx,                            \
+                                      struct futhark_##T##_1d **out0,                         \
+                                      const struct futhark_i64_1d *in0,                       \
+                                      const struct futhark_i64_1d *in1,                       \
+                                      const struct futhark_##T##_1d *in2) {                   \
+    ENTER(ctx);                                                                               \
+    int ret = do_segred(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a, \
+                        &in1->a, &in2->a, "segred_" #OP "_" #T);                              \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_segreduce_##OP##_##T(struct futhark_context *ctx,                         \
+                                         struct futhark_##T##_1d **out0,                      \
+                                         const struct futhark_##T##_2d *in0) {                \
+    ENTER(ctx);                                                                               \
+    int ret =                                                                                 \
+        do_segreduce(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a);   \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_hist_##OP##_##T(struct futhark_context *ctx,                              \
+                                    struct futhark_##T##_1d **out0, const int64_t in0,        \
+                                    const struct futhark_i32_1d *in1,                         \
+                                    const struct futhark_##T##_1d *in2) {                     \
+    ENTER(ctx);                                                                               \
+    int ret = do_hist(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, in0, NULL, \
+                      &in1->a, &in2->a, "hist_" #OP "_" #T);                                  \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_rbi_##OP##_##T(struct futhark_context *ctx,                               \
+                                   struct futhark_##T##_1d **out0,                            \
+                                   const struct futhark_##T##_1d *in0,                        \
+                                   const struct futhark_i32_1d *in1,                          \
+                                   const struct futhark_##T##_1d *in2) {                      \
+    ENTER(ctx);                                                                               \
+    int ret = do_hist(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, 0,         \
+                      &in0->a, &in1->a, &in2->a, "rbi_" #OP "_" #T);                          \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }
+
+#define DEFINE_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(DEFINE_SEGOP_ENTRIES, T, CT)
+FUTHARK_FOR_EACH_NUM_TYPE(DEFINE_FOR_TYPE)
+
+/* ------------------------------------------------------------------ matmul */
+
+static int do_bmm(struct futhark_context *ctx, fa_dtype in_t, struct fut_array **out, int rank,
+                  const struct fut_array *A, const struct fut_array *B, const char *entry) {
+  int64_t b = 1, M, K, K2, N;
+  if (rank == 3) {
+    b = A->shape[0];
+    M = A->shape[1];
+    K = A->shape[2];
+    K2 = B->shape[1];
+    N = B->shape[2];
+    if (B->shape[0] != b) return bad_sizes(ctx, entry);
+  } else {
+    M = A->shape[0];
+    K = A->shape[1];
+    K2 = B->shape[0];
+    N = B->shape[1];
+  }
+  if (K != K2) return bad_sizes(ctx, entry);
+  const int64_t dims3[3] = {b, M, N}, dims2[2] = {M, N};
+  struct fut_array *res =
+      out_array(ctx, b * M * N * 4, rank, rank == 3 ? dims3 : dims2, "bmm.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  struct rts_event *ev = rts_kernel_begin(
+      ctx, "segmap_matmul",
+      rts_msgprintf("{\"batch\":%lld,\"M\":%lld,\"N\":%lld,\"K\":%lld,\"flop\":%lld}",
+                    (long long)b, (long long)M, (long long)N, (long long)K,
+                    (long long)(2 * b * M * N * K)));
+  int code = fa_matmul(ctx->stream, in_t, A->mem.mem, B->mem.mem, (float *)res->mem.mem, b, M,
+                       N, K);
+  int err = rts_kernel_end(ctx, ev, "segmap_matmul", code);
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
+int futhark_entry_bmm_f32(struct futhark_context *ctx, struct futhark_f32_3d **out0,
+                          const struct futhark_f32_3d *in0, const struct futhark_f32_3d *in1) {
+  ENTER(ctx);
+  int ret = do_bmm(ctx, FA_F32, (struct fut_array **)out0, 3, &in0->a, &in1->a, "bmm_f32");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_bmm_f16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
+                          const struct futhark_f16_3d *in0, const struct futhark_f16_3d *in1) {
+  ENTER(ctx);
+  int ret = do_bmm(ctx, FA_F16, (struct fut_array **)out0, 3, &in0->a, &in1->a, "bmm_f16");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_bmm_bf16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
+                           const struct futhark_u16_3d *in0, const struct futhark_u16_3d *in1) {
+  ENTER(ctx);
+  int ret = do_bmm(ctx, FA_BF16, (struct fut_array **)out0, 3, &in0->a, &in1->a, "bmm_bf16");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_matmul_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
+                             const struct futhark_f32_2d *in0, const struct futhark_f32_2d *in1) {
+  ENTER(ctx);
+  int ret = do_bmm(ctx, FA_F32, (struct fut_array **)out0, 2, &in0->a, &in1->a, "matmul_f32");
+  LEAVE(ctx);
+  return ret;
+}
+
+/* -------------------------------------------------------------- radix sort */
+
+static int do_sort(struct futhark_context *ctx, int key_bytes, int val_bytes,
+                   struct fut_array **out_keys, struct fut_array **out_vals,
+                   const struct fut_array *keys, const struct fut_array *vals,
+                   const char *entry) {
+  const int64_t n = keys->shape[0];
+  if (vals != NULL && vals->shape[0] != n) return bad_sizes(ctx, entry);
+  struct fut_array *rk = out_array(ctx, n * key_bytes, 1, &n, "sort.keys");
+  struct fut_array *rv = vals ? out_array(ctx, n * val_bytes, 1, &n, "sort.vals") : NULL;
+  struct memblock_device tk = {0}, tv = {0}, scratch = {0};
+  int err = (rk == NULL || (vals && rv == NULL)) ? FUTHARK_OUT_OF_MEMORY : 0;
+  if (err == 0) err = rts_memblock_alloc(ctx, &tk, n * key_bytes, "sort.keys_tmp");
+  if (err == 0 && vals) err = rts_memblock_alloc(ctx, &tv, n * val_bytes, "sort.vals_tmp");
+  if (err == 0)
+    err = rts_memblock_alloc(ctx, &scratch, (int64_t)fa_radix_sort_scratch_bytes(n),
+                             "sort.scratch");
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "radix_sort", rts_msgprintf("{\"n\":%lld,\"key_bytes\":%d,\"val_bytes\":%d}",
+                                         (long long)n, key_bytes, val_bytes));
+    int code = fa_radix_sort(ctx->stream, key_bytes, val_bytes, keys->mem.mem, rk->mem.mem,
+                             tk.mem, vals ? vals->mem.mem : NULL, rv ? rv->mem.mem : NULL,
+                             vals ? tv.mem : NULL, n, 0, key_bytes * 8, scratch.mem,
+                             (size_t)scratch.size);
+    err = rts_kernel_end(ctx, ev, "radix_sort", code);
+  }
+  rts_memblock_unref(ctx, &tk, "sort.keys_tmp");
+  rts_memblock_unref(ctx, &tv, "sort.vals_tmp");
+  rts_memblock_unref(ctx, &scratch, "sort.scratch");
+  if (err != 0) {
+    drop_array(ctx, rk);
+    drop_array(ctx, rv);
+    return err;
+  }
+  *out_keys = rk;
+  if (out_vals) *out_vals = rv;
+  return 0;
+}
+
+int futhark_entry_radix_sort_u32(struct futhark_context *ctx, struct futhark_u32_1d **out0,
+                                 const struct futhark_u32_1d *in0) {
+  ENTER(ctx);
+  int ret = do_sort(ctx, 4, 0, (struct fut_array **)out0, NULL, &in0->a, NULL, "radix_sort_u32");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_radix_sort_u64(struct futhark_context *ctx, struct futhark_u64_1d **out0,
+                                 const struct futhark_u64_1d *in0) {
+  ENTER(ctx);
+  int ret = do_sort(ctx, 8, 0, (struct fut_array **)out0, NULL, &in0->a, NULL, "radix_sort_u64");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_radix_sort_pairs_u32_i32(struct futhark_context *ctx,
+                                           struct futhark_u32_1d **out0,
+                                           struct futhark_i32_1d **out1,
+                                           const struct futhark_u32_1d *in0,
+                                           const struct futhark_i32_1d *in1) {
+  ENTER(ctx);
+  int ret = do_sort(ctx, 4, 4, (struct fut_array **)out0, (struct fut_array **)out1, &in0->a,
+                    &in1->a, "radix_sort_pairs_u32_i32");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_radix_sort_pairs_u64_i32(struct futhark_context *ctx,
+                                           struct futhark_u64_1d **out0,
+                                           struct futhark_i32_1d **out1,
+                                           const struct futhark_u64_1d *in0,
+                                           const struct futhark_i32_1d *in1) {
+  ENTER(ctx);
+  int ret = do_sort(ctx, 8, 4, (struct fut_array **)out0, (struct fut_array **)out1, &in0->a,
+                    &in1->a, "radix_sort_pairs_u64_i32");
+  LEAVE(ctx);
+  return ret;
+}
+
+/* ---------------------------------------------------------- data movement */
+
+int futhark_entry_transpose_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
+                                const struct futhark_f32_2d *in0) {
+  ENTER(ctx);
+  const int64_t rows = in0->a.shape[0], cols = in0->a.shape[1];
+  const int64_t dims[2] = {cols, rows};
+  int ret = 0;
+  struct fut_array *res = out_array(ctx, rows * cols * 4, 2, dims, "transpose.out");
+  if (res == NULL) {
+    ret = FUTHARK_OUT_OF_MEMORY;
+  } else {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "map_transpose_4b",
+        rts_msgprintf("{\"rows\":%lld,\"cols\":%lld}", (long long)rows, (long long)cols));
+    int code = fa_map_transpose(ctx->stream, 4, res->mem.mem, in0->a.mem.mem, 1, rows, cols);
+    ret = rts_kernel_end(ctx, ev, "map_transpose_4b", code);
+    if (ret != 0) drop_array(ctx, res);
+    else *out0 = (struct futhark_f32_2d *)res;
+  }
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_iota_i64(struct futhark_context *ctx, struct futhark_i64_1d **out0,
+                           const int64_t in0) {
+  ENTER(ctx);
+  int ret = 0;
+  if (in0 < 0) {
+    rts_set_error(ctx, rts_msgprintf("Error: Range 0..<%lld is invalid.\n", (long long)in0));
+    ret = FUTHARK_PROGRAM_ERROR;
+  } else {
+    struct fut_array *res = out_array(ctx, in0 * 8, 1, &in0, "iota.out");
+    if (res == NULL) {
+      ret = FUTHARK_OUT_OF_MEMORY;
+    } else {
+      int code = fa_iota(ctx->stream, FA_I64, res->mem.mem, in0, 0, 1);
+      ret = rts_kernel_end(ctx, NULL, "iota_i64", code);
+      if (ret != 0) drop_array(ctx, res);
+      else *out0 = (struct futhark_i64_1d *)res;
+    }
+  }
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_replicate_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
+                                const int64_t in0, const int32_t in1) {
+  ENTER(ctx);
+  int ret = 0;
+  if (in0 < 0) {
+    rts_set_error(ctx, rts_msgprintf("Error: negative size %lld.\n", (long long)in0));
+    ret = FUTHARK_PROGRAM_ERROR;
+  } else {
+    struct fut_array *res = out_array(ctx, in0 * 4, 1, &in0, "replicate.out");
+    if (res == NULL) {
+      ret = FUTHARK_OUT_OF_MEMORY;
+    } else {
+      int code = fa_replicate(ctx->stream, 4, res->mem.mem, in0, (uint32_t)in1);
+      ret = rts_kernel_end(ctx, NULL, "replicate_i32", code);
+      if (ret != 0) drop_array(ctx, res);
+      else *out0 = (struct futhark_i32_1d *)res;
+    }
+  }
+  LEAVE(ctx);
+  return ret;
+}
+
+void *futhark_context_get_stream(struct futhark_context *ctx) { return ctx->stream; }

@@ -1,0 +1,173 @@
+/*
+ * futhark_amd_kernels.h -- C ABI of the gfx950 SegOp kernel library
+ * (libfuthark_amd_kernels.so).
+ *
+ * Each launcher below stands where the Futhark GPU backends place one or more
+ * generated `gpu_kernel_<name>(ctx, grid..., block..., shared_bytes, args...)`
+ * host wrappers (reference: src/Futhark/CodeGen/Backends/GPU.hs:31-69) around
+ * kernels emitted by the SegOp code generators
+ * (src/Futhark/CodeGen/ImpGen/GPU/{SegRed,SegScan/SinglePass,SegHist,SegMap}.hs).
+ * Instead of kernel text compiled at context creation, the kernels are
+ * hand-written HIP compiled offline for gfx950; the launcher picks grid, block
+ * and LDS sizes itself.
+ *
+ * Conventions
+ *  - plain C: pointers and sizes only.  All data pointers are DEVICE pointers.
+ *  - every call is asynchronous on `stream` (a hipStream_t passed as void*).
+ *  - scratch memory is supplied by the caller (the runtime's pooled allocator);
+ *    `fa_*_scratch_bytes` reports how much a call needs.  No launcher
+ *    allocates or frees device memory.
+ *  - return value: 0 on success, a positive hipError_t value if a HIP call
+ *    failed, or a negative FA_E* code for an argument the library rejects.
+ */
+#ifndef FUTHARK_AMD_KERNELS_H
+#define FUTHARK_AMD_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *fa_stream_t; /* hipStream_t */
+
+/* Element types (Futhark primitive types that occur on the path). */
+typedef enum {
+  FA_I32 = 0,
+  FA_I64 = 1,
+  FA_F32 = 2,
+  FA_F64 = 3,
+  FA_U32 = 4,
+  FA_U64 = 5,
+  FA_F16 = 6,  /* IEEE binary16 bits in a uint16_t (docs/c-api.rst:229-233) */
+  FA_BF16 = 7, /* bfloat16 bits in a uint16_t: f32 = bits << 16 */
+  FA_DTYPE_COUNT
+} fa_dtype;
+
+/* Scalar operators with the neutral element the kernels use for padding:
+ * ADD: 0;  MAX: lowest (INT_MIN / -inf);  MIN: highest (INT_MAX / +inf).
+ * Semantics are those of rts/c/scalar.h: two's-complement wrap-around add
+ * (scalar.h:29-30), smax/smin (scalar.h:488-503), fmaxf/fminf, i.e. NaN-ignoring
+ * (scalar.h:931-934). */
+typedef enum { FA_ADD = 0, FA_MAX = 1, FA_MIN = 2, FA_OP_COUNT } fa_op;
+
+#define FA_EINVAL (-1)   /* bad argument (null pointer, negative size, ...) */
+#define FA_ENOTSUP (-2)  /* dtype/op combination not built */
+#define FA_ESCRATCH (-3) /* scratch buffer too small */
+#define FA_EALIGN (-4)   /* pointer not aligned as the kernel requires */
+
+/* Human-readable text for a return code (static storage). */
+const char *fa_strerror(int code);
+
+/* Library/ABI version: major*1000 + minor. */
+int fa_version(void);
+
+/* ------------------------------------------------------------------ SegRed
+ * Non-segmented reduction `reduce op ne xs`.
+ * Replaces: segred_nonseg (SegRed.hs:327-394): stage one, per-block partials,
+ * last-block-finishes stage two with an atomic counter (SegRed.hs:923-1047).
+ * out: one element.  scratch: fa_segred_scratch_bytes(); its first 64 bytes
+ * must be zero before the first use and are left zero by every call. */
+size_t fa_segred_scratch_bytes(fa_dtype t);
+int fa_segred_nonseg(fa_stream_t stream, fa_dtype t, fa_op op,
+                     const void *xs, int64_t n, void *out,
+                     void *scratch, size_t scratch_bytes);
+
+/* Regular segmented reduction `map (reduce op ne) xss`, xss : [m][k] row-major.
+ * Replaces: segred_small / segred_large (SegRed.hs:396-636).  No scratch. */
+int fa_segred_regular(fa_stream_t stream, fa_dtype t, fa_op op,
+                      const void *xss, int64_t m, int64_t k, void *out);
+
+/* ----------------------------------------------------------------- SegScan
+ * Single-pass scan with decoupled look-back.
+ * Replaces: segscan (SegScan/SinglePass.hs:327-879) plus the status-flag fill
+ * kernel the reference launches before it (SinglePass.hs:379-389).
+ *
+ * flags == NULL : `scan op ne xs`.
+ * flags != NULL : the flag-tuple operator of Pass/Flatten/Builtins.hs:374-393,
+ *   (fx,x) (+) (fy,y) = (fx||fy, if fy then y else x op y), neutral (false,ne);
+ *   flags is one byte per element, nonzero = a segment starts here.
+ * exclusive != 0: out[i] = (inclusive result)[i-1] within the segment, `ne` at
+ *   i == 0 and at segment starts (prelude/soacs.fut:212-215 for the
+ *   unsegmented case).
+ *
+ * scratch protocol: the buffer must have been zero-filled once when it was
+ * allocated; after that it may be passed to any number of fa_segscan /
+ * fa_segred_irregular calls provided `epoch` is strictly larger on every call
+ * (1 <= epoch < 2^28; zero-fill again before wrapping).  Tile descriptors
+ * carry the epoch, so no per-call clearing kernel is needed. */
+size_t fa_segscan_scratch_bytes(fa_dtype t, int64_t n);
+int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op,
+               const void *xs, const uint8_t *flags, int64_t n, int exclusive,
+               void *out, void *scratch, size_t scratch_bytes, uint32_t epoch);
+
+/* Irregular segmented reduction (Pass/Flatten/Builtins.hs:582-602):
+ *   out[i] = lens[i] == 0 ? ne : segscan(flags-from-offsets, vs)[offsets[i]+lens[i]-1]
+ * computed without materialising the scan.  offsets must be non-decreasing,
+ * within [0,n].  Same scratch protocol as fa_segscan. */
+int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op,
+                        const void *vs, int64_t n,
+                        const int64_t *offsets, const int64_t *lens, int64_t m,
+                        void *out, void *scratch, size_t scratch_bytes,
+                        uint32_t epoch);
+
+/* ----------------------------------------------------------------- SegHist
+ * `reduce_by_index dest op ne is vs` (prelude/soacs.fut:132-146): for every i
+ * with 0 <= is[i] < H, dest[is[i]] = dest[is[i]] op vs[i]; other indices are
+ * ignored (SegHist.hs:450-458,750-755).  dest is updated in place.
+ * Replaces: seghist_local / seghist_global and the SegRed over sub-histograms
+ * (SegHist.hs:377-467,576-828,1137-1186).  `is` is i32 (is64 == 0) or i64.
+ * scratch: fa_seghist_scratch_bytes(); contents need no initialisation. */
+size_t fa_seghist_scratch_bytes(fa_dtype t, int64_t H);
+int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op,
+               const void *is, int is64, const void *vs, int64_t n,
+               void *dest, int64_t H, void *scratch, size_t scratch_bytes);
+
+/* -------------------------------------------------------------- radix sort
+ * Stable LSD radix sort with 8-bit digits: per pass a digit histogram
+ * (SegHist), an exclusive scan of the counts (SegScan) and a ranked scatter
+ * (cf. tests/issue2234.fut:10-58 for the composition, 2-bit digits there).
+ * key_bytes is 4 or 8; keys compare as unsigned.  val_bytes is 0, 4 or 8.
+ * keys_in/vals_in are not modified; the result lands in keys_out/vals_out.
+ * keys_tmp/vals_tmp are n-element ping-pong buffers.  begin_bit/end_bit select
+ * the key bits that take part (multiple of 8 apart). */
+size_t fa_radix_sort_scratch_bytes(int64_t n);
+int fa_radix_sort(fa_stream_t stream, int key_bytes, int val_bytes,
+                  const void *keys_in, void *keys_out, void *keys_tmp,
+                  const void *vals_in, void *vals_out, void *vals_tmp,
+                  int64_t n, int begin_bit, int end_bit,
+                  void *scratch, size_t scratch_bytes);
+
+/* ------------------------------------------------- tiled SegMap (matmul)
+ * C[b][i][j] = sum_k A[b][i][k] * B[b][k][j], all row-major, f32 output and
+ * f32 accumulation.  in_t is FA_F32, FA_F16 or FA_BF16.
+ * Replaces: the block/register-tiled segmap_intrablock that
+ * mmBlkRegTiling produces (src/Futhark/Optimise/BlkRegTiling.hs:463-621). */
+int fa_matmul(fa_stream_t stream, fa_dtype in_t,
+              const void *A, const void *B, float *C,
+              int64_t batch, int64_t M, int64_t N, int64_t K);
+
+/* ------------------------------------------------ builtin data movement
+ * Batched 2-D transpose: dst[b][j][i] = src[b][i][j], src : [batch][rows][cols].
+ * Replaces: map_transpose_{1,2,4,8}b (rts/opencl/transpose.cl). */
+int fa_map_transpose(fa_stream_t stream, int elem_bytes,
+                     void *dst, const void *src,
+                     int64_t batch, int64_t rows, int64_t cols);
+
+/* Fill n elements of elem_bytes (1,2,4,8) each with the given bit pattern.
+ * Replaces: builtin#replicate_* (ImpGen/GPU/Base.hs:1274-1350). */
+int fa_replicate(fa_stream_t stream, int elem_bytes, void *dst, int64_t n,
+                 uint64_t pattern);
+
+/* dst[i] = start + i*step for i < n, i32/i64 (ImpGen/GPU/Base.hs:1353-1436). */
+int fa_iota(fa_stream_t stream, fa_dtype t, void *dst, int64_t n,
+            int64_t start, int64_t step);
+
+/* Plain device copy kernel used for calibration of bandwidth counters. */
+int fa_copy(fa_stream_t stream, void *dst, const void *src, size_t bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FUTHARK_AMD_KERNELS_H */

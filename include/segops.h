@@ -1,0 +1,261 @@
+/*
+ * segops.h -- public C API of the `segops` program library (libsegops.so), in
+ * the shape `futhark hip --library` gives every compiled program
+ * (docs/c-api.rst; header layout src/Futhark/CodeGen/Backends/GenericC.hs:390-424;
+ * array functions GenericC/Types.hs:159-240; entry points
+ * GenericC/EntryPoints.hs:133-208).  A C caller written against a Futhark
+ * library with these entry points links against this one unchanged.
+ *
+ * The Futhark source each entry point stands for:
+ *
+ *   entry reduce_OP_T  (xs: []T) : T           = reduce OP NE xs
+ *   entry scan_OP_T    (xs: []T) : []T         = scan OP NE xs
+ *   entry exscan_OP_T  (xs: []T) : []T         -- prelude/soacs.fut:212-215
+ *   entry segscan_OP_T (flags: []u8) (vs: []T) : []T =
+ *     (unzip (scan (\(fx,x) (fy,y) -> (fx || fy, if fy then y else x `OP` y))
+ *                  (false,NE) (zip (map (!=0) flags) vs))).1
+ *                                   -- Pass/Flatten/Builtins.hs:374-401
+ *   entry segred_OP_T [m] (offsets: [m]i64) (lens: [m]i64) (vs: []T) : [m]T =
+ *     let flags = scatter (replicate n false) offsets (replicate m true)
+ *     let s = segscan OP NE flags vs
+ *     in map2 (\o l -> if l == 0 then NE else s[o+l-1]) offsets lens
+ *                                   -- Builtins.hs:570-602
+ *   entry segreduce_OP_T (xss: [][]T) : []T    = map (reduce OP NE) xss
+ *   entry hist_OP_T (k: i64) (is: []i32) (vs: []T) : [k]T =
+ *     hist OP NE k (map i64.i32 is) vs           -- prelude/soacs.fut:132-146
+ *   entry rbi_OP_T (dest: *[]T) (is: []i32) (vs: []T) : []T =
+ *     reduce_by_index dest OP NE (map i64.i32 is) vs
+ *   entry bmm_f32 (A: [][][]f32) (B: [][][]f32) : [][][]f32 =
+ *     map2 (\a b -> map (\ar -> map (\bc -> reduce (+) 0 (map2 (*) ar bc))
+ *                                   (transpose b)) a) A B
+ *                                   -- tests/reg-tiling/mmm.fut:17-21, batched
+ *   entry bmm_f16: the same with f16 inputs, products and sums in f32
+ *   entry bmm_bf16: [][][]u16 inputs, x -> f32.from_bits (u32.u16 x << 16)
+ *   entry radix_sort_T (keys: []T) : []T       -- 8-bit LSD passes, stable
+ *   entry radix_sort_pairs_K_V (keys: []K) (vals: []V) : ([]K, []V)
+ *   entry transpose_f32 (xss: [][]f32) : [][]f32 = transpose xss
+ *
+ * OP in {add, max, min}; NE = 0, T.lowest, T.highest; T in {i32, i64, f32, f64}.
+ */
+#ifndef SEGOPS_H
+#define SEGOPS_H
+
+#include <stdint.h>
+#include <stddef.h>
+#include <stdbool.h>
+#include <stdio.h>
+#include <float.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FUTHARK_BACKEND_hip
+#define FUTHARK_SUCCESS 0
+#define FUTHARK_PROGRAM_ERROR 2
+#define FUTHARK_OUT_OF_MEMORY 3
+
+/* Device pointers cross the raw-array functions as this type. */
+typedef void *futhark_device_ptr;
+
+/* --------------------------------------------------------- Initialisation */
+struct futhark_context_config;
+struct futhark_context_config *futhark_context_config_new(void);
+void futhark_context_config_free(struct futhark_context_config *cfg);
+int futhark_context_config_set_tuning_param(struct futhark_context_config *cfg,
+                                            const char *param_name, size_t new_value);
+void futhark_context_config_set_debugging(struct futhark_context_config *cfg, int flag);
+void futhark_context_config_set_profiling(struct futhark_context_config *cfg, int flag);
+void futhark_context_config_set_logging(struct futhark_context_config *cfg, int flag);
+void futhark_context_config_set_cache_file(struct futhark_context_config *cfg, const char *f);
+int futhark_get_tuning_param_count(void);
+const char *futhark_get_tuning_param_name(int i);
+const char *futhark_get_tuning_param_class(int i);
+/* GPU backends (docs/c-api.rst:609-669) */
+void futhark_context_config_set_device(struct futhark_context_config *cfg, const char *s);
+void futhark_context_config_set_unified_memory(struct futhark_context_config *cfg, int flag);
+void futhark_context_config_set_default_thread_block_size(struct futhark_context_config *cfg, int size);
+void futhark_context_config_set_default_group_size(struct futhark_context_config *cfg, int size);
+void futhark_context_config_set_default_grid_size(struct futhark_context_config *cfg, int num);
+void futhark_context_config_set_default_num_groups(struct futhark_context_config *cfg, int num);
+void futhark_context_config_set_default_tile_size(struct futhark_context_config *cfg, int size);
+void futhark_context_config_set_default_reg_tile_size(struct futhark_context_config *cfg, int size);
+void futhark_context_config_set_default_cache(struct futhark_context_config *cfg, int size);
+void futhark_context_config_set_default_registers(struct futhark_context_config *cfg, int size);
+void futhark_context_config_set_default_threshold(struct futhark_context_config *cfg, int size);
+void futhark_context_config_add_build_option(struct futhark_context_config *cfg, const char *opt);
+const char *futhark_context_config_get_program(struct futhark_context_config *cfg);
+void futhark_context_config_set_program(struct futhark_context_config *cfg, const char *s);
+
+struct futhark_context;
+struct futhark_context *futhark_context_new(struct futhark_context_config *cfg);
+void futhark_context_free(struct futhark_context *ctx);
+
+/* ----------------------------------------------------------------- Arrays
+ * For every array type futhark_T_Rd:
+ *   new      copies `data` (row-major, host) to the device, asynchronously
+ *   new_raw  wraps caller-owned device memory; never freed by the library
+ *   free     drops one reference
+ *   values   asynchronous copy to host; sync before reading
+ *   index    one element to host; 1 + "Index out of bounds." if outside
+ *   values_raw, shape
+ */
+#define FUTHARK_DECLARE_ARRAY_1D(NAME, CT)                                                     \
+  struct futhark_##NAME##_1d;                                                                  \
+  struct futhark_##NAME##_1d *futhark_new_##NAME##_1d(struct futhark_context *ctx,             \
+                                                      const CT *data, int64_t dim0);           \
+  struct futhark_##NAME##_1d *futhark_new_raw_##NAME##_1d(struct futhark_context *ctx,         \
+                                                          futhark_device_ptr data,             \
+                                                          int64_t dim0);                       \
+  int futhark_free_##NAME##_1d(struct futhark_context *ctx, struct futhark_##NAME##_1d *arr);  \
+  int futhark_values_##NAME##_1d(struct futhark_context *ctx, struct futhark_##NAME##_1d *arr, \
+                                 CT *data);                                                    \
+  int futhark_index_##NAME##_1d(struct futhark_context *ctx, CT *out,                          \
+                                struct futhark_##NAME##_1d *arr, int64_t i0);                  \
+  futhark_device_ptr futhark_values_raw_##NAME##_1d(struct futhark_context *ctx,               \
+                                                    struct futhark_##NAME##_1d *arr);          \
+  const int64_t *futhark_shape_##NAME##_1d(struct futhark_context *ctx,                        \
+                                           struct futhark_##NAME##_1d *arr);
+
+#define FUTHARK_DECLARE_ARRAY_2D(NAME, CT)                                                     \
+  struct futhark_##NAME##_2d;                                                                  \
+  struct futhark_##NAME##_2d *futhark_new_##NAME##_2d(struct futhark_context *ctx,             \
+                                                      const CT *data, int64_t dim0,            \
+                                                      int64_t dim1);                           \
+  struct futhark_##NAME##_2d *futhark_new_raw_##NAME##_2d(struct futhark_context *ctx,         \
+                                                          futhark_device_ptr data,             \
+                                                          int64_t dim0, int64_t dim1);         \
+  int futhark_free_##NAME##_2d(struct futhark_context *ctx, struct futhark_##NAME##_2d *arr);  \
+  int futhark_values_##NAME##_2d(struct futhark_context *ctx, struct futhark_##NAME##_2d *arr, \
+                                 CT *data);                                                    \
+  int futhark_index_##NAME##_2d(struct futhark_context *ctx, CT *out,                          \
+                                struct futhark_##NAME##_2d *arr, int64_t i0, int64_t i1);      \
+  futhark_device_ptr futhark_values_raw_##NAME##_2d(struct futhark_context *ctx,               \
+                                                    struct futhark_##NAME##_2d *arr);          \
+  const int64_t *futhark_shape_##NAME##_2d(struct futhark_context *ctx,                        \
+                                           struct futhark_##NAME##_2d *arr);
+
+#define FUTHARK_DECLARE_ARRAY_3D(NAME, CT)                                                     \
+  struct futhark_##NAME##_3d;                                                                  \
+  struct futhark_##NAME##_3d *futhark_new_##NAME##_3d(struct futhark_context *ctx,             \
+                                                      const CT *data, int64_t dim0,            \
+                                                      int64_t dim1, int64_t dim2);             \
+  struct futhark_##NAME##_3d *futhark_new_raw_##NAME##_3d(struct futhark_context *ctx,         \
+                                                          futhark_device_ptr data,             \
+                                                          int64_t dim0, int64_t dim1,          \
+                                                          int64_t dim2);                       \
+  int futhark_free_##NAME##_3d(struct futhark_context *ctx, struct futhark_##NAME##_3d *arr);  \
+  int futhark_values_##NAME##_3d(struct futhark_context *ctx, struct futhark_##NAME##_3d *arr, \
+                                 CT *data);                                                    \
+  int futhark_index_##NAME##_3d(struct futhark_context *ctx, CT *out,                          \
+                                struct futhark_##NAME##_3d *arr, int64_t i0, int64_t i1,       \
+                                int64_t i2);                                                   \
+  futhark_device_ptr futhark_values_raw_##NAME##_3d(struct futhark_context *ctx,               \
+                                                    struct futhark_##NAME##_3d *arr);          \
+  const int64_t *futhark_shape_##NAME##_3d(struct futhark_context *ctx,                        \
+                                           struct futhark_##NAME##_3d *arr);
+
+FUTHARK_DECLARE_ARRAY_1D(i32, int32_t)
+FUTHARK_DECLARE_ARRAY_1D(i64, int64_t)
+FUTHARK_DECLARE_ARRAY_1D(u8, uint8_t)
+FUTHARK_DECLARE_ARRAY_1D(u32, uint32_t)
+FUTHARK_DECLARE_ARRAY_1D(u64, uint64_t)
+FUTHARK_DECLARE_ARRAY_1D(f32, float)
+FUTHARK_DECLARE_ARRAY_1D(f64, double)
+FUTHARK_DECLARE_ARRAY_2D(i32, int32_t)
+FUTHARK_DECLARE_ARRAY_2D(i64, int64_t)
+FUTHARK_DECLARE_ARRAY_2D(f32, float)
+FUTHARK_DECLARE_ARRAY_2D(f64, double)
+FUTHARK_DECLARE_ARRAY_3D(f32, float)
+FUTHARK_DECLARE_ARRAY_3D(f16, uint16_t) /* f16 crosses the API as its bits */
+FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
+
+/* ----------------------------------------------------------- Entry points
+ * int futhark_entry_NAME(ctx, outputs..., inputs...): 0 on success; scalar
+ * outputs are valid after futhark_context_sync; array outputs are new values
+ * the caller frees. */
+#define FUTHARK_FOR_EACH_NUM_TYPE(X) X(i32, int32_t) X(i64, int64_t) X(f32, float) X(f64, double)
+#define FUTHARK_FOR_EACH_OP(X, T, CT) X(add, T, CT) X(max, T, CT) X(min, T, CT)
+
+#define FUTHARK_DECLARE_SEGOP_ENTRIES(OP, T, CT)                                              \
+  int futhark_entry_reduce_##OP##_##T(struct futhark_context *ctx, CT *out0,                  \
+                                      const struct futhark_##T##_1d *in0);                    \
+  int futhark_entry_scan_##OP##_##T(struct futhark_context *ctx,                              \
+                                    struct futhark_##T##_1d **out0,                           \
+                                    const struct futhark_##T##_1d *in0);                      \
+  int futhark_entry_exscan_##OP##_##T(struct futhark_context *ctx,                            \
+                                      struct futhark_##T##_1d **out0,                         \
+                                      const struct futhark_##T##_1d *in0);                    \
+  int futhark_entry_segscan_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_1d **out0,                        \
+                                       const struct futhark_u8_1d *in0,                       \
+                                       const struct futhark_##T##_1d *in1);                   \
+  int futhark_entry_segred_##OP##_##T(struct futhark_context *ctx,                            \
+                                      struct futhark_##T##_1d **out0,                         \
+                                      const struct futhark_i64_1d *in0,                       \
+                                      const struct futhark_i64_1d *in1,                       \
+                                      const struct futhark_##T##_1d *in2);                    \
+  int futhark_entry_segreduce_##OP##_##T(struct futhark_context *ctx,                         \
+                                         struct futhark_##T##_1d **out0,                      \
+                                         const struct futhark_##T##_2d *in0);                 \
+  int futhark_entry_hist_##OP##_##T(struct futhark_context *ctx,                              \
+                                    struct futhark_##T##_1d **out0, const int64_t in0,        \
+                                    const struct futhark_i32_1d *in1,                         \
+                                    const struct futhark_##T##_1d *in2);                      \
+  int futhark_entry_rbi_##OP##_##T(struct futhark_context *ctx,                               \
+                                   struct futhark_##T##_1d **out0,                            \
+                                   const struct futhark_##T##_1d *in0,                        \
+                                   const struct futhark_i32_1d *in1,                          \
+                                   const struct futhark_##T##_1d *in2);
+
+#define FUTHARK_DECLARE_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(FUTHARK_DECLARE_SEGOP_ENTRIES, T, CT)
+FUTHARK_FOR_EACH_NUM_TYPE(FUTHARK_DECLARE_FOR_TYPE)
+
+int futhark_entry_bmm_f32(struct futhark_context *ctx, struct futhark_f32_3d **out0,
+                          const struct futhark_f32_3d *in0, const struct futhark_f32_3d *in1);
+int futhark_entry_bmm_f16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
+                          const struct futhark_f16_3d *in0, const struct futhark_f16_3d *in1);
+int futhark_entry_bmm_bf16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
+                           const struct futhark_u16_3d *in0, const struct futhark_u16_3d *in1);
+int futhark_entry_matmul_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
+                             const struct futhark_f32_2d *in0, const struct futhark_f32_2d *in1);
+
+int futhark_entry_radix_sort_u32(struct futhark_context *ctx, struct futhark_u32_1d **out0,
+                                 const struct futhark_u32_1d *in0);
+int futhark_entry_radix_sort_u64(struct futhark_context *ctx, struct futhark_u64_1d **out0,
+                                 const struct futhark_u64_1d *in0);
+int futhark_entry_radix_sort_pairs_u32_i32(struct futhark_context *ctx,
+                                           struct futhark_u32_1d **out0,
+                                           struct futhark_i32_1d **out1,
+                                           const struct futhark_u32_1d *in0,
+                                           const struct futhark_i32_1d *in1);
+int futhark_entry_radix_sort_pairs_u64_i32(struct futhark_context *ctx,
+                                           struct futhark_u64_1d **out0,
+                                           struct futhark_i32_1d **out1,
+                                           const struct futhark_u64_1d *in0,
+                                           const struct futhark_i32_1d *in1);
+
+int futhark_entry_transpose_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
+                                const struct futhark_f32_2d *in0);
+int futhark_entry_iota_i64(struct futhark_context *ctx, struct futhark_i64_1d **out0,
+                           const int64_t in0);
+int futhark_entry_replicate_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
+                                const int64_t in0, const int32_t in1);
+
+/* ---------------------------------------------------------- Miscellaneous */
+int futhark_context_sync(struct futhark_context *ctx);
+char *futhark_context_get_error(struct futhark_context *ctx); /* caller frees */
+void futhark_context_set_logging_file(struct futhark_context *ctx, FILE *f);
+void futhark_context_pause_profiling(struct futhark_context *ctx);
+void futhark_context_unpause_profiling(struct futhark_context *ctx);
+char *futhark_context_report(struct futhark_context *ctx); /* JSON; caller frees */
+int futhark_context_clear_caches(struct futhark_context *ctx);
+
+/* Not part of the reference API: the HIP stream all work of this context is
+ * queued on, for callers that time kernels with their own events. */
+void *futhark_context_get_stream(struct futhark_context *ctx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SEGOPS_H */

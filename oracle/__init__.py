@@ -1,0 +1,207 @@
+"""ctypes loader for the CPU oracle (liboracle.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and the
+cpu_baseline leg of bench.py, never by the product.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import subprocess
+from pathlib import Path
+
+import numpy as np
+
+_DIR = Path(__file__).resolve().parent
+_LIB = None
+
+_CT = {"i32": (C.c_int32, np.int32), "i64": (C.c_int64, np.int64),
+       "f32": (C.c_float, np.float32), "f64": (C.c_double, np.float64)}
+
+
+def lib() -> C.CDLL:
+    global _LIB
+    if _LIB is None:
+        so = _DIR / "liboracle.so"
+        if not so.exists():
+            subprocess.check_call(["make", "-C", str(_DIR), "-s"])
+        _LIB = C.CDLL(str(so))
+    return _LIB
+
+
+def _p(a: np.ndarray):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def _arr(x, dt):
+    return np.ascontiguousarray(x, dtype=dt)
+
+
+def reduce(op: str, t: str, xs, variant: str = "lit"):
+    ct, dt = _CT[t]
+    xs = _arr(xs, dt)
+    fn = getattr(lib(), f"orc_reduce_{op}_{t}_{variant}")
+    fn.restype = ct
+    fn.argtypes = [C.c_void_p, C.c_int64]
+    return dt(fn(_p(xs), xs.size))
+
+
+def scan(op: str, t: str, xs, variant: str = "lit", exclusive: bool = False):
+    _, dt = _CT[t]
+    xs = _arr(xs, dt)
+    out = np.empty_like(xs)
+    fn = getattr(lib(), f"orc_{'ex' if exclusive else ''}scan_{op}_{t}_{variant}")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_void_p]
+    fn(_p(xs), xs.size, _p(out))
+    return out
+
+
+def segscan(op: str, t: str, flags, xs, variant: str = "lit"):
+    _, dt = _CT[t]
+    xs, flags = _arr(xs, dt), _arr(flags, np.uint8)
+    assert xs.size == flags.size
+    out = np.empty_like(xs)
+    fn = getattr(lib(), f"orc_segscan_{op}_{t}_{variant}")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+    fn(_p(flags), _p(xs), xs.size, _p(out))
+    return out
+
+
+def segred(op: str, t: str, offsets, lens, xs, variant: str = "lit"):
+    _, dt = _CT[t]
+    xs, offsets, lens = _arr(xs, dt), _arr(offsets, np.int64), _arr(lens, np.int64)
+    out = np.empty(offsets.size, dtype=dt)
+    fn = getattr(lib(), f"orc_segred_{op}_{t}_{variant}")
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p]
+    fn(_p(offsets), _p(lens), offsets.size, _p(xs), xs.size, _p(out))
+    return out
+
+
+def segreduce(op: str, t: str, xss):
+    _, dt = _CT[t]
+    xss = _arr(xss, dt)
+    m, k = xss.shape
+    out = np.empty(m, dtype=dt)
+    fn = getattr(lib(), f"orc_segreduce_{op}_{t}_lit")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
+    fn(_p(xss), m, k, _p(out))
+    return out
+
+
+def rbi(op: str, t: str, dest, is_, vs, variant: str = "lit"):
+    """reduce_by_index on a copy of dest."""
+    _, dt = _CT[t]
+    dest = _arr(dest, dt).copy()
+    is_, vs = _arr(is_, np.int32), _arr(vs, dt)
+    assert is_.size == vs.size
+    fn = getattr(lib(), f"orc_rbi_{op}_{t}_{variant}")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64]
+    fn(_p(dest), dest.size, _p(is_), _p(vs), is_.size)
+    return dest
+
+
+NEUTRAL = {
+    ("add", "i32"): 0, ("max", "i32"): np.iinfo(np.int32).min, ("min", "i32"): np.iinfo(np.int32).max,
+    ("add", "i64"): 0, ("max", "i64"): np.iinfo(np.int64).min, ("min", "i64"): np.iinfo(np.int64).max,
+    ("add", "f32"): 0.0, ("max", "f32"): -np.inf, ("min", "f32"): np.inf,
+    ("add", "f64"): 0.0, ("max", "f64"): -np.inf, ("min", "f64"): np.inf,
+}
+
+
+def hist(op: str, t: str, k: int, is_, vs, variant: str = "lit"):
+    _, dt = _CT[t]
+    return rbi(op, t, np.full(k, NEUTRAL[(op, t)], dtype=dt), is_, vs, variant)
+
+
+def bmm_f32(A, B, variant: str = "f64acc"):
+    A, B = _arr(A, np.float32), _arr(B, np.float32)
+    if A.ndim == 2:
+        A, B = A[None], B[None]
+        squeeze = True
+    else:
+        squeeze = False
+    b, M, K = A.shape
+    _, K2, N = B.shape
+    assert K == K2 and B.shape[0] == b
+    out = np.empty((b, M, N), dtype=np.float32)
+    fn = getattr(lib(), f"orc_bmm_f32_{variant}")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p] * 3 + [C.c_int64] * 4
+    fn(_p(A), _p(B), _p(out), b, M, N, K)
+    return out[0] if squeeze else out
+
+
+def widen(bits, kind: str):
+    bits = _arr(bits, np.uint16)
+    out = np.empty(bits.shape, dtype=np.float32)
+    fn = getattr(lib(), f"orc_widen_{kind}")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+    fn(_p(bits), _p(out), bits.size)
+    return out
+
+
+def radix_sort(keys, vals=None):
+    keys = np.ascontiguousarray(keys)
+    ko = np.empty_like(keys)
+    fn = lib().orc_radix_sort
+    fn.restype = None
+    fn.argtypes = [C.c_void_p] * 4 + [C.c_int64, C.c_int, C.c_int]
+    if vals is None:
+        fn(_p(keys), _p(ko), None, None, keys.size, keys.itemsize, 0)
+        return ko
+    vals = np.ascontiguousarray(vals)
+    vo = np.empty_like(vals)
+    fn(_p(keys), _p(ko), _p(vals), _p(vo), keys.size, keys.itemsize, vals.itemsize)
+    return ko, vo
+
+
+def transpose_f32(x):
+    x = _arr(x, np.float32)
+    out = np.empty((x.shape[1], x.shape[0]), dtype=np.float32)
+    fn = lib().orc_transpose_f32
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]
+    fn(_p(x), _p(out), x.shape[0], x.shape[1])
+    return out
+
+
+# ---- futhark-multicore-style CPU baseline (oracle/multicore.c) -------------
+def mc_threads() -> int:
+    return int(lib().mc_num_threads())
+
+
+def mc_reduce_add(t: str, xs, threads: int | None = None):
+    ct, dt = _CT[t]
+    xs = _arr(xs, dt)
+    fn = getattr(lib(), f"mc_reduce_add_{t}")
+    fn.restype = ct
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int]
+    return dt(fn(_p(xs), xs.size, threads or mc_threads()))
+
+
+def mc_segscan(t: str, flags, xs, op: str = "add", threads: int | None = None, out=None):
+    _, dt = _CT[t]
+    xs = _arr(xs, dt)
+    fl = None if flags is None else _arr(flags, np.uint8)
+    if out is None:
+        out = np.empty_like(xs)
+    fn = getattr(lib(), f"mc_segscan_{t}")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int]
+    fn(None if fl is None else _p(fl), _p(xs), xs.size, _p(out), {"add": 0, "max": 1}[op],
+       threads or mc_threads())
+    return out
+
+
+def mc_rbi_add_i32(dest, is_, vs, threads: int | None = None):
+    dest = _arr(dest, np.int32).copy()
+    is_, vs = _arr(is_, np.int32), _arr(vs, np.int32)
+    fn = lib().mc_rbi_add_i32
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+    fn(_p(dest), dest.size, _p(is_), _p(vs), is_.size, threads or mc_threads())
+    return dest

@@ -1,0 +1,297 @@
+/*
+ * oracle.c -- CPU restatement of what `futhark c` computes for the SegOp path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  Nothing that ships may call into this file: only
+ * tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg load
+ * liboracle.so, and only as the checker / the timed CPU baseline.
+ *
+ * `futhark c` sequentialises every SOAC with
+ * src/Futhark/Transform/FirstOrderTransform.hs:
+ *   reduce/scan   acc = ne; for i < n: acc = op(acc, x[i])      (:613-656)
+ *   hist          in-order read-modify-write, out-of-range bins skipped (:505-560)
+ * and scalar operators mean what rts/c/scalar.h says: add wraps in two's
+ * complement (:29-30), smax/smin (:488-503), fmax/fmin = fmaxf/fminf (:931-934).
+ * Functions named *_lit follow that evaluation order literally in the element
+ * type.  Functions named *_f64acc accumulate floating-point sums in double
+ * and round once per output; they are the yardstick for the 1e-5 tolerance,
+ * because any parallel schedule reassociates and the literal f32 fold is itself
+ * far from the exact sum at these sizes.
+ *
+ * Pinning (tests/test_oracle_golden.py): every function here is checked
+ * against the golden vectors the reference's own tests hold (tests/golden/),
+ * and against numpy closed forms / library routines on seeded inputs.
+ * bf16 matmul has no Futhark program to compare with (no such type in the
+ * reference): parity unpinned for orc_bmm_bf16 beyond its definition
+ * (bits << 16, then the f32 path).
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ----------------------------------------------------------- scalar ops */
+#define OPS_INT(T, U, S)                                                        \
+  static inline T add_##S(T a, T b) { return (T)((U)a + (U)b); }                \
+  static inline T max_##S(T a, T b) { return a < b ? b : a; }                   \
+  static inline T min_##S(T a, T b) { return a < b ? a : b; }
+OPS_INT(int32_t, uint32_t, i32)
+OPS_INT(int64_t, uint64_t, i64)
+static inline float add_f32(float a, float b) { return a + b; }
+static inline float max_f32(float a, float b) { return fmaxf(a, b); }
+static inline float min_f32(float a, float b) { return fminf(a, b); }
+static inline double add_f64(double a, double b) { return a + b; }
+static inline double max_f64(double a, double b) { return fmax(a, b); }
+static inline double min_f64(double a, double b) { return fmin(a, b); }
+
+/* neutral elements: 0, T.lowest, T.highest (prelude/math.fut:555-556,633-634,1077-1078) */
+#define NE_add_i32 0
+#define NE_max_i32 INT32_MIN
+#define NE_min_i32 INT32_MAX
+#define NE_add_i64 0
+#define NE_max_i64 INT64_MIN
+#define NE_min_i64 INT64_MAX
+#define NE_add_f32 0.0f
+#define NE_max_f32 (-INFINITY)
+#define NE_min_f32 (INFINITY)
+#define NE_add_f64 0.0
+#define NE_max_f64 (-(double)INFINITY)
+#define NE_min_f64 ((double)INFINITY)
+
+/* ------------------------------------- reduce / scan / segmented, literal
+ * FirstOrderTransform.hs:613-656; flag-tuple operator
+ * src/Futhark/Pass/Flatten/Builtins.hs:374-393; exclusive scan
+ * prelude/soacs.fut:212-215; irregular segmented reduce Builtins.hs:570-602. */
+#define DEFINE_LIT(OP, S, T)                                                                   \
+  T orc_reduce_##OP##_##S##_lit(const T *xs, int64_t n) {                                      \
+    T acc = NE_##OP##_##S;                                                                     \
+    for (int64_t i = 0; i < n; i++) acc = OP##_##S(acc, xs[i]);                                \
+    return acc;                                                                                \
+  }                                                                                            \
+  void orc_scan_##OP##_##S##_lit(const T *xs, int64_t n, T *out) {                             \
+    T acc = NE_##OP##_##S;                                                                     \
+    for (int64_t i = 0; i < n; i++) {                                                          \
+      acc = OP##_##S(acc, xs[i]);                                                              \
+      out[i] = acc;                                                                            \
+    }                                                                                          \
+  }                                                                                            \
+  void orc_exscan_##OP##_##S##_lit(const T *xs, int64_t n, T *out) {                           \
+    T acc = NE_##OP##_##S;                                                                     \
+    for (int64_t i = 0; i < n; i++) {                                                          \
+      out[i] = acc;                                                                            \
+      acc = OP##_##S(acc, xs[i]);                                                              \
+    }                                                                                          \
+  }                                                                                            \
+  void orc_segscan_##OP##_##S##_lit(const uint8_t *flags, const T *xs, int64_t n, T *out) {    \
+    int af = 0;                                                                                \
+    T av = NE_##OP##_##S;                                                                      \
+    for (int64_t i = 0; i < n; i++) {                                                          \
+      const int yf = flags[i] != 0;                                                            \
+      av = yf ? xs[i] : OP##_##S(av, xs[i]);                                                   \
+      af = af || yf;                                                                           \
+      out[i] = av;                                                                             \
+    }                                                                                          \
+    (void)af;                                                                                  \
+  }                                                                                            \
+  /* returns 0, or 1 if an offset lies outside [0,n) for a non-empty segment */                \
+  int orc_segred_##OP##_##S##_lit(const int64_t *offsets, const int64_t *lens, int64_t m,      \
+                                  const T *xs, int64_t n, T *out) {                            \
+    uint8_t *flags = (uint8_t *)calloc((size_t)(n > 0 ? n : 1), 1);                            \
+    T *s = (T *)malloc(sizeof(T) * (size_t)(n > 0 ? n : 1));                                   \
+    for (int64_t i = 0; i < m; i++)                                                            \
+      if (offsets[i] >= 0 && offsets[i] < n) flags[offsets[i]] = 1; /* scatter drops OOB */    \
+    orc_segscan_##OP##_##S##_lit(flags, xs, n, s);                                             \
+    int bad = 0;                                                                               \
+    for (int64_t i = 0; i < m; i++) {                                                          \
+      if (lens[i] == 0) out[i] = NE_##OP##_##S;                                                \
+      else {                                                                                   \
+        const int64_t p = offsets[i] + lens[i] - 1;                                            \
+        if (p < 0 || p >= n) { bad = 1; out[i] = NE_##OP##_##S; }                              \
+        else out[i] = s[p];                                                                    \
+      }                                                                                        \
+    }                                                                                          \
+    free(flags);                                                                               \
+    free(s);                                                                                   \
+    return bad;                                                                                \
+  }                                                                                            \
+  void orc_segreduce_##OP##_##S##_lit(const T *xss, int64_t m, int64_t k, T *out) {            \
+    for (int64_t i = 0; i < m; i++) out[i] = orc_reduce_##OP##_##S##_lit(xss + i * k, k);      \
+  }                                                                                            \
+  /* hist / reduce_by_index: FirstOrderTransform.hs:505-560 */                                 \
+  void orc_rbi_##OP##_##S##_lit(T *dest, int64_t H, const int32_t *is, const T *vs,            \
+                                int64_t n) {                                                   \
+    for (int64_t i = 0; i < n; i++) {                                                          \
+      const int64_t b = (int64_t)is[i];                                                        \
+      if (b >= 0 && b < H) dest[b] = OP##_##S(dest[b], vs[i]);                                 \
+    }                                                                                          \
+  }
+
+#define DEFINE_LIT_ALL_OPS(S, T) DEFINE_LIT(add, S, T) DEFINE_LIT(max, S, T) DEFINE_LIT(min, S, T)
+DEFINE_LIT_ALL_OPS(i32, int32_t)
+DEFINE_LIT_ALL_OPS(i64, int64_t)
+DEFINE_LIT_ALL_OPS(f32, float)
+DEFINE_LIT_ALL_OPS(f64, double)
+
+/* ------------------------------- f32 sums accumulated in double (yardstick) */
+float orc_reduce_add_f32_f64acc(const float *xs, int64_t n) {
+  double acc = 0.0;
+  for (int64_t i = 0; i < n; i++) acc += (double)xs[i];
+  return (float)acc;
+}
+void orc_scan_add_f32_f64acc(const float *xs, int64_t n, float *out) {
+  double acc = 0.0;
+  for (int64_t i = 0; i < n; i++) {
+    acc += (double)xs[i];
+    out[i] = (float)acc;
+  }
+}
+void orc_exscan_add_f32_f64acc(const float *xs, int64_t n, float *out) {
+  double acc = 0.0;
+  for (int64_t i = 0; i < n; i++) {
+    out[i] = (float)acc;
+    acc += (double)xs[i];
+  }
+}
+void orc_segscan_add_f32_f64acc(const uint8_t *flags, const float *xs, int64_t n, float *out) {
+  double acc = 0.0;
+  for (int64_t i = 0; i < n; i++) {
+    acc = flags[i] ? (double)xs[i] : acc + (double)xs[i];
+    out[i] = (float)acc;
+  }
+}
+void orc_segred_add_f32_f64acc(const int64_t *offsets, const int64_t *lens, int64_t m,
+                               const float *xs, int64_t n, float *out) {
+  /* Segments that tile the array: the sum of a segment is the scanned value at
+   * its last element. */
+  for (int64_t i = 0; i < m; i++) {
+    double acc = 0.0;
+    for (int64_t j = offsets[i]; j < offsets[i] + lens[i] && j < n; j++) acc += (double)xs[j];
+    out[i] = (float)acc;
+  }
+}
+void orc_rbi_add_f32_f64acc(float *dest, int64_t H, const int32_t *is, const float *vs,
+                            int64_t n) {
+  double *acc = (double *)malloc(sizeof(double) * (size_t)(H > 0 ? H : 1));
+  for (int64_t b = 0; b < H; b++) acc[b] = (double)dest[b];
+  for (int64_t i = 0; i < n; i++) {
+    const int64_t b = (int64_t)is[i];
+    if (b >= 0 && b < H) acc[b] += (double)vs[i];
+  }
+  for (int64_t b = 0; b < H; b++) dest[b] = (float)acc[b];
+  free(acc);
+}
+
+/* ------------------------------------------------------------------ matmul
+ * tests/reg-tiling/mmm.fut:17-21: C[i][j] = reduce (+) 0 (map2 (*) A[i,:] B[:,j]),
+ * batched with an outer map2.  `lit` keeps products and the running sum in f32
+ * in k order; `f64acc` accumulates in double. */
+void orc_bmm_f32_lit(const float *A, const float *B, float *C, int64_t b, int64_t M, int64_t N,
+                     int64_t K) {
+  for (int64_t q = 0; q < b; q++)
+    for (int64_t i = 0; i < M; i++)
+      for (int64_t j = 0; j < N; j++) {
+        float acc = 0.0f;
+        for (int64_t k = 0; k < K; k++)
+          acc = acc + A[(q * M + i) * K + k] * B[(q * K + k) * N + j];
+        C[(q * M + i) * N + j] = acc;
+      }
+}
+void orc_bmm_f32_f64acc(const float *A, const float *B, float *C, int64_t b, int64_t M,
+                        int64_t N, int64_t K) {
+  double *row = (double *)malloc(sizeof(double) * (size_t)(N > 0 ? N : 1));
+  for (int64_t q = 0; q < b; q++)
+    for (int64_t i = 0; i < M; i++) {
+      for (int64_t j = 0; j < N; j++) row[j] = 0.0;
+      for (int64_t k = 0; k < K; k++) {
+        const double a = (double)A[(q * M + i) * K + k];
+        const float *brow = B + (q * K + k) * N;
+        for (int64_t j = 0; j < N; j++) row[j] += a * (double)brow[j];
+      }
+      for (int64_t j = 0; j < N; j++) C[(q * M + i) * N + j] = (float)row[j];
+    }
+  free(row);
+}
+
+/* f16 -> f32, exact (every binary16 value is a binary32 value); what
+ * rts/c/half.h:220-236 computes with tables. */
+float orc_f16_to_f32(uint16_t h) {
+  const uint32_t sign = (uint32_t)(h >> 15) << 31;
+  const uint32_t exp = (h >> 10) & 0x1f, man = h & 0x3ff;
+  uint32_t bits;
+  if (exp == 0) {
+    if (man == 0) bits = sign;
+    else {
+      /* subnormal: value = man * 2^-24 */
+      float f = (float)man * 5.9604644775390625e-08f;
+      memcpy(&bits, &f, 4);
+      bits |= sign;
+    }
+  } else if (exp == 31) bits = sign | 0x7f800000u | (man << 13);
+  else bits = sign | ((exp + 112) << 23) | (man << 13);
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+float orc_bf16_to_f32(uint16_t h) {
+  const uint32_t bits = (uint32_t)h << 16;
+  float f;
+  memcpy(&f, &bits, 4);
+  return f;
+}
+/* 16-bit inputs widened to f32, then the f32 matmul (Appendix programs bmm_f16/bmm_bf16:
+ * f32.f16 x * f32.f16 y summed in f32). */
+void orc_widen_f16(const uint16_t *in, float *out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) out[i] = orc_f16_to_f32(in[i]);
+}
+void orc_widen_bf16(const uint16_t *in, float *out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) out[i] = orc_bf16_to_f32(in[i]);
+}
+
+/* -------------------------------------------------------------- radix sort
+ * Stable LSD radix sort, 8-bit digits: per pass a histogram of the digit, an
+ * exclusive scan of the 256 counts, and an in-order scatter (the composition of
+ * tests/issue2234.fut:10-44 with 8-bit instead of 2-bit digits).  Keys compare
+ * as unsigned; vals may be NULL. */
+static void radix_pass(const uint8_t *kin, uint8_t *kout, const uint8_t *vin, uint8_t *vout,
+                       int64_t n, int kb, int vb, int shift) {
+  int64_t count[256] = {0}, start[256];
+  for (int64_t i = 0; i < n; i++) {
+    uint64_t k = 0;
+    memcpy(&k, kin + i * kb, (size_t)kb);
+    count[(k >> shift) & 0xff]++;
+  }
+  int64_t acc = 0;
+  for (int d = 0; d < 256; d++) {
+    start[d] = acc;
+    acc += count[d];
+  }
+  for (int64_t i = 0; i < n; i++) {
+    uint64_t k = 0;
+    memcpy(&k, kin + i * kb, (size_t)kb);
+    const int64_t p = start[(k >> shift) & 0xff]++;
+    memcpy(kout + p * kb, kin + i * kb, (size_t)kb);
+    if (vin) memcpy(vout + p * vb, vin + i * vb, (size_t)vb);
+  }
+}
+void orc_radix_sort(const void *keys, void *keys_out, const void *vals, void *vals_out,
+                    int64_t n, int key_bytes, int val_bytes) {
+  const size_t kbytes = (size_t)(n > 0 ? n : 1) * (size_t)key_bytes;
+  const size_t vbytes = (size_t)(n > 0 ? n : 1) * (size_t)(val_bytes > 0 ? val_bytes : 1);
+  uint8_t *ka = (uint8_t *)malloc(kbytes), *kb2 = (uint8_t *)malloc(kbytes);
+  uint8_t *va = vals ? (uint8_t *)malloc(vbytes) : NULL, *vb2 = vals ? (uint8_t *)malloc(vbytes) : NULL;
+  memcpy(ka, keys, (size_t)n * (size_t)key_bytes);
+  if (vals) memcpy(va, vals, (size_t)n * (size_t)val_bytes);
+  for (int pass = 0; pass < key_bytes; pass++) {
+    radix_pass(ka, kb2, va, vb2, n, key_bytes, val_bytes, 8 * pass);
+    uint8_t *t = ka; ka = kb2; kb2 = t;
+    t = va; va = vb2; vb2 = t;
+  }
+  memcpy(keys_out, ka, (size_t)n * (size_t)key_bytes);
+  if (vals) memcpy(vals_out, va, (size_t)n * (size_t)val_bytes);
+  free(ka); free(kb2); free(va); free(vb2);
+}
+
+/* --------------------------------------------------------- data movement */
+void orc_transpose_f32(const float *in, float *out, int64_t rows, int64_t cols) {
+  for (int64_t i = 0; i < rows; i++)
+    for (int64_t j = 0; j < cols; j++) out[j * rows + i] = in[i * cols + j];
+}

@@ -1,0 +1,216 @@
+"""GPU parity: SegRed and SegScan through the generated-library API against the
+CPU oracle.  Integers bit-exact; f32 sums within 1e-5 relative of the
+f64-accumulated oracle; max/min bit-exact (order-independent)."""
+import numpy as np
+import pytest
+
+import oracle
+from futhark_amd import datagen as dg
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 3, 63, 64, 65, 255, 1023, 4095, 4096, 4097, 8191, 100003, (1 << 20) + 7]
+NP = {"i32": np.int32, "i64": np.int64, "f32": np.float32, "f64": np.float64}
+F32_RTOL = 1e-5
+
+
+def _data(t, n, aid):
+    if t in ("i32", "i64"):
+        return dg.uniform_int(aid, n, -1000 if t == "i32" else -(1 << 20),
+                              1000 if t == "i32" else (1 << 20), NP[t])
+    x = dg.uniform_f32(aid, n)
+    return x.astype(NP[t])
+
+
+def _close(got, want, rtol=F32_RTOL):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    err = np.abs(got - want)
+    bound = rtol * np.abs(want) + 1e-30
+    bad = err > bound
+    assert not bad.any(), (int(bad.sum()), float((err / (np.abs(want) + 1e-30)).max()))
+
+
+@pytest.mark.parametrize("t", ["i32", "i64", "f32", "f64"])
+@pytest.mark.parametrize("op", ["add", "max", "min"])
+def test_reduce_sizes(ctx, t, op):
+    for n in SIZES:
+        xs = _data(t, n, 1)
+        a = ctx.new(f"{t}_1d", xs)
+        got = ctx.call(f"reduce_{op}_{t}", [NP[t]], a)
+        a.free()
+        if op == "add" and t == "f32":
+            _close(got, oracle.reduce(op, t, xs, "f64acc"))
+        elif op == "add" and t == "f64":
+            _close(got, np.sum(xs.astype(np.longdouble)), 1e-12)
+        else:
+            assert got == oracle.reduce(op, t, xs), (n, got)
+
+
+@pytest.mark.parametrize("t", ["i32", "i64", "f32", "f64"])
+@pytest.mark.parametrize("op", ["add", "max"])
+@pytest.mark.parametrize("excl", [False, True])
+def test_scan_sizes(ctx, t, op, excl):
+    for n in SIZES:
+        xs = _data(t, n, 2)
+        a = ctx.new(f"{t}_1d", xs)
+        out = ctx.call(f"{'ex' if excl else ''}scan_{op}_{t}", [f"{t}_1d"], a)
+        got = out.values()
+        assert got.shape == (n,)
+        a.free(); out.free()
+        if op == "add" and t == "f32":
+            _close(got, oracle.scan(op, t, xs, "f64acc", exclusive=excl))
+        elif op == "add" and t == "f64":
+            want = np.cumsum(xs.astype(np.longdouble))
+            if excl:
+                want = np.concatenate(([0], want[:-1]))
+            _close(got, want, 1e-12)
+        else:
+            assert np.array_equal(got, oracle.scan(op, t, xs, exclusive=excl)), n
+
+
+@pytest.mark.parametrize("t", ["i32", "i64", "f32"])
+@pytest.mark.parametrize("op", ["add", "max", "min"])
+def test_segscan_sizes(ctx, t, op):
+    for n in SIZES:
+        xs = _data(t, n, 3)
+        for mean in (3, 700, 10 ** 9):  # many short, tile-sized, one segment without flags[0]
+            flags = (dg.raw_u64(77 + mean % 13, n) % np.uint64(mean) == 0).astype(np.uint8)
+            a, f = ctx.new(f"{t}_1d", xs), ctx.new("u8_1d", flags)
+            out = ctx.call(f"segscan_{op}_{t}", [f"{t}_1d"], f, a)
+            got = out.values()
+            a.free(); f.free(); out.free()
+            if op == "add" and t == "f32":
+                _close(got, oracle.segscan(op, t, flags, xs, "f64acc"))
+            else:
+                assert np.array_equal(got, oracle.segscan(op, t, flags, xs)), (n, mean)
+
+
+def test_segscan_flag_bytes_other_than_one(ctx):
+    xs = np.arange(1, 1001, dtype=np.int32)
+    flags = np.zeros(1000, np.uint8)
+    flags[[0, 10, 500, 999]] = [255, 2, 128, 7]  # nonzero means start (map (!=0))
+    a, f = ctx.new("i32_1d", xs), ctx.new("u8_1d", flags)
+    out = ctx.call("segscan_add_i32", ["i32_1d"], f, a)
+    assert np.array_equal(out.values(), oracle.segscan("add", "i32", flags, xs))
+
+
+@pytest.mark.parametrize("t", ["i32", "i64", "f32"])
+@pytest.mark.parametrize("op", ["add", "max"])
+def test_segred_irregular(ctx, t, op):
+    for n in [1, 5, 4096, 4097, 100003, (1 << 20) + 7]:
+        for mean in (2, 50, 1024, 1 << 22):
+            offsets, lens, flags = dg.segments(5, n, mean)
+            # sprinkle empty segments (tests/flattening/reduce/nonuniform-2d.fut has one)
+            if len(offsets) > 3:
+                pos = [0, len(offsets) // 2, len(offsets)]
+                offsets = np.insert(offsets, pos, [0, offsets[len(offsets) // 2], n])
+                lens = np.insert(lens, pos, [0, 0, 0])
+            xs = _data(t, n, 4)
+            o, l, v = ctx.new("i64_1d", offsets), ctx.new("i64_1d", lens), ctx.new(f"{t}_1d", xs)
+            out = ctx.call(f"segred_{op}_{t}", [f"{t}_1d"], o, l, v)
+            got = out.values()
+            for h in (o, l, v, out):
+                h.free()
+            if op == "add" and t == "f32":
+                _close(got, oracle.segred(op, t, offsets, lens, xs, "f64acc"))
+            else:
+                assert np.array_equal(got, oracle.segred(op, t, offsets, lens, xs)), (n, mean)
+
+
+def test_segred_all_empty_and_no_segments(ctx):
+    o = ctx.new("i64_1d", np.zeros(4, np.int64)); l = ctx.new("i64_1d", np.zeros(4, np.int64))
+    v = ctx.new("f32_1d", np.zeros(0, np.float32))
+    out = ctx.call("segred_max_f32", ["f32_1d"], o, l, v)
+    assert np.array_equal(out.values(), np.full(4, -np.inf, np.float32))
+    e = ctx.new("i64_1d", np.zeros(0, np.int64))
+    v2 = ctx.new("f32_1d", np.ones(10, np.float32))
+    out2 = ctx.call("segred_add_f32", ["f32_1d"], e, e, v2)
+    assert out2.values().shape == (0,)
+
+
+def test_reference_goldens_on_gpu(ctx, goldens):
+    for c in goldens["reduce0"]["cases"]:
+        xs = np.arange(c["n"], dtype=np.int64).astype(np.int32)
+        assert int(ctx.call("reduce_add_i32", [np.int32], ctx.new("i32_1d", xs))) == c["out"]
+    for c in goldens["scan0"]["cases"]:
+        xs = np.arange(c["n"], dtype=np.int64).astype(np.int32)
+        out = ctx.call("scan_add_i32", ["i32_1d"], ctx.new("i32_1d", xs))
+        assert int(out.index(c["n"] - 1)) == c["out"]
+    for c in goldens["exscan0"]["cases"]:
+        xs = np.arange(c["n"], dtype=np.int64).astype(np.int32)
+        out = ctx.call("exscan_add_i32", ["i32_1d"], ctx.new("i32_1d", xs))
+        assert int(out.index(c["n"] - 1)) == c["out"]
+    c = goldens["scan4"]["cases"][0]
+    xs = np.array(c["in"], np.int32)
+    for _ in range(2):
+        bits = ctx.new("i32_1d", xs + 1)
+        ps = ctx.call("scan_add_i32", ["i32_1d"], bits).values()
+        s = ctx.call("reduce_add_i32", [np.int32], bits)
+        xs = ps + s + xs
+    assert xs.tolist() == c["out"]
+    c = goldens["nonuniform_2d"]["cases"][0]
+    sizes = np.array(c["sizes"], np.int64)
+    lens = 3 * sizes
+    offsets = np.concatenate(([0], np.cumsum(lens)[:-1]))
+    vals = np.concatenate([(np.arange(3)[:, None] + np.arange(s)[None, :]).ravel() for s in sizes])
+    out = ctx.call("segred_add_i64", ["i64_1d"], ctx.new("i64_1d", offsets),
+                   ctx.new("i64_1d", lens), ctx.new("i64_1d", vals.astype(np.int64)))
+    assert out.values().tolist() == c["out"]
+
+
+@pytest.mark.parametrize("t", ["i32", "f32"])
+def test_segreduce_regular(ctx, goldens, t):
+    c = goldens["segsum"]["cases"][0]
+    out = ctx.call("segreduce_add_f32", ["f32_1d"], ctx.new("f32_2d", np.array(c["xss"], np.float32)))
+    assert out.values().tolist() == c["out"]
+    for m, k in [(1, 1), (1000, 1), (1000, 2), (777, 7), (300, 33), (100, 64), (50, 1000),
+                 (7, 9001), (3, 70000), (0, 5), (5, 0)]:
+        xss = _data(t, m * k, 9).reshape(m, k)
+        out = ctx.call(f"segreduce_add_{t}", [f"{t}_1d"], ctx.new(f"{t}_2d", xss))
+        got = out.values()
+        if t == "f32":
+            _close(got, xss.astype(np.float64).sum(axis=1))
+        else:
+            assert np.array_equal(got, oracle.segreduce("add", t, xss))
+        outm = ctx.call(f"segreduce_max_{t}", [f"{t}_1d"], ctx.new(f"{t}_2d", xss))
+        assert np.array_equal(outm.values(), oracle.segreduce("max", t, xss))
+
+
+def test_config1_full_size(ctx):
+    n = 1 << 24
+    xi = dg.uniform_int(16, n, -1000, 1000)
+    a = ctx.new("i32_1d", xi)
+    assert ctx.call("reduce_add_i32", [np.int32], a) == oracle.reduce("add", "i32", xi)
+    out = ctx.call("scan_add_i32", ["i32_1d"], a)
+    assert np.array_equal(out.values(), oracle.scan("add", "i32", xi))
+    a.free(); out.free()
+    xf = dg.uniform_f32(17, n)
+    a = ctx.new("f32_1d", xf)
+    _close(ctx.call("reduce_add_f32", [np.float32], a), oracle.reduce("add", "f32", xf, "f64acc"))
+    out = ctx.call("scan_add_f32", ["f32_1d"], a)
+    _close(out.values(), oracle.scan("add", "f32", xf, "f64acc"))
+
+
+@pytest.mark.parametrize("t,op", [("f32", "add"), ("f32", "max"), ("i64", "add"), ("i64", "max")])
+def test_config2_full_size(ctx, t, op):
+    n = 1 << 26
+    offsets, lens, flags = dg.segments(32, n, 1024)
+    xs = _data(t, n, 33)
+    f, v = ctx.new("u8_1d", flags), ctx.new(f"{t}_1d", xs)
+    out = ctx.call(f"segscan_{op}_{t}", [f"{t}_1d"], f, v)
+    got = out.values()
+    out.free()
+    if (t, op) == ("f32", "add"):
+        _close(got, oracle.segscan(op, t, flags, xs, "f64acc"))
+    else:
+        assert np.array_equal(got, oracle.segscan(op, t, flags, xs))
+    # size-independent property: last scanned element of a segment == its reduction
+    o, l = ctx.new("i64_1d", offsets), ctx.new("i64_1d", lens)
+    red = ctx.call(f"segred_{op}_{t}", [f"{t}_1d"], o, l, v).values()
+    ends = offsets + lens - 1
+    if (t, op) == ("f32", "add"):
+        _close(red, oracle.segred(op, t, offsets, lens, xs, "f64acc"))
+        _close(red, got[ends], 2e-6)
+    else:
+        assert np.array_equal(red, got[ends])
+        assert np.array_equal(red, oracle.segred(op, t, offsets, lens, xs))

@@ -1,0 +1,181 @@
+"""Pins the CPU oracle: reference-held golden vectors, closed forms and library
+routines.  Each check is chosen so that a plausible slip in the oracle (wrong
+neutral element, dropped wrap-around, off-by-one exclusive scan, unstable sort,
+transposed operand) fails it."""
+import numpy as np
+import pytest
+
+import oracle
+
+
+def _f(xs):
+    return np.array([np.nan if x == "nan" else x for x in xs], dtype=np.float32)
+
+
+def test_reduce0_iota_wraps(goldens):
+    for c in goldens["reduce0"]["cases"]:
+        xs = np.arange(c["n"], dtype=np.int64).astype(np.int32)
+        assert int(oracle.reduce("add", "i32", xs)) == c["out"]
+
+
+def test_scan0_and_exscan0(goldens):
+    for c in goldens["scan0"]["cases"]:
+        xs = np.arange(c["n"], dtype=np.int64).astype(np.int32)
+        assert int(oracle.scan("add", "i32", xs)[-1]) == c["out"]
+    for c in goldens["exscan0"]["cases"]:
+        xs = np.arange(c["n"], dtype=np.int64).astype(np.int32)
+        assert int(oracle.scan("add", "i32", xs, exclusive=True)[-1]) == c["out"]
+
+
+def test_scan4_radix_distilled(goldens):
+    for c in goldens["scan4"]["cases"]:
+        xs = np.array(c["in"], dtype=np.int32)
+        for _ in range(2):
+            bits = xs + 1
+            ps = oracle.scan("add", "i32", bits)
+            s = oracle.reduce("add", "i32", bits)
+            xs = ps + s + xs
+        assert xs.tolist() == c["out"]
+
+
+def test_hist_simple_large_max_min(goldens):
+    for c in goldens["hist_simple"]["cases"]:
+        img = np.array(c["image"], dtype=np.int32)
+        out = oracle.rbi("add", "i32", np.array(c["dest"], dtype=np.int32), img, img)
+        assert out.tolist() == c["out"]
+    for c in goldens["hist_large"]["cases"][:2] + goldens["hist_large"]["cases"][2:]:
+        n, m = c["n"], c["m"]
+        i = np.arange(m, dtype=np.int64)
+        h = oracle.hist("add", "i32", n, (i % n).astype(np.int32), i.astype(np.int32))
+        assert int(oracle.reduce("add", "i32", h)) == c["out"]
+    for name, op in (("hist_max", "max"), ("hist_min", "min")):
+        for c in goldens[name]["cases"]:
+            out = oracle.rbi(op, "i32", np.zeros(c["n"], np.int32), c["is"], c["vs"])
+            assert out.tolist() == c["out"]
+
+
+def test_hist_f32_including_nan(goldens):
+    for c in goldens["hist_f32"]["cases"]:
+        for variant in ("lit", "f64acc"):
+            out = oracle.rbi("add", "f32", _f(c["dest"]), c["is"], _f(c["vs"]), variant)
+            np.testing.assert_allclose(out, _f(c["out"]), rtol=2e-3, equal_nan=True)
+
+
+def test_hist_segmented(goldens):
+    c = goldens["hist_segmented"]["cases"][0]
+    for xs, want in zip(c["xss"], c["out"]):
+        got = oracle.hist("add", "i32", c["m"], xs, np.ones(len(xs), np.int32))
+        assert got.tolist() == want
+
+
+def test_segsum_and_segreduce_iota(goldens):
+    c = goldens["segsum"]["cases"][0]
+    assert oracle.segreduce("add", "f32", c["xss"]).tolist() == c["out"]
+    for c in goldens["segreduce_iota"]["cases"]:
+        n, m = c["n"], c["m"]
+        xss = np.repeat(np.arange(n, dtype=np.int32)[:, None], m, axis=1).reshape(n, m)
+        assert oracle.segreduce("add", "i32", xss).tolist() == c["out"]
+
+
+def test_irregular_segments_with_empty_segment(goldens):
+    c = goldens["nonuniform_2d"]["cases"][0]
+    sizes = np.array(c["sizes"], dtype=np.int64)
+    lens = 3 * sizes
+    offsets = np.concatenate(([0], np.cumsum(lens)[:-1]))
+    vals = np.concatenate([(np.arange(3)[:, None] + np.arange(s)[None, :]).ravel() for s in sizes])
+    out = oracle.segred("add", "i64", offsets, lens, vals.astype(np.int64))
+    assert out.tolist() == c["out"]
+
+
+def test_segscan_operator_against_per_segment_cumsum():
+    rng = np.random.default_rng(1)
+    n = 5000
+    flags = (rng.random(n) < 0.01).astype(np.uint8)
+    xs = rng.integers(-1000, 1000, n).astype(np.int64)
+    got = oracle.segscan("add", "i64", flags, xs)
+    want = np.empty_like(xs)
+    starts = [0] + [i for i in range(1, n) if flags[i]] + [n]
+    for a, b in zip(starts[:-1], starts[1:]):
+        want[a:b] = np.cumsum(xs[a:b])
+    assert np.array_equal(got, want)
+    # max restarts too, and flags[0] == 0 folds the neutral element in front
+    gm = oracle.segscan("max", "f32", flags, xs.astype(np.float32))
+    wm = np.empty(n, np.float32)
+    for a, b in zip(starts[:-1], starts[1:]):
+        wm[a:b] = np.maximum.accumulate(xs[a:b].astype(np.float32))
+    assert np.array_equal(gm, wm)
+
+
+def test_mmm_golden_and_numpy(goldens):
+    c = goldens["mmm"]["cases"][0]
+    for variant in ("lit", "f64acc"):
+        assert oracle.bmm_f32(c["A"], c["B"], variant).tolist() == c["out"]
+    rng = np.random.default_rng(2)
+    A = rng.standard_normal((3, 17, 29)).astype(np.float32)
+    B = rng.standard_normal((3, 29, 13)).astype(np.float32)
+    want = np.matmul(A.astype(np.float64), B.astype(np.float64))
+    np.testing.assert_allclose(oracle.bmm_f32(A, B, "f64acc"), want, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(oracle.bmm_f32(A, B, "lit"), want, rtol=1e-4, atol=1e-4)
+
+
+def test_f16_bf16_widening_is_exact():
+    bits = np.arange(0, 1 << 16, dtype=np.uint16)
+    want = bits.view(np.float16).astype(np.float32)
+    got = oracle.widen(bits, "f16")
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    gb = oracle.widen(bits, "bf16")
+    assert np.array_equal(gb.view(np.uint32), bits.astype(np.uint32) << 16)
+    # tests/f16kernel.fut: [1,2,3]f16 sums to 6
+    assert float(oracle.widen(np.array([1, 2, 3], np.float16).view(np.uint16), "f16").sum()) == 6.0
+
+
+def test_radix_sort_is_stable_and_matches_numpy(goldens):
+    c = goldens["radixsort"]["cases"][0]
+    keys = np.array(c["keys"], np.float32).view(np.uint32)  # positive floats order as u32
+    vals = np.array(c["vals"], np.float32)
+    ko, vo = oracle.radix_sort(keys, vals.view(np.uint32))
+    assert vo.view(np.float32).tolist() == np.array(c["out_vals"], np.float32).tolist()
+    rng = np.random.default_rng(3)
+    for dt in (np.uint32, np.uint64):
+        keys = rng.integers(0, 50, 20000).astype(dt) << dt(20 if dt == np.uint32 else 40)
+        idx = np.arange(keys.size, dtype=np.int32)
+        ko, vo = oracle.radix_sort(keys, idx)
+        perm = np.argsort(keys, kind="stable")
+        assert np.array_equal(ko, keys[perm]) and np.array_equal(vo, idx[perm])
+        full = rng.integers(0, np.iinfo(dt).max, 10000, dtype=dt)
+        assert np.array_equal(oracle.radix_sort(full), np.sort(full))
+
+
+def test_f64acc_variants_are_close_to_exact_and_lit_drifts():
+    rng = np.random.default_rng(4)
+    xs = rng.random(1 << 20).astype(np.float32)
+    exact = xs.astype(np.float64).cumsum()
+    got = oracle.scan("add", "f32", xs, "f64acc")
+    np.testing.assert_allclose(got, exact, rtol=1e-7)
+    lit = oracle.scan("add", "f32", xs, "lit")
+    assert np.array_equal(lit, np.cumsum(xs, dtype=np.float32))  # same left fold
+    ex = oracle.scan("add", "f32", xs, "f64acc", exclusive=True)
+    assert ex[0] == 0.0 and np.array_equal(ex[1:], got[:-1])
+
+
+def test_transpose():
+    x = np.arange(12, dtype=np.float32).reshape(3, 4)
+    assert np.array_equal(oracle.transpose_f32(x), x.T)
+
+
+def test_multicore_baseline_agrees_with_oracle():
+    rng = np.random.default_rng(5)
+    n = 300000
+    xs = rng.integers(-1000, 1000, n).astype(np.int32)
+    flags = (rng.random(n) < 0.001).astype(np.uint8)
+    assert oracle.mc_reduce_add("i32", xs, 4) == oracle.reduce("add", "i32", xs)
+    assert np.array_equal(oracle.mc_segscan("i32", None, xs, "add", 4), oracle.scan("add", "i32", xs))
+    assert np.array_equal(oracle.mc_segscan("i32", flags, xs, "add", 4),
+                          oracle.segscan("add", "i32", flags, xs))
+    assert np.array_equal(oracle.mc_segscan("i32", flags, xs, "max", 3),
+                          oracle.segscan("max", "i32", flags, xs))
+    is_ = rng.integers(-5, 300, n).astype(np.int32)
+    assert np.array_equal(oracle.mc_rbi_add_i32(np.zeros(256, np.int32), is_, xs, 4),
+                          oracle.rbi("add", "i32", np.zeros(256, np.int32), is_, xs))
+    big = oracle.mc_rbi_add_i32(np.zeros(200000, np.int32), is_, xs, 4)  # atomic path
+    assert np.array_equal(big, oracle.rbi("add", "i32", np.zeros(200000, np.int32), is_, xs))
