@@ -1,0 +1,231 @@
+#!/usr/bin/env python3
+"""Benchmark of the SegOp hot path on one MI355X.
+
+Default workload: segmented inclusive scan with (+) over 2^26 f32 values in
+irregular segments (geometric lengths, mean 1024, u8 start flags) -- the
+configuration the headline metric is quoted on.  One step = one
+futhark_entry_* call (one pass of the path over the resident input) followed
+by freeing its result; inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  `value` is whole-job throughput in GB/s over the
+algorithmic bytes of the workload; `roofline` prices the dominant kernel with
+HIP events recorded on the context's stream; `cpu_baseline` times the
+futhark-multicore-style CPU restatement (oracle/multicore.c) on the host cores.
+Other workloads (--workload) report the same fields for the other SegOps.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+
+
+def make_workload(name: str, ctx):
+    """Returns dict(step, bytes, unit_work, dtype, kernel, cpu, describe, bound)."""
+    from futhark_amd import datagen as dg
+    import oracle
+
+    w = {}
+    if name.startswith("segscan_") or name.startswith("segred_"):
+        kind, op, t, sz = name.split("_")
+        n = 1 << int(sz[2:])
+        es = 4 if t == "f32" else 8
+        offsets, lens, flags = dg.segments(32, n, 1024)
+        xs = dg.uniform_f32(33, n) if t == "f32" else dg.uniform_int(34, n, -(1 << 20), 1 << 20, np.int64)
+        v = ctx.new(f"{t}_1d", xs)
+        if kind == "segscan":
+            f = ctx.new("u8_1d", flags)
+
+            def step():
+                ctx.call(f"segscan_{op}_{t}", [f"{t}_1d"], f, v).free()
+            w["bytes"] = n * (2 * es + 1)
+            w["kernel"] = "segscan"
+            if t in ("f32", "i64"):
+                w["cpu"] = lambda out=np.empty_like(xs): oracle.mc_segscan(t, flags, xs, op, out=out)
+        else:
+            o, l = ctx.new("i64_1d", offsets), ctx.new("i64_1d", lens)
+
+            def step():
+                ctx.call(f"segred_{op}_{t}", [f"{t}_1d"], o, l, v).free()
+            w["bytes"] = n * es + len(offsets) * (8 + es)
+            w["kernel"] = "segred_irregular"
+        w.update(step=step, dtype=t, bound="hbm", keep=[v],
+                 describe=f"{kind} ({op}) over 2^{sz[2:]} {t}, {len(offsets)} irregular segments "
+                          f"(geometric, mean 1024), u8 flags / i64 offsets")
+    elif name.startswith("reduce_") or name.startswith("scan_"):
+        kind, op, t, sz = name.split("_")
+        n = 1 << int(sz[2:])
+        es = 4
+        xs = dg.uniform_f32(17, n) if t == "f32" else dg.uniform_int(16, n, -1000, 1000)
+        a = ctx.new(f"{t}_1d", xs)
+        if kind == "reduce":
+            nt = np.float32 if t == "f32" else np.int32
+
+            def step():
+                ctx.call(f"reduce_{op}_{t}", [nt], a)
+            w["bytes"] = n * es
+            w["kernel"] = "segred_nonseg"
+            w["cpu"] = lambda: oracle.mc_reduce_add(t, xs)
+        else:
+            def step():
+                ctx.call(f"scan_{op}_{t}", [f"{t}_1d"], a).free()
+            w["bytes"] = 2 * n * es
+            w["kernel"] = "segscan"
+            w["cpu"] = lambda out=np.empty_like(xs): oracle.mc_segscan(t, None, xs, op, out=out)
+        w.update(step=step, dtype=t, bound="hbm", keep=[a],
+                 describe=f"{kind} ({op}) over 2^{sz[2:]} {t}")
+    elif name.startswith("hist_"):
+        # hist_add_i32_H65536_uniform_2p27
+        _, op, t, hs, dist, sz = name.split("_")
+        n, H = 1 << int(sz[2:]), int(hs[1:])
+        is_ = dg.hist_indices(48, n, H, dist)
+        vs = dg.uniform_int(49, n, -1000, 1000) if t == "i32" else dg.uniform_f32(50, n)
+        i, v = ctx.new("i32_1d", is_), ctx.new(f"{t}_1d", vs)
+
+        def step():
+            ctx.call(f"hist_{op}_{t}", [f"{t}_1d"], H, i, v).free()
+        w.update(step=step, bytes=n * 8 + 2 * H * 4, kernel="seghist", dtype=t, bound="hbm",
+                 keep=[i, v], describe=f"hist ({op}) of 2^{sz[2:]} {t} into {H} bins, {dist} i32 "
+                                       f"indices, 1% out of range")
+        if t == "i32" and op == "add":
+            w["cpu"] = lambda: oracle.mc_rbi_add_i32(np.zeros(H, np.int32), is_, vs)
+    elif name.startswith("sort_"):
+        # sort_u32_2p26 | sort_u64i32_2p26
+        _, kt, sz = name.split("_")
+        n = 1 << int(sz[2:])
+        if kt == "u32":
+            k = ctx.new("u32_1d", dg.uniform_u32(80, n))
+
+            def step():
+                ctx.call("radix_sort_u32", ["u32_1d"], k).free()
+            w.update(bytes=4 * 12 * n, keep=[k])
+        else:
+            k = ctx.new("u64_1d", dg.uniform_u64(81, n))
+            vv = ctx.new("i32_1d", np.arange(n, dtype=np.int32))
+
+            def step():
+                a, b = ctx.call("radix_sort_pairs_u64_i32", ["u64_1d", "i32_1d"], k, vv)
+                a.free(); b.free()
+            w.update(bytes=8 * 32 * n, keep=[k, vv])
+        w.update(step=step, kernel="radix_sort", dtype=kt, bound="hbm",
+                 describe=f"stable LSD radix sort, 8-bit digits, 2^{sz[2:]} {kt}")
+    elif name.startswith("bmm_"):
+        # bmm_f16_1x4096 | bmm_f32_64x512
+        _, t, shape = name.split("_")
+        b, m = (int(x) for x in shape.split("x"))
+        sc = 1.0 / np.sqrt(m)
+        A = dg.normal_f32(64, b * m * m, sc).reshape(b, m, m)
+        B = dg.normal_f32(65, b * m * m, sc).reshape(b, m, m)
+        if t == "f32":
+            a, bb = ctx.new("f32_3d", A), ctx.new("f32_3d", B)
+        elif t == "f16":
+            a, bb = ctx.new("f16_3d", dg.to_f16_bits(A)), ctx.new("f16_3d", dg.to_f16_bits(B))
+        else:
+            a, bb = ctx.new("u16_3d", dg.to_bf16_bits(A)), ctx.new("u16_3d", dg.to_bf16_bits(B))
+
+        def step():
+            ctx.call(f"bmm_{t}", ["f32_3d"], a, bb).free()
+        w.update(step=step, flops=2 * b * m * m * m, kernel="segmap_matmul", dtype=t, bound="mfma",
+                 keep=[a, bb], describe=f"batched matmul b={b} M=N=K={m}, {t} in, f32 accumulate")
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    return w
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="segscan_add_f32_2p26")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
+                         "(the reference is single-device); run with --gpus 1")
+
+    from futhark_amd import Context
+
+    ctx = Context(profiling=True)
+    ctx.L.futhark_context_pause_profiling(ctx.ptr)
+    w = make_workload(args.workload, ctx)
+    step = w["step"]
+
+    for _ in range(args.warmup):
+        step()
+    ctx.sync()
+
+    # Timed region 1: whole-job throughput, wall clock around K steps.
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    ctx.sync()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    # Timed region 2: the same K steps with a HIP event pair around every kernel
+    # launch, recorded on the context's stream (futhark_context_report).
+    ctx.L.futhark_context_unpause_profiling(ctx.ptr)
+    for _ in range(args.steps):
+        step()
+    ctx.sync()
+    report = json.loads(ctx.report())
+    durs = [e["duration"] for e in report["events"] if e["name"] == w["kernel"]]
+    kernel_us = float(np.mean(durs)) if durs else float("nan")
+
+    if w["bound"] == "hbm":
+        work, unit, peak = w["bytes"], "GB/s", HBM_PEAK_GBS
+        value = work / (ms_per_step * 1e-3) / 1e9
+        achieved = work / (kernel_us * 1e-6) / 1e9
+        metric = "achieved GB/s"
+    else:
+        work, unit, peak = w["flops"], "TFLOP/s", MFMA_PEAK_TFLOPS[w["dtype"]]
+        value = work / (ms_per_step * 1e-3) / 1e12
+        achieved = work / (kernel_us * 1e-6) / 1e12
+        metric = "achieved TFLOP/s"
+
+    cpu = None
+    if not args.no_cpu_baseline and "cpu" in w:
+        import oracle
+        w["cpu"]()  # warm-up
+        reps, t_cpu = 0, 0.0
+        start = time.perf_counter()
+        while t_cpu < args.cpu_seconds and reps < 200:
+            w["cpu"]()
+            reps += 1
+            t_cpu = time.perf_counter() - start
+        cpu = {"value": round(w["bytes"] * reps / t_cpu / 1e9, 3), "unit": "GB/s",
+               "cores": oracle.mc_threads(), "kind": "port",
+               "sample": f"{reps} passes of the full workload with the futhark-multicore-style "
+                         f"restatement in oracle/multicore.c ({t_cpu:.1f} s)"}
+
+    out = {
+        "metric": f"{metric} ({args.workload}), 1xMI355X",
+        "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
+        "config": {"workload": w["describe"], "name": args.workload,
+                   "algorithmic_bytes_per_step" if w["bound"] == "hbm" else "flop_per_step": work},
+        "roofline": {"bound": w["bound"], "achieved": round(achieved, 3), "peak": peak,
+                     "unit": unit, "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel": w["kernel"], "kernel_us": round(kernel_us, 3)},
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    ctx.close()
+
+
+if __name__ == "__main__":
+    main()

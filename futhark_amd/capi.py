@@ -11,7 +11,10 @@ from pathlib import Path
 
 import numpy as np
 
-_LIBDIR = Path(__file__).resolve().parent / "lib"
+import os
+
+# FUTHARK_AMD_LIBDIR points at another directory holding the two libraries.
+_LIBDIR = Path(os.environ.get("FUTHARK_AMD_LIBDIR") or Path(__file__).resolve().parent / "lib")
 
 NUM_TYPES = {"i32": (C.c_int32, np.int32), "i64": (C.c_int64, np.int64),
              "f32": (C.c_float, np.float32), "f64": (C.c_double, np.float64)}

@@ -3,31 +3,38 @@
 // Result-wise this follows the reference's SegRed code generator
 // (src/Futhark/CodeGen/ImpGen/GPU/SegRed.hs): a commutative stage one in which
 // thread t folds elements t, t+T, t+2T, ... (SegRed.hs:802-832), per-block
-// partials, and a stage two run by whichever block finishes last, detected
-// with an atomic counter (SegRed.hs:923-1047).  The schedule is new: 128-bit
-// loads, four loads in flight per thread, a wave64 DPP reduction and a single
-// LDS exchange per block.
+// partials, and a stage two run by one block of the same launch
+// (SegRed.hs:923-1047 picks the block that arrives last with an atomic counter;
+// here the block that starts last waits for the others).  The schedule is new:
+// 128-bit loads, four loads in flight per thread, a wave64 DPP reduction and a
+// single LDS exchange per block.
 #include "common.hip.h"
 
 namespace fa {
 
-// Blocks per launch: enough resident waves on every CU to cover HBM latency
-// without making stage two long.
+// Stage two without fences or a last-arrival counter: every block draws a
+// ticket when it STARTS (off the critical path; same-address device atomics
+// complete at about one per 12 ns on MI355X), publishes its partial as a
+// single 64-bit {value, epoch} word (two words for 8-byte types), and the
+// block holding the last ticket waits for all partials and folds them.  Every
+// other block has started before the finisher drew its ticket and depends on
+// nothing, so the wait terminates.
+constexpr int SEGRED_BLOCK = 256;
+constexpr int SEGRED_UNROLL = 4;
+constexpr int SEGRED_MAX_GRID = 1024;
+constexpr size_t SEGRED_HEADER_BYTES = 256;
+
 static int segred_grid_limit() {
   static int limit = 0;
   if (limit == 0) {
     int dev = 0, cus = NUM_CUS_HINT;
     if (hipGetDevice(&dev) == hipSuccess) {
-      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+      (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
     }
-    limit = cus * 8;
+    limit = cus * 2 > SEGRED_MAX_GRID ? SEGRED_MAX_GRID : cus * 2;
   }
   return limit;
 }
-
-constexpr int SEGRED_BLOCK = 256;
-constexpr int SEGRED_UNROLL = 4;
-constexpr int SEGRED_MAX_GRID = 4096;  // bounds the partials array
 
 template <class T, class Op, int BLOCK>
 __device__ __forceinline__ T block_reduce(T v, T *lds /* BLOCK/64 slots */) {
@@ -42,12 +49,41 @@ __device__ __forceinline__ T block_reduce(T v, T *lds /* BLOCK/64 slots */) {
   return r;
 }
 
+template <class T>
+__device__ __forceinline__ void partial_publish(uint64_t *desc, int slot, uint32_t epoch, T v) {
+  if constexpr (sizeof(T) == 4) {
+    st_relaxed_u64(desc + 2 * slot, ((uint64_t)bit_cast<uint32_t>(v) << 32) | epoch);
+  } else {
+    const uint64_t b = bit_cast<uint64_t>(v);
+    st_relaxed_u64(desc + 2 * slot, ((b & 0xffffffffull) << 32) | epoch);
+    st_relaxed_u64(desc + 2 * slot + 1, ((b >> 32) << 32) | epoch);
+  }
+}
+
+template <class T>
+__device__ __forceinline__ T partial_wait(const uint64_t *desc, int slot, uint32_t epoch) {
+  uint64_t w0;
+  while ((uint32_t)(w0 = ld_relaxed_u64(desc + 2 * slot)) != epoch) __builtin_amdgcn_s_sleep(1);
+  if constexpr (sizeof(T) == 4) {
+    return bit_cast<T>((uint32_t)(w0 >> 32));
+  } else {
+    uint64_t w1;
+    while ((uint32_t)(w1 = ld_relaxed_u64(desc + 2 * slot + 1)) != epoch)
+      __builtin_amdgcn_s_sleep(1);
+    return bit_cast<T>((w0 >> 32) | ((w1 >> 32) << 32));
+  }
+}
+
 template <class T, class Op>
 __global__ __launch_bounds__(SEGRED_BLOCK) void segred_nonseg_kernel(
-    const T *__restrict__ xs, int64_t n, T *__restrict__ out, T *partials, uint32_t *counter) {
+    const T *__restrict__ xs, int64_t n, T *__restrict__ out, uint32_t *ticket, uint64_t *desc,
+    uint32_t epoch) {
   constexpr int VEC = Vec16<T>::N;
   __shared__ T lds[SEGRED_BLOCK / WAVE];
-  __shared__ uint32_t is_last;
+  __shared__ uint32_t s_ticket;
+
+  uint32_t my_ticket = 0;
+  if (gridDim.x > 1 && threadIdx.x == 0) my_ticket = atomicAdd(ticket, 1u);
 
   const int64_t nvec = n / VEC;
   const int64_t stride = (int64_t)gridDim.x * SEGRED_BLOCK;
@@ -60,14 +96,14 @@ __global__ __launch_bounds__(SEGRED_BLOCK) void segred_nonseg_kernel(
   for (; i + (SEGRED_UNROLL - 1) * stride < nvec; i += SEGRED_UNROLL * stride) {
     Vec16<T> v[SEGRED_UNROLL];
 #pragma unroll
-    for (int u = 0; u < SEGRED_UNROLL; u++) v[u] = load_vec16_nt(xs + (i + u * stride) * VEC);
+    for (int u = 0; u < SEGRED_UNROLL; u++) v[u] = load_vec16(xs + (i + u * stride) * VEC);
 #pragma unroll
     for (int u = 0; u < SEGRED_UNROLL; u++)
 #pragma unroll
       for (int e = 0; e < VEC; e++) acc[e] = Op::apply(acc[e], v[u].e[e]);
   }
   for (; i < nvec; i += stride) {
-    Vec16<T> v = load_vec16_nt(xs + i * VEC);
+    Vec16<T> v = load_vec16(xs + i * VEC);
 #pragma unroll
     for (int e = 0; e < VEC; e++) acc[e] = Op::apply(acc[e], v.e[e]);
   }
@@ -89,30 +125,20 @@ __global__ __launch_bounds__(SEGRED_BLOCK) void segred_nonseg_kernel(
   }
 
   if (threadIdx.x == 0) {
-    using U = typename std::conditional<sizeof(T) == 4, uint32_t, uint64_t>::type;
-    __hip_atomic_store(reinterpret_cast<U *>(partials) + blockIdx.x, bit_cast<U>(v),
-                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __threadfence();
-    uint32_t old = atomicAdd(counter, 1u);
-    is_last = (old == gridDim.x - 1) ? 1u : 0u;
+    partial_publish<T>(desc, (int)blockIdx.x, epoch, v);
+    s_ticket = my_ticket;
+    // Last ticket of this launch: rearm the counter for the next one.
+    if (my_ticket == gridDim.x - 1) st_relaxed_u32(ticket, 0u);
   }
   __syncthreads();
-  if (!is_last) return;
-  __threadfence();
+  if (s_ticket != gridDim.x - 1) return;
 
-  // Stage two: this block arrived last, so every partial is visible.
+  // Stage two, in slot order, so the result does not depend on timing.
   T r = Op::identity();
-  for (int p = threadIdx.x; p < (int)gridDim.x; p += SEGRED_BLOCK) {
-    using U = typename std::conditional<sizeof(T) == 4, uint32_t, uint64_t>::type;
-    U bits = __hip_atomic_load(reinterpret_cast<U *>(partials) + p, __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
-    r = Op::apply(r, bit_cast<T>(bits));
-  }
+  for (int p = threadIdx.x; p < (int)gridDim.x; p += SEGRED_BLOCK)
+    r = Op::apply(r, partial_wait<T>(desc, p, epoch));
   r = block_reduce<T, Op, SEGRED_BLOCK>(r, lds);
-  if (threadIdx.x == 0) {
-    *out = r;
-    __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (threadIdx.x == 0) *out = r;
 }
 
 // ------------------------------------------------- regular segments [m][k]
@@ -170,18 +196,17 @@ __global__ __launch_bounds__(1024) void segred_large_kernel(const T *__restrict_
 
 template <class T, class Op>
 static int launch_nonseg(hipStream_t s, const void *xs, int64_t n, void *out, void *scratch,
-                         size_t scratch_bytes) {
+                         size_t scratch_bytes, uint32_t epoch) {
   constexpr int VEC = Vec16<T>::N;
-  if (scratch_bytes < 64 + (size_t)SEGRED_MAX_GRID * sizeof(T)) return FA_ESCRATCH;
+  if (scratch_bytes < SEGRED_HEADER_BYTES + (size_t)SEGRED_MAX_GRID * 16) return FA_ESCRATCH;
   if (!is_aligned(xs, 16) || !is_aligned(scratch, 16)) return FA_EALIGN;
-  int64_t want = ceil_div(n / VEC, (int64_t)SEGRED_BLOCK * SEGRED_UNROLL);
-  int limit = segred_grid_limit();
-  if (limit > SEGRED_MAX_GRID) limit = SEGRED_MAX_GRID;
-  int grid = (int)(want < 1 ? 1 : (want > limit ? limit : want));
-  uint32_t *counter = (uint32_t *)scratch;
-  T *partials = (T *)((char *)scratch + 64);
+  const int64_t want = ceil_div(n / VEC, (int64_t)SEGRED_BLOCK * SEGRED_UNROLL);
+  const int limit = segred_grid_limit();
+  const int grid = (int)(want < 1 ? 1 : (want > limit ? limit : want));
+  uint32_t *ticket = (uint32_t *)scratch;
+  uint64_t *desc = (uint64_t *)((char *)scratch + SEGRED_HEADER_BYTES);
   hipLaunchKernelGGL((segred_nonseg_kernel<T, Op>), dim3(grid), dim3(SEGRED_BLOCK), 0, s,
-                     (const T *)xs, n, (T *)out, partials, counter);
+                     (const T *)xs, n, (T *)out, ticket, desc, epoch);
   return launch_status();
 }
 
@@ -216,17 +241,18 @@ static int launch_regular(hipStream_t s, const void *xss, int64_t m, int64_t k, 
 #include "dispatch.hip.h"
 
 extern "C" size_t fa_segred_scratch_bytes(fa_dtype t) {
-  size_t s = dtype_size(t);
-  if (s < 4) s = 8;
-  return 64 + (size_t)SEGRED_MAX_GRID * s;
+  (void)t;
+  return SEGRED_HEADER_BYTES + (size_t)SEGRED_MAX_GRID * 16;
 }
 
 extern "C" int fa_segred_nonseg(fa_stream_t stream, fa_dtype t, fa_op op, const void *xs,
-                                int64_t n, void *out, void *scratch, size_t scratch_bytes) {
+                                int64_t n, void *out, void *scratch, size_t scratch_bytes,
+                                uint32_t epoch) {
   if (n < 0 || out == nullptr || scratch == nullptr || (n > 0 && xs == nullptr))
     return FA_EINVAL;
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  FA_DISPATCH_TYPE_OP(launch_nonseg, t, op, s, xs, n, out, scratch, scratch_bytes);
+  FA_DISPATCH_TYPE_OP(launch_nonseg, t, op, s, xs, n, out, scratch, scratch_bytes, epoch);
 }
 
 extern "C" int fa_segred_regular(fa_stream_t stream, fa_dtype t, fa_op op, const void *xss,

@@ -20,8 +20,27 @@
 
 namespace fa {
 
-constexpr int SCAN_ROWS = 4;
-constexpr int SCAN_WAVES = 4;
+// Tile shape.  Every tile costs one atomic on the shared ticket counter, and
+// same-address device atomics complete at roughly one per 12 ns on MI355X, so
+// tiles are made large (16 waves x 8 rows x 16 bytes x 64 lanes = 128 KiB of
+// 4-byte elements) to keep the ticket rate far below that limit.
+#ifndef FA_SCAN_ROWS4
+#define FA_SCAN_ROWS4 8 /* 4-byte elements: 32 per thread */
+#endif
+#ifndef FA_SCAN_ROWS8
+#define FA_SCAN_ROWS8 4 /* 8-byte elements: 8 per thread (more spills registers) */
+#endif
+#ifndef FA_SCAN_WAVES
+#define FA_SCAN_WAVES 16
+#endif
+#ifndef FA_SCAN_LOAD
+#define FA_SCAN_LOAD load_vec16_nt
+#endif
+#ifndef FA_SCAN_STORE
+#define FA_SCAN_STORE store_vec16_nt
+#endif
+template <class T> constexpr int scan_rows() { return sizeof(T) == 4 ? FA_SCAN_ROWS4 : FA_SCAN_ROWS8; }
+constexpr int SCAN_WAVES = FA_SCAN_WAVES;
 constexpr int SCAN_BLOCK = SCAN_WAVES * WAVE;
 static_assert(SCAN_WAVES >= 4, "the irregular reduction runs four searches on four waves");
 
@@ -33,7 +52,7 @@ constexpr size_t SCAN_HEADER_BYTES = 256;  // ticket counter, padded
 constexpr size_t SCAN_DESC_BYTES = 16;     // per tile
 
 template <class T> constexpr int scan_tile_elems() {
-  return SCAN_BLOCK * SCAN_ROWS * Vec16<T>::N;
+  return SCAN_BLOCK * scan_rows<T>() * Vec16<T>::N;
 }
 
 __device__ __forceinline__ uint32_t desc_meta(uint32_t epoch, uint32_t flag, uint32_t status) {
@@ -104,6 +123,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
     uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles,
     const int64_t *__restrict__ offsets, const int64_t *__restrict__ lens, int64_t m) {
   constexpr int VEC = Vec16<T>::N;
+  constexpr int SCAN_ROWS = scan_rows<T>();
   constexpr int WCHUNK = SCAN_ROWS * WAVE * VEC;
   constexpr int TILE = SCAN_WAVES * WCHUNK;
   using Pair = SegPair<T>;
@@ -115,7 +135,9 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   __shared__ uint32_t s_pf;
   __shared__ uint32_t s_bits[MODE == MODE_SEGRED ? TILE / 32 : 1];
   __shared__ int64_t s_bounds[4];
-  __shared__ T s_vals[MODE == MODE_SEGRED ? TILE : 1];
+  // MODE_SEGRED keeps the scanned tile in dynamic LDS (TILE elements).
+  extern __shared__ __align__(16) unsigned char s_dyn[];
+  T *s_vals = reinterpret_cast<T *>(s_dyn);
 
   if (threadIdx.x == 0) {
     const uint32_t t = atomicAdd(ticket, 1u);
@@ -142,7 +164,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
     const int64_t idx = wbase + (int64_t)(r * WAVE + lane) * VEC;
     fm[r] = 0u;
     if (idx + VEC <= n) {
-      Vec16<T> v = load_vec16_nt(xs + idx);
+      Vec16<T> v = FA_SCAN_LOAD(xs + idx);
 #pragma unroll
       for (int e = 0; e < VEC; e++) x[r][e] = v.e[e];
       if constexpr (SEG && MODE == MODE_SCAN) {
@@ -338,7 +360,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
     if constexpr (MODE == MODE_SCAN) {
       const int64_t idx = wbase + (int64_t)(r * WAVE + lane) * VEC;
       if (idx + VEC <= n) {
-        store_vec16_nt(out + idx, o);
+        FA_SCAN_STORE(out + idx, o);
       } else {
 #pragma unroll
         for (int e = 0; e < VEC; e++)
@@ -422,9 +444,18 @@ static int launch_segred_irregular(hipStream_t s, const void *vs, int64_t n,
   if (tiles > INT32_MAX) return FA_EINVAL;
   uint32_t *ticket = (uint32_t *)scratch;
   uint64_t *desc = (uint64_t *)((char *)scratch + SCAN_HEADER_BYTES);
-  hipLaunchKernelGGL((segscan_kernel<T, Op, true, false, MODE_SEGRED>), dim3((unsigned)tiles),
-                     dim3(SCAN_BLOCK), 0, s, (const T *)vs, (const uint8_t *)nullptr, n,
-                     (T *)out, ticket, desc, epoch, tiles, offsets, lens, m);
+  auto kernel = segscan_kernel<T, Op, true, false, MODE_SEGRED>;
+  const size_t lds = (size_t)scan_tile_elems<T>() * sizeof(T);
+  static bool lds_limit_raised = false;  // per instantiation
+  if (!lds_limit_raised) {
+    hipError_t e = hipFuncSetAttribute((const void *)kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    lds_limit_raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(SCAN_BLOCK), lds, s, (const T *)vs,
+                     (const uint8_t *)nullptr, n, (T *)out, ticket, desc, epoch, tiles, offsets,
+                     lens, m);
   return launch_status();
 }
 

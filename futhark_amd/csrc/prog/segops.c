@@ -217,7 +217,8 @@ static const fa_op OP_add = FA_ADD, OP_max = FA_MAX, OP_min = FA_MIN;
 static int do_reduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es, void *out,
                      const struct fut_array *in) {
   const int64_t n = in->shape[0];
-  void *scratch = rts_red_scratch(ctx, fa_segred_scratch_bytes(t));
+  uint32_t epoch = 0;
+  void *scratch = rts_scan_scratch(ctx, fa_segred_scratch_bytes(t), &epoch);
   if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
   struct memblock_device res = {0};
   int err = rts_memblock_alloc(ctx, &res, (int64_t)es, "reduce.res");
@@ -226,7 +227,7 @@ static int do_reduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
       ctx, "segred_nonseg", rts_msgprintf("{\"n\":%lld,\"bytes\":%lld}", (long long)n,
                                           (long long)(n * (int64_t)es)));
   int code = fa_segred_nonseg(ctx->stream, t, op, in->mem.mem, n, res.mem, scratch,
-                              ctx->red_scratch_bytes);
+                              ctx->scan_scratch_bytes, epoch);
   err = rts_kernel_end(ctx, ev, "segred_nonseg", code);
   if (err == 0) err = rts_copy_d2h(ctx, out, res.mem, es);
   rts_memblock_unref(ctx, &res, "reduce.res");

@@ -430,26 +430,6 @@ void *rts_scan_scratch(struct futhark_context *ctx, size_t bytes, uint32_t *epoc
   return ctx->scan_scratch;
 }
 
-void *rts_red_scratch(struct futhark_context *ctx, size_t bytes) {
-  if (bytes > ctx->red_scratch_bytes) {
-    size_t want = bytes < (1u << 16) ? (1u << 16) : bytes;
-    if (ctx->red_scratch != NULL) (void)gpu_free_actual(ctx, ctx->red_scratch);
-    ctx->red_scratch = NULL;
-    ctx->red_scratch_bytes = 0;
-    void *mem = NULL;
-    int err = gpu_alloc_actual(ctx, want, &mem);
-    if (err != 0) {
-      if (err == FUTHARK_OUT_OF_MEMORY)
-        rts_set_error(ctx, rts_msgprintf("Failed to allocate %zu bytes of reduction scratch.\n", want));
-      return NULL;
-    }
-    ctx->red_scratch = mem;
-    ctx->red_scratch_bytes = want;
-    if (rts_memset0(ctx, mem, want) != 0) return NULL;
-  }
-  return ctx->red_scratch;
-}
-
 /* -------------------------------------------------------------- profiling */
 
 static void event_list_free(struct futhark_context *ctx) {
@@ -596,7 +576,6 @@ void futhark_context_free(struct futhark_context *ctx) {
   if (ctx->stream != NULL) {
     (void)hipStreamSynchronize((hipStream_t)ctx->stream);
     if (ctx->scan_scratch) (void)hipFree(ctx->scan_scratch);
-    if (ctx->red_scratch) (void)hipFree(ctx->red_scratch);
     (void)rts_gpu_free_all(ctx);
     (void)hipStreamDestroy((hipStream_t)ctx->stream);
   }

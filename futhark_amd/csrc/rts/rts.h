@@ -153,14 +153,12 @@ struct futhark_context {
   /* profiling */
   struct event_list event_list;
 
-  /* look-back / partials scratch owned by the context, grown on demand.
-   * scan_scratch is zero-filled when (re)allocated and then used with a
-   * strictly increasing epoch. */
+  /* look-back / partials scratch owned by the context, grown on demand; it is
+   * zero-filled when (re)allocated and then used with a strictly increasing
+   * epoch, one per kernel launch. */
   void *scan_scratch;
   size_t scan_scratch_bytes;
   uint32_t scan_epoch;
-  void *red_scratch;
-  size_t red_scratch_bytes;
 
   /* deferred error from an asynchronous call, reported at the next sync */
   int pending_error;
@@ -190,9 +188,9 @@ int rts_copy_d2h(struct futhark_context *ctx, void *dst, const void *src, size_t
 int rts_copy_d2d(struct futhark_context *ctx, void *dst, const void *src, size_t bytes);
 int rts_memset0(struct futhark_context *ctx, void *dst, size_t bytes);
 
-/* scratch for scans and reductions; NULL on failure (error set). */
+/* look-back scratch for scans and reductions with a fresh epoch for one launch;
+ * NULL on failure (error set). */
 void *rts_scan_scratch(struct futhark_context *ctx, size_t bytes, uint32_t *epoch_out);
-void *rts_red_scratch(struct futhark_context *ctx, size_t bytes);
 
 /* Profiling bracket around one kernel-library call.  `desc` is JSON object
  * text or NULL.  rts_kernel_end turns a nonzero launcher code into an error. */

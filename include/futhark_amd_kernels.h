@@ -67,12 +67,13 @@ int fa_version(void);
  * Non-segmented reduction `reduce op ne xs`.
  * Replaces: segred_nonseg (SegRed.hs:327-394): stage one, per-block partials,
  * last-block-finishes stage two with an atomic counter (SegRed.hs:923-1047).
- * out: one element.  scratch: fa_segred_scratch_bytes(); its first 64 bytes
- * must be zero before the first use and are left zero by every call. */
+ * out: one element.  scratch: at least fa_segred_scratch_bytes(), under the
+ * zero-once / increasing-epoch protocol described at fa_segscan (the same
+ * buffer may serve both). */
 size_t fa_segred_scratch_bytes(fa_dtype t);
 int fa_segred_nonseg(fa_stream_t stream, fa_dtype t, fa_op op,
                      const void *xs, int64_t n, void *out,
-                     void *scratch, size_t scratch_bytes);
+                     void *scratch, size_t scratch_bytes, uint32_t epoch);
 
 /* Regular segmented reduction `map (reduce op ne) xss`, xss : [m][k] row-major.
  * Replaces: segred_small / segred_large (SegRed.hs:396-636).  No scratch. */
