@@ -1,0 +1,279 @@
+// SegHist for gfx950: reduce_by_index with LDS-privatised sub-histograms.
+//
+// What is computed follows src/Futhark/CodeGen/ImpGen/GPU/SegHist.hs: for every
+// element whose bin lies in [0,H) the destination bin is combined with the value
+// (out-of-range bins are skipped, SegHist.hs:450-458,750-755); each block keeps
+// sub-histograms in LDS, spreads threads over several copies of a bin to cut
+// contention (SegHist.hs:654-656) and the copies are combined into the
+// destination at the end (SegHist.hs:770-828,1137-1186).
+//
+// Measured on MI355X: device-scope atomics on HBM complete at about 27 G/s for
+// scattered addresses and collapse under contention, while LDS atomics keep up
+// with the HBM input stream.  So every element update is an LDS atomic:
+//   * one block of 1024 threads per CU holds a bin range of up to 128 KiB in LDS
+//     (up to 32768 four-byte bins);
+//   * small ranges are replicated C times, copy index = lane mod C, laid out
+//     bin-major ([bin][copy]) so the lanes of a wave hit distinct banks;
+//   * H larger than one range is covered by P ranges in ONE launch: P blocks
+//     that sit on the same XCD read the same input chunk at about the same time
+//     (the second read is an L2 hit) and each keeps the updates of its range;
+//   * blocks flush with coalesced device-scope atomics, skipping neutral bins.
+// H beyond the multi-range limit goes to a partition pass (bins split into
+// LDS-sized ranges by a stable ranked scatter) followed by the same LDS kernel
+// per partition.
+#include "dispatch.hip.h"
+
+namespace fa {
+
+constexpr int HIST_BLOCK = 1024;
+constexpr int HIST_LDS_BYTES = 128 * 1024;  // bin storage per block
+constexpr int HIST_MAX_RANGES = 4;          // ranges covered by one launch
+constexpr int NUM_XCDS = 8;
+
+// ------------------------------------------------------------ atomic updates
+// `Scope` is __HIP_MEMORY_SCOPE_WORKGROUP for LDS and _AGENT for HBM.
+
+template <class T> struct SameSizeInt;
+template <> struct SameSizeInt<float> { using S = int32_t; using U = uint32_t; };
+template <> struct SameSizeInt<double> { using S = int64_t; using U = uint64_t; };
+
+template <class T, class Op, int Scope> struct AtomicUpdate;
+
+template <class T, int Scope> struct AtomicUpdate<T, OpAdd<T>, Scope> {
+  static __device__ __forceinline__ void apply(T *p, T v) {
+    if constexpr (std::is_integral<T>::value) {
+      using U = typename std::make_unsigned<T>::type;
+      __hip_atomic_fetch_add(reinterpret_cast<U *>(p), (U)v, __ATOMIC_RELAXED, Scope);
+    } else {
+      __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, Scope);
+    }
+  }
+};
+
+// Float max/min through the integer view: non-negative floats order like signed
+// integers, negative floats order inversely like unsigned integers.  NaN inputs
+// are dropped (fmax(x, NaN) = x).  Valid while the cell itself is not NaN.
+template <class T, int Scope, bool IS_MAX>
+__device__ __forceinline__ void float_minmax_update(T *p, T v) {
+  using S = typename SameSizeInt<T>::S;
+  using U = typename SameSizeInt<T>::U;
+  if (v != v) return;
+  const S bits = bit_cast<S>(v);
+  if (IS_MAX) {
+    if (bits >= 0) __hip_atomic_fetch_max(reinterpret_cast<S *>(p), bits, __ATOMIC_RELAXED, Scope);
+    else __hip_atomic_fetch_min(reinterpret_cast<U *>(p), (U)bits, __ATOMIC_RELAXED, Scope);
+  } else {
+    if (bits >= 0) __hip_atomic_fetch_min(reinterpret_cast<S *>(p), bits, __ATOMIC_RELAXED, Scope);
+    else __hip_atomic_fetch_max(reinterpret_cast<U *>(p), (U)bits, __ATOMIC_RELAXED, Scope);
+  }
+}
+
+template <class T, int Scope> struct AtomicUpdate<T, OpMax<T>, Scope> {
+  static __device__ __forceinline__ void apply(T *p, T v) {
+    if constexpr (std::is_integral<T>::value) __hip_atomic_fetch_max(p, v, __ATOMIC_RELAXED, Scope);
+    else float_minmax_update<T, Scope, true>(p, v);
+  }
+};
+template <class T, int Scope> struct AtomicUpdate<T, OpMin<T>, Scope> {
+  static __device__ __forceinline__ void apply(T *p, T v) {
+    if constexpr (std::is_integral<T>::value) __hip_atomic_fetch_min(p, v, __ATOMIC_RELAXED, Scope);
+    else float_minmax_update<T, Scope, false>(p, v);
+  }
+};
+
+// Update of a destination cell in HBM.  Float max/min use a compare-and-swap
+// loop on the operator itself, so that a NaN already in `dest` is replaced the
+// way fmax/fmin replace it (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:844-905).
+template <class T, class Op>
+__device__ __forceinline__ void global_update(T *p, T v) {
+  constexpr bool float_minmax = !std::is_integral<T>::value && !std::is_same<Op, OpAdd<T>>::value;
+  if constexpr (float_minmax) {
+    using U = typename SameSizeInt<T>::U;
+    U *q = reinterpret_cast<U *>(p);
+    U old = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    while (true) {
+      const T want = Op::apply(bit_cast<T>(old), v);
+      const U wbits = bit_cast<U>(want);
+      if (wbits == old) break;
+      if (__hip_atomic_compare_exchange_strong(q, &old, wbits, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT))
+        break;
+    }
+  } else {
+    AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_AGENT>::apply(p, v);
+  }
+}
+
+template <class T> __device__ __forceinline__ bool bits_equal(T a, T b) {
+  if constexpr (sizeof(T) == 4) return bit_cast<uint32_t>(a) == bit_cast<uint32_t>(b);
+  else return bit_cast<uint64_t>(a) == bit_cast<uint64_t>(b);
+}
+
+// Four consecutive elements with 16-byte loads (pointers are 16-byte aligned).
+template <class E> __device__ __forceinline__ void load_elems4(E (&dst)[4], const E *src) {
+  constexpr int NV = (int)(4 * sizeof(E) / 16);
+  uint4 raw[NV];
+#pragma unroll
+  for (int q = 0; q < NV; q++) raw[q] = reinterpret_cast<const uint4 *>(src)[q];
+  __builtin_memcpy(dst, raw, sizeof(raw));
+}
+
+// ------------------------------------------------------------- LDS histogram
+// Grid layout: block b sits on XCD b % 8.  j = b / 8; range p = j % P;
+// chunk set s = (j / P) * 8 + b % 8 of S = gridDim.x / P sets.  The P blocks of
+// one chunk set read the same elements, each keeping the bins of its range.
+template <class T, class Op, class I>
+__global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
+    const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t bin_base,
+    int64_t H, int range_bins, int P, int log2_copies) {
+  extern __shared__ __align__(16) unsigned char s_raw[];
+  T *sh = reinterpret_cast<T *>(s_raw);
+  constexpr int VEC = 4;  // elements per thread per step
+
+  const int b = blockIdx.x;
+  const int j = b / NUM_XCDS;
+  const int p = j % P;
+  const int64_t S = gridDim.x / P;
+  const int64_t s = (int64_t)(j / P) * NUM_XCDS + b % NUM_XCDS;
+  const int64_t lo = bin_base + (int64_t)p * range_bins;
+  int64_t hi = lo + range_bins;
+  if (hi > bin_base + H) hi = bin_base + H;
+  const int nb = (int)(hi > lo ? hi - lo : 0);
+  const int C = 1 << log2_copies;
+  const int cells = nb * C;
+
+  for (int i = threadIdx.x; i < cells; i += HIST_BLOCK) sh[i] = Op::identity();
+  __syncthreads();
+
+  const int copy = threadIdx.x & (C - 1);
+  const int64_t nvec = n / VEC;
+  const int64_t stride = S * HIST_BLOCK;
+  auto update = [&](int64_t bin, T v) {
+    const int64_t r = bin - lo;
+    if ((uint64_t)r < (uint64_t)nb)
+      AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(&sh[((int)r << log2_copies) + copy], v);
+  };
+  if (nb > 0) {
+    for (int64_t i = s * HIST_BLOCK + threadIdx.x; i < nvec; i += stride) {
+      I bi[VEC];
+      T bv[VEC];
+      load_elems4(bi, is + i * VEC);
+      load_elems4(bv, vs + i * VEC);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
+    }
+    if (s == 0) {
+      const int64_t t = nvec * VEC + threadIdx.x;
+      if (threadIdx.x < VEC && t < n) update((int64_t)is[t], vs[t]);
+    }
+  }
+  __syncthreads();
+
+  // Flush: combine the copies of a bin in copy order, skip untouched bins.
+  for (int r = threadIdx.x; r < nb; r += HIST_BLOCK) {
+    T acc = sh[r << log2_copies];
+    for (int c = 1; c < C; c++) acc = Op::apply(acc, sh[(r << log2_copies) + c]);
+    if (!bits_equal(acc, Op::identity())) global_update<T, Op>(dest + (lo - bin_base) + r, acc);
+  }
+}
+
+// Fallback for very large H until the partitioned path takes over: one
+// device-scope atomic per element.
+template <class T, class Op, class I>
+__global__ __launch_bounds__(256) void seghist_global_kernel(const I *__restrict__ is,
+                                                             const T *__restrict__ vs, int64_t n,
+                                                             T *dest, int64_t H) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const int64_t bin = (int64_t)is[i];
+    if ((uint64_t)bin < (uint64_t)H) global_update<T, Op>(dest + bin, vs[i]);
+  }
+}
+
+static int hist_num_cus() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    cus = NUM_CUS_HINT;
+    if (hipGetDevice(&dev) == hipSuccess)
+      (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  }
+  return cus;
+}
+
+// Launches the LDS kernel over bins [0,H) of `dest` (H <= max ranges * range size).
+template <class T, class Op, class I>
+static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
+                           int64_t H) {
+  const int max_range = HIST_LDS_BYTES / (int)sizeof(T);
+  const int P = (int)ceil_div(H, max_range);
+  const int range_bins = (int)ceil_div(H, P);
+  int log2_copies = 0;
+  while (log2_copies < 5 && (int64_t)range_bins * (2 << log2_copies) * (int64_t)sizeof(T) <= 32 * 1024)
+    log2_copies++;
+  const size_t lds = (size_t)range_bins * sizeof(T) << log2_copies;
+  // One block per CU when the range fills LDS, two when two fit.
+  const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
+  int grid = hist_num_cus() * per_cu;
+  grid -= grid % (NUM_XCDS * P);
+  if (grid < NUM_XCDS * P) grid = NUM_XCDS * P;
+  auto kernel = seghist_lds_kernel<T, Op, I>;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void *)kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
+    if (e != hipSuccess) return (int)e;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(HIST_BLOCK), lds, st, is, vs, n, dest, (int64_t)0,
+                     H, range_bins, P, log2_copies);
+  return launch_status();
+}
+
+template <class T, class Op>
+static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs, int64_t n,
+                       void *dest, int64_t H, void *scratch, size_t scratch_bytes) {
+  (void)scratch;
+  (void)scratch_bytes;
+  if (H == 0 || n == 0) return 0;
+  if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
+  const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)sizeof(T));
+  if (H <= lds_limit) {
+    if (is64) return launch_lds_hist<T, Op, int64_t>(st, (const int64_t *)is, (const T *)vs, n, (T *)dest, H);
+    return launch_lds_hist<T, Op, int32_t>(st, (const int32_t *)is, (const T *)vs, n, (T *)dest, H);
+  }
+  const int grid = hist_num_cus() * 8;
+  if (is64)
+    hipLaunchKernelGGL((seghist_global_kernel<T, Op, int64_t>), dim3(grid), dim3(256), 0, st,
+                       (const int64_t *)is, (const T *)vs, n, (T *)dest, H);
+  else
+    hipLaunchKernelGGL((seghist_global_kernel<T, Op, int32_t>), dim3(grid), dim3(256), 0, st,
+                       (const int32_t *)is, (const T *)vs, n, (T *)dest, H);
+  return launch_status();
+}
+
+}  // namespace fa
+
+extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int64_t H) {
+  (void)t;
+  (void)H;
+  return 256;
+}
+
+extern "C" int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op, const void *is, int is64,
+                          const void *vs, int64_t n, void *dest, int64_t H, void *scratch,
+                          size_t scratch_bytes) {
+  if (n < 0 || H < 0 || (H > 0 && dest == nullptr) || (n > 0 && (is == nullptr || vs == nullptr)))
+    return FA_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (t) {
+    case FA_I32:
+    case FA_I64:
+    case FA_F32:
+    case FA_F64:
+      break;
+    default:
+      return FA_ENOTSUP;
+  }
+  FA_DISPATCH_TYPE_OP(launch_hist, t, op, s, is, is64, vs, n, dest, H, scratch, scratch_bytes);
+}

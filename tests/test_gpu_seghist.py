@@ -1,0 +1,113 @@
+"""GPU parity: SegHist (hist / reduce_by_index) through the generated-library
+API against the CPU oracle.  Integer operators and float max/min bit-exact;
+f32 add within 1e-5 relative of the f64-accumulated oracle (atomic order is
+not fixed)."""
+import numpy as np
+import pytest
+
+import oracle
+from futhark_amd import datagen as dg
+
+pytestmark = pytest.mark.gpu
+NP = {"i32": np.int32, "i64": np.int64, "f32": np.float32, "f64": np.float64}
+
+
+def _vals(t, n, aid):
+    if t in ("i32", "i64"):
+        return dg.uniform_int(aid, n, -1000, 1000, NP[t])
+    return (dg.uniform_f32(aid, n) - np.float32(0.25)).astype(NP[t])  # mixed signs
+
+
+def _check(t, op, got, want_lit, want_acc=None):
+    if op == "add" and t in ("f32", "f64"):
+        ref = want_acc if want_acc is not None else want_lit
+        err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+        assert np.all(err <= 1e-5 * np.abs(ref) + 1e-6), float(err.max())
+    else:
+        assert np.array_equal(got, want_lit)
+
+
+@pytest.mark.parametrize("t", ["i32", "i64", "f32", "f64"])
+@pytest.mark.parametrize("op", ["add", "max", "min"])
+def test_hist_small_and_ragged(ctx, t, op):
+    for n, H in [(0, 5), (5, 0), (1, 1), (100, 7), (4097, 256), (100003, 1000), (300001, 32768),
+                 (300001, 32769), (200000, 65536), (150000, 100001), (100000, 200000)]:
+        is_ = dg.hist_indices(40, n, max(H, 1), "uniform", 3)
+        vs = _vals(t, n, 41)
+        i, v = ctx.new("i32_1d", is_), ctx.new(f"{t}_1d", vs)
+        out = ctx.call(f"hist_{op}_{t}", [f"{t}_1d"], H, i, v)
+        got = out.values()
+        assert got.shape == (H,)
+        acc = oracle.hist(op, t, H, is_, vs, "f64acc") if (op, t) == ("add", "f32") else None
+        _check(t, op, got, oracle.hist(op, t, H, is_, vs), acc)
+        for h in (i, v, out):
+            h.free()
+
+
+def test_reference_goldens(ctx, goldens):
+    for c in goldens["hist_simple"]["cases"]:
+        img = np.array(c["image"], np.int32)
+        d, i = ctx.new("i32_1d", np.array(c["dest"], np.int32)), ctx.new("i32_1d", img)
+        out = ctx.call("rbi_add_i32", ["i32_1d"], d, i, i)
+        assert out.values().tolist() == c["out"]
+        assert d.values().tolist() == c["dest"]  # the input is not consumed
+    for c in goldens["hist_large"]["cases"]:
+        n, m = c["n"], c["m"]
+        k = np.arange(m, dtype=np.int64)
+        out = ctx.call("hist_add_i32", ["i32_1d"], n, ctx.new("i32_1d", (k % n).astype(np.int32)),
+                       ctx.new("i32_1d", k.astype(np.int32)))
+        assert int(ctx.call("reduce_add_i32", [np.int32], out)) == c["out"]
+        out.free()
+    f = lambda xs: np.array([np.nan if x == "nan" else x for x in xs], np.float32)
+    for c in goldens["hist_f32"]["cases"]:
+        out = ctx.call("rbi_add_f32", ["f32_1d"], ctx.new("f32_1d", f(c["dest"])),
+                       ctx.new("i32_1d", np.array(c["is"], np.int32)), ctx.new("f32_1d", f(c["vs"])))
+        np.testing.assert_allclose(out.values(), f(c["out"]), rtol=2e-3, equal_nan=True)
+    for name, op in (("hist_max", "max"), ("hist_min", "min")):
+        for c in goldens[name]["cases"]:
+            out = ctx.call(f"rbi_{op}_i32", ["i32_1d"], ctx.new("i32_1d", np.zeros(c["n"], np.int32)),
+                           ctx.new("i32_1d", np.array(c["is"], np.int32)),
+                           ctx.new("i32_1d", np.array(c["vs"], np.int32)))
+            assert out.values().tolist() == c["out"]
+
+
+def test_float_max_with_nan_and_negative_values(ctx):
+    dest = np.array([np.nan, -np.inf, 2.0, -3.0, 0.0, -0.5], np.float32)
+    is_ = np.array([0, 0, 1, 1, 2, 3, 3, 4, 5, 5, 9, -1], np.int32)
+    vs = np.array([-7.0, -9.0, np.nan, -4.0, 1.0, -2.0, -2.5, -1.0, np.nan, -0.25, 5.0, 5.0], np.float32)
+    for op in ("max", "min"):
+        out = ctx.call(f"rbi_{op}_f32", ["f32_1d"], ctx.new("f32_1d", dest), ctx.new("i32_1d", is_),
+                       ctx.new("f32_1d", vs))
+        want = oracle.rbi(op, "f32", dest, is_, vs)
+        assert np.array_equal(out.values(), want, equal_nan=True), (op, out.values(), want)
+
+
+@pytest.mark.parametrize("H", [256, 65536, 1 << 22])
+@pytest.mark.parametrize("dist", ["uniform", "zipf"])
+def test_config3_full_size_i32(ctx, H, dist):
+    n = 1 << 27
+    is_ = dg.hist_indices(48, n, H, dist)
+    vs = dg.uniform_int(49, n, -1000, 1000)
+    i, v = ctx.new("i32_1d", is_), ctx.new("i32_1d", vs)
+    out = ctx.call("hist_add_i32", ["i32_1d"], H, i, v)
+    got = out.values()
+    assert np.array_equal(got, oracle.hist("add", "i32", H, is_, vs))
+    # size-independent property: the total equals the sum of the in-range values
+    ok = (is_ >= 0) & (is_ < H)
+    assert int(got.astype(np.int64).sum()) == int(vs[ok].astype(np.int64).sum())
+    for h in (i, v, out):
+        h.free()
+
+
+@pytest.mark.parametrize("H", [256, 65536])
+def test_config3_full_size_f32(ctx, H):
+    n = 1 << 27
+    is_ = dg.hist_indices(48, n, H, "uniform")
+    ws = dg.uniform_f32(50, n)
+    i, w = ctx.new("i32_1d", is_), ctx.new("f32_1d", ws)
+    out = ctx.call("hist_max_f32", ["f32_1d"], H, i, w)
+    assert np.array_equal(out.values(), oracle.hist("max", "f32", H, is_, ws))
+    out.free()
+    out = ctx.call("hist_add_f32", ["f32_1d"], H, i, w)
+    got, ref = out.values(), oracle.hist("add", "f32", H, is_, ws, "f64acc")
+    assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(ref))
