@@ -1,0 +1,89 @@
+"""GPU parity: tiled SegMap (batched matmul) through the generated-library API.
+
+Tolerance: |got - ref| <= tol * sum_k |a_ik||b_kj| per output, ref accumulated in
+f64; tol = 1e-5 for f32 inputs and 1e-2 for f16/bf16 inputs (f32 accumulate).
+The bound is relative to the magnitude of the summands because a dot product
+of zero-mean data can be arbitrarily close to zero."""
+import numpy as np
+import pytest
+
+import oracle
+from futhark_amd import datagen as dg
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(t, b, M, N, K, aid=60):
+    sc = 1.0 / np.sqrt(max(K, 1))
+    A = dg.normal_f32(aid, b * M * K, sc).reshape(b, M, K)
+    B = dg.normal_f32(aid + 1, b * K * N, sc).reshape(b, K, N)
+    if t == "f32":
+        return A, B, A, B, "f32_3d"
+    if t == "f16":
+        Ab, Bb = dg.to_f16_bits(A), dg.to_f16_bits(B)
+        return Ab, Bb, oracle.widen(Ab, "f16"), oracle.widen(Bb, "f16"), "f16_3d"
+    Ab, Bb = dg.to_bf16_bits(A), dg.to_bf16_bits(B)
+    return Ab, Bb, oracle.widen(Ab, "bf16"), oracle.widen(Bb, "bf16"), "u16_3d"
+
+
+def _check(got, Af, Bf, tol):
+    ref = np.matmul(Af.astype(np.float64), Bf.astype(np.float64))
+    scale = np.matmul(np.abs(Af).astype(np.float64), np.abs(Bf).astype(np.float64))
+    err = np.abs(got.astype(np.float64) - ref)
+    assert np.all(err <= tol * scale + 1e-30), float((err / (scale + 1e-30)).max())
+
+
+@pytest.mark.parametrize("t,tol", [("f32", 1e-5), ("f16", 1e-2), ("bf16", 1e-2)])
+def test_shapes(ctx, t, tol):
+    for b, M, N, K in [(1, 2, 2, 3), (3, 17, 29, 13), (2, 64, 64, 64), (1, 100, 70, 130),
+                       (1, 256, 256, 32), (1, 256, 256, 64), (2, 256, 512, 96), (1, 512, 256, 512),
+                       (1, 5, 7, 0), (0, 4, 4, 4)]:
+        Ain, Bin, Af, Bf, kind = _inputs(t, b, M, N, K)
+        out = ctx.call(f"bmm_{t}", ["f32_3d"], ctx.new(kind, Ain), ctx.new(kind, Bin))
+        got = out.values()
+        assert got.shape == (b, M, N)
+        _check(got, Af, Bf, tol)
+
+
+def test_reference_golden(ctx, goldens):
+    c = goldens["mmm"]["cases"][0]
+    out = ctx.call("matmul_f32", ["f32_2d"], ctx.new("f32_2d", np.array(c["A"], np.float32)),
+                   ctx.new("f32_2d", np.array(c["B"], np.float32)))
+    assert out.values().tolist() == c["out"]
+
+
+def test_structured_operands_catch_transposition(ctx):
+    # A = row index, B = one-hot columns: any swap of operands or indices shows.
+    M = N = 256
+    K = 64
+    A = (np.arange(M)[:, None] * 0.5 + np.arange(K)[None, :] * 0.125).astype(np.float32)
+    B = np.zeros((K, N), np.float32)
+    B[np.arange(N) % K, np.arange(N)] = 1.0
+    B[(np.arange(N) * 7 + 3) % K, np.arange(N)] += 2.0
+    want = A.astype(np.float64) @ B.astype(np.float64)
+    for t, kind in (("f32", "f32_3d"), ("f16", "f16_3d"), ("bf16", "u16_3d")):
+        cvt = {"f32": lambda x: x, "f16": dg.to_f16_bits, "bf16": dg.to_bf16_bits}[t]
+        out = ctx.call(f"bmm_{t}", ["f32_3d"], ctx.new(kind, cvt(A)[None]), ctx.new(kind, cvt(B)[None]))
+        got = out.values()[0]
+        if t == "bf16":  # A is not exactly representable in bf16
+            Aw = oracle.widen(dg.to_bf16_bits(A), "bf16").astype(np.float64)
+            np.testing.assert_allclose(got, Aw @ B.astype(np.float64), rtol=1e-6)
+        else:
+            np.testing.assert_allclose(got, want, rtol=1e-6)
+
+
+@pytest.mark.parametrize("t,tol", [("f32", 1e-5), ("f16", 1e-2), ("bf16", 1e-2)])
+@pytest.mark.parametrize("b,m", [(1, 4096), (64, 512)])
+def test_config4_full_size(ctx, t, tol, b, m):
+    Ain, Bin, Af, Bf, kind = _inputs(t, b, m, m, m, 64)
+    out = ctx.call(f"bmm_{t}", ["f32_3d"], ctx.new(kind, Ain), ctx.new(kind, Bin))
+    got = out.values()
+    # full oracle on a sample of rows (the CPU triple loop over 4096^3 takes minutes)
+    rows = np.array([0, 1, 31, 32, 127, 128, 255, 256, m // 2 + 3, m - 1])
+    for q in (0, b - 1):
+        _check(got[q][rows], Af[q][rows], Bf[q], tol)
+    # size-independent property: linearity in the row sums, C 1 = A (B 1)
+    lhs = got.astype(np.float64).sum(axis=2)
+    rhs = np.matmul(Af.astype(np.float64), Bf.astype(np.float64).sum(axis=2)[..., None])[..., 0]
+    scale = np.matmul(np.abs(Af).astype(np.float64), np.abs(Bf).astype(np.float64).sum(axis=2)[..., None])[..., 0]
+    assert np.all(np.abs(lhs - rhs) <= tol * scale)
