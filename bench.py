@@ -151,6 +151,10 @@ def main() -> None:
     ap.add_argument("--workload", default="segscan_add_f32_2p26")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run the plain copy kernel (fa_copy, 256 MiB) a few times, so "
+                         "that a rocprofv3 --pmc run of this command holds a dispatch of known "
+                         "traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -210,6 +214,18 @@ def main() -> None:
                "cores": oracle.mc_threads(), "kind": "port",
                "sample": f"{reps} passes of the full workload with the futhark-multicore-style "
                          f"restatement in oracle/multicore.c ({t_cpu:.1f} s)"}
+
+    if args.calibrate_copy:
+        import ctypes as C
+        from futhark_amd import lib_path
+        k = C.CDLL(str(lib_path("libfuthark_amd_kernels.so")))
+        k.fa_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]
+        nbytes = 256 << 20
+        src = ctx.new("u8_1d", np.zeros(nbytes, np.uint8))
+        dst = ctx.new("u8_1d", np.zeros(nbytes, np.uint8))
+        for _ in range(5):
+            assert k.fa_copy(ctx.stream, dst.device_ptr, src.device_ptr, nbytes) == 0
+        ctx.sync()
 
     out = {
         "metric": f"{metric} ({args.workload}), 1xMI355X",

@@ -237,8 +237,8 @@ float orc_bf16_to_f32(uint16_t h) {
   memcpy(&f, &bits, 4);
   return f;
 }
-/* 16-bit inputs widened to f32, then the f32 matmul (Appendix programs bmm_f16/bmm_bf16:
- * f32.f16 x * f32.f16 y summed in f32). */
+/* 16-bit inputs widened to f32, then the f32 matmul: products f32.f16 x * f32.f16 y
+ * summed in f32 (for bf16 the widening is bits << 16). */
 void orc_widen_f16(const uint16_t *in, float *out, int64_t n) {
   for (int64_t i = 0; i < n; i++) out[i] = orc_f16_to_f32(in[i]);
 }
