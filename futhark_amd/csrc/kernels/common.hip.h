@@ -244,7 +244,7 @@ __device__ __forceinline__ void st_relaxed_u32(uint32_t *p, uint32_t v) {
 
 static inline bool is_aligned(const void *p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
-static inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+static inline __host__ __device__ int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 // Launch check: returns the positive hipError_t value on failure.
 static inline int launch_status() {

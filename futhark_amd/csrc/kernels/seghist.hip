@@ -18,10 +18,12 @@
 //     that sit on the same XCD read the same input chunk at about the same time
 //     (the second read is an L2 hit) and each keeps the updates of its range;
 //   * blocks flush with coalesced device-scope atomics, skipping neutral bins.
-// H beyond the multi-range limit goes to a partition pass (bins split into
-// LDS-sized ranges by a stable ranked scatter) followed by the same LDS kernel
-// per partition.
-#include "dispatch.hip.h"
+// H beyond the multi-range limit (up to 255 ranges) first partitions the
+// (index, value) pairs by bin range with one pass of the radix kernels (a
+// stable ranked scatter, radix.hip.h), then runs LDS histograms over the
+// partitions; out-of-range indices land in a partition that is never read.
+// Only H beyond 255 ranges falls back to one device atomic per element.
+#include "radix.hip.h"
 
 namespace fa {
 
@@ -177,8 +179,68 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
   }
 }
 
-// Fallback for very large H until the partitioned path takes over: one
-// device-scope atomic per element.
+// ------------------------------------------------- partitioned large histograms
+// Digit of a pair = index of the LDS-sized bin range its bin falls in; 255 for
+// bins outside [0,H).
+template <class U> struct DigitBinRange {
+  uint64_t H;
+  int shift;
+  __device__ __forceinline__ uint32_t operator()(U key, int) const {
+    return (uint64_t)key < H ? (uint32_t)((uint64_t)key >> shift) : 255u;
+  }
+};
+
+// Input: pairs grouped by bin range (range r occupies [gbase[r], gbase[r+1])).
+// Each block takes a contiguous chunk of the valid pairs and, for every range
+// the chunk touches, accumulates in LDS and flushes.
+template <class T, class Op, class U>
+__global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
+    const U *__restrict__ pis, const T *__restrict__ pvs, const uint32_t *__restrict__ gbase,
+    T *dest, int64_t H, int shift) {
+  extern __shared__ __align__(16) unsigned char s_raw[];
+  T *sh = reinterpret_cast<T *>(s_raw);
+  __shared__ uint32_t s_start[RS_RADIX];
+  if (threadIdx.x < RS_RADIX) s_start[threadIdx.x] = gbase[threadIdx.x];
+  __syncthreads();
+  const int64_t n_valid = s_start[RS_RADIX - 1];
+  const int64_t chunk = ceil_div(ceil_div(n_valid, (int64_t)gridDim.x), 4) * 4;
+  const int64_t c0 = (int64_t)blockIdx.x * chunk;
+  const int64_t c1 = c0 + chunk < n_valid ? c0 + chunk : n_valid;
+  const int range_bins = 1 << shift;
+  const int num_ranges = (int)((H + range_bins - 1) >> shift);
+  for (int r = 0; r < num_ranges && c0 < c1; r++) {
+    const int64_t r0 = s_start[r], r1 = s_start[r + 1];
+    const int64_t lo = r0 > c0 ? r0 : c0, hi = r1 < c1 ? r1 : c1;
+    if (lo >= hi) continue;  // uniform over the block
+    const int64_t bin0 = (int64_t)r << shift;
+    const int nb = (int)((H - bin0) < range_bins ? (H - bin0) : range_bins);
+    for (int i = threadIdx.x; i < nb; i += HIST_BLOCK) sh[i] = Op::identity();
+    __syncthreads();
+    int64_t i = lo + threadIdx.x;
+    for (; i + 3 * HIST_BLOCK < hi; i += 4 * HIST_BLOCK) {
+      U b[4];
+      T v[4];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        b[q] = pis[i + q * HIST_BLOCK];
+        v[q] = pvs[i + q * HIST_BLOCK];
+      }
+#pragma unroll
+      for (int q = 0; q < 4; q++)
+        AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(&sh[(int)((int64_t)b[q] - bin0)], v[q]);
+    }
+    for (; i < hi; i += HIST_BLOCK)
+      AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(&sh[(int)((int64_t)pis[i] - bin0)], pvs[i]);
+    __syncthreads();
+    for (int q = threadIdx.x; q < nb; q += HIST_BLOCK) {
+      const T acc = sh[q];
+      if (!bits_equal(acc, Op::identity())) global_update<T, Op>(dest + bin0 + q, acc);
+    }
+    __syncthreads();
+  }
+}
+
+// Last resort (more than 255 bin ranges): one device-scope atomic per element.
 template <class T, class Op, class I>
 __global__ __launch_bounds__(256) void seghist_global_kernel(const I *__restrict__ is,
                                                              const T *__restrict__ vs, int64_t n,
@@ -230,17 +292,59 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
   return launch_status();
 }
 
+template <class T> constexpr int hist_part_shift() {
+  return sizeof(T) == 4 ? 15 : 14;  // 128 KiB of bins per range
+}
+
+static size_t hist_align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+template <class T, class Op, class U>
+static int launch_part_hist(hipStream_t st, const U *is, const T *vs, int64_t n, T *dest,
+                            int64_t H, void *scratch, size_t scratch_bytes) {
+  constexpr int shift = hist_part_shift<T>();
+  const int64_t tiles = rs_num_tiles(n);
+  const size_t rs_bytes = hist_align(rs_scratch_bytes(tiles, 1));
+  const size_t is_bytes = hist_align((size_t)n * sizeof(U));
+  if (scratch_bytes < rs_bytes + is_bytes + (size_t)n * sizeof(T)) return FA_ESCRATCH;
+  if (!is_aligned(scratch, 256)) return FA_EALIGN;
+  U *pis = (U *)((char *)scratch + rs_bytes);
+  T *pvs = (T *)((char *)scratch + rs_bytes + is_bytes);
+  RsScratch sc = rs_carve(scratch, tiles, 1);
+  DigitBinRange<U> fn{(uint64_t)H, shift};
+  int rc = rs_prepare<U>(st, is, n, fn, 1, sc);
+  if (rc != 0) return rc;
+  rc = rs_pass<U, (int)sizeof(T)>(st, is, pis, vs, pvs, n, fn, 0, sc);
+  if (rc != 0) return rc;
+  auto kernel = seghist_part_kernel<T, Op, U>;
+  static bool raised = false;
+  if (!raised) {
+    hipError_t e = hipFuncSetAttribute((const void *)kernel,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
+    if (e != hipSuccess) return (int)e;
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(hist_num_cus()), dim3(HIST_BLOCK), HIST_LDS_BYTES, st, pis, pvs,
+                     sc.gbase, dest, H, shift);
+  return launch_status();
+}
+
 template <class T, class Op>
 static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs, int64_t n,
                        void *dest, int64_t H, void *scratch, size_t scratch_bytes) {
-  (void)scratch;
-  (void)scratch_bytes;
   if (H == 0 || n == 0) return 0;
   if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
   const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)sizeof(T));
   if (H <= lds_limit) {
     if (is64) return launch_lds_hist<T, Op, int64_t>(st, (const int64_t *)is, (const T *)vs, n, (T *)dest, H);
     return launch_lds_hist<T, Op, int32_t>(st, (const int32_t *)is, (const T *)vs, n, (T *)dest, H);
+  }
+  const int64_t part_limit = (int64_t)255 << hist_part_shift<T>();
+  if (H <= part_limit && n < ((int64_t)1 << 30)) {
+    if (is64)
+      return launch_part_hist<T, Op, uint64_t>(st, (const uint64_t *)is, (const T *)vs, n,
+                                               (T *)dest, H, scratch, scratch_bytes);
+    return launch_part_hist<T, Op, uint32_t>(st, (const uint32_t *)is, (const T *)vs, n, (T *)dest,
+                                             H, scratch, scratch_bytes);
   }
   const int grid = hist_num_cus() * 8;
   if (is64)
@@ -254,10 +358,15 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
 
 }  // namespace fa
 
-extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int64_t H) {
-  (void)t;
-  (void)H;
-  return 256;
+extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int64_t H) {
+  const size_t es = dtype_size(t);
+  if (es != 4 && es != 8) return 0;
+  if (n < 0) n = 0;
+  const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)es);
+  const int64_t part_limit = (int64_t)255 << (es == 4 ? 15 : 14);
+  if (H <= lds_limit || H > part_limit) return 256;
+  return hist_align(rs_scratch_bytes(rs_num_tiles(n), 1)) +
+         hist_align((size_t)n * (is64 ? 8 : 4)) + (size_t)n * es + 256;
 }
 
 extern "C" int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op, const void *is, int is64,

