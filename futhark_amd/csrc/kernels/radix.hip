@@ -1,26 +1,12 @@
-// Stable LSD radix sort for gfx950, 8-bit digits, one read and one write of the
-// data per pass.
+// Stable LSD radix sort for gfx950, 8-bit digits.
 //
-// Result-wise each pass is the composition the reference reaches radix sort
-// through (tests/issue2234.fut:10-44, tests/ad/custom/radixsort.fut:13-25): a
-// histogram of the digit (SegHist), an exclusive scan of the counts (SegScan)
-// and a scatter to offset + rank (src/Futhark/Tools.hs:328-363).  The schedule
-// fuses them so that no n-length intermediate ever exists:
-//   * one up-front kernel builds the digit histograms of ALL passes from a
-//     single read of the keys (LDS sub-histograms per wave, one flush);
-//   * a pass is ONE kernel.  A tile (1024 threads x 16 keys) ranks its keys:
-//     inside a wave, lanes with equal digits find each other with eight
-//     ballots; per-wave digit counters in LDS chain the 16 rounds.  The tile's
-//     256 digit counts are published and the counts of all earlier tiles are
-//     gathered by decoupled look-back, one thread per digit (the chained-scan
-//     protocol of SegScan/SinglePass.hs:625-777 applied to 256 counters at
-//     once), which replaces the separate count-scan kernel;
-//   * the tile is reordered in LDS so that global stores are contiguous runs
-//     per digit.
-// Order is preserved at every level (round, lane, wave, tile): the sort is
-// stable.  The same pass, with a digit function that maps a histogram bin to
-// its LDS-sized bin range, partitions (index, value) pairs for large
-// histograms (seghist.hip).
+// Each pass is the composition the reference reaches radix sort through
+// (tests/issue2234.fut:10-44, tests/ad/custom/radixsort.fut:13-25): a histogram
+// of the digit per tile (SegHist), an exclusive scan of the counts laid out
+// digit-major (SegScan, the single-pass kernel of segscan.hip) and a scatter
+// to the scanned offset plus the rank of the key inside its tile
+// (src/Futhark/Tools.hs:328-363 for scatter).  The rank is computed without any
+// n-length intermediate (radix.hip.h).  The sort is stable.
 #include "radix.hip.h"
 
 namespace fa {
@@ -37,10 +23,9 @@ template <class K, int VB>
 static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const void *vin, void *vout,
                        void *vtmp, int64_t n, int begin_bit, int end_bit, void *scratch) {
   const int passes = (end_bit - begin_bit) / 8;
-  const int64_t tiles = rs_num_tiles(n);
-  RsScratch sc = rs_carve(scratch, tiles, passes);
+  RsScratch sc = rs_carve(scratch, rs_num_tiles(n));
   DigitBits<K> fn{begin_bit};
-  int rc = rs_prepare<K>(st, kin, n, fn, passes, sc);
+  int rc = rs_prepare(st, sc);
   if (rc != 0) return rc;
   // With an even number of passes the ping-pong ends in `out` if it starts by
   // writing `tmp`; with an odd number it starts by writing `out`.
@@ -50,7 +35,7 @@ static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const voi
     const bool to_out = ((passes - 1 - p) % 2) == 0;
     K *dst_k = to_out ? kout : ktmp;
     void *dst_v = to_out ? vout : vtmp;
-    rc = rs_pass<K, VB>(st, src_k, dst_k, src_v, dst_v, n, fn, p, sc);
+    rc = rs_pass<K, VB>(st, src_k, dst_k, src_v, dst_v, n, fn, p, (uint32_t)(p + 1), sc);
     if (rc != 0) return rc;
     src_k = dst_k;
     src_v = dst_v;
@@ -62,14 +47,14 @@ static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const voi
 
 extern "C" size_t fa_radix_sort_scratch_bytes(int64_t n) {
   if (n < 0) n = 0;
-  return rs_scratch_bytes(rs_num_tiles(n), 8);
+  return rs_scratch_bytes(rs_num_tiles(n));
 }
 
 extern "C" int fa_radix_sort(fa_stream_t stream, int key_bytes, int val_bytes, const void *keys_in,
                              void *keys_out, void *keys_tmp, const void *vals_in, void *vals_out,
                              void *vals_tmp, int64_t n, int begin_bit, int end_bit, void *scratch,
                              size_t scratch_bytes) {
-  if (n < 0 || n >= ((int64_t)1 << 30)) return FA_EINVAL;
+  if (n < 0 || n >= ((int64_t)1 << 31)) return FA_EINVAL;
   if (key_bytes != 4 && key_bytes != 8) return FA_ENOTSUP;
   if (val_bytes != 0 && val_bytes != 4 && val_bytes != 8) return FA_ENOTSUP;
   if (begin_bit < 0 || end_bit > key_bytes * 8 || end_bit < begin_bit ||

@@ -190,17 +190,18 @@ template <class U> struct DigitBinRange {
   }
 };
 
-// Input: pairs grouped by bin range (range r occupies [gbase[r], gbase[r+1])).
-// Each block takes a contiguous chunk of the valid pairs and, for every range
-// the chunk touches, accumulates in LDS and flushes.
+// Input: pairs grouped by bin range; range r starts at offs[r * num_tiles] (the
+// digit-major offsets of the partition pass).  Each block takes a contiguous
+// chunk of the valid pairs and, for every range the chunk touches, accumulates
+// in LDS and flushes.
 template <class T, class Op, class U>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
-    const U *__restrict__ pis, const T *__restrict__ pvs, const uint32_t *__restrict__ gbase,
-    T *dest, int64_t H, int shift) {
+    const U *__restrict__ pis, const T *__restrict__ pvs, const uint32_t *__restrict__ offs,
+    int64_t num_tiles, T *dest, int64_t H, int shift) {
   extern __shared__ __align__(16) unsigned char s_raw[];
   T *sh = reinterpret_cast<T *>(s_raw);
   __shared__ uint32_t s_start[RS_RADIX];
-  if (threadIdx.x < RS_RADIX) s_start[threadIdx.x] = gbase[threadIdx.x];
+  if (threadIdx.x < RS_RADIX) s_start[threadIdx.x] = offs[(int64_t)threadIdx.x * num_tiles];
   __syncthreads();
   const int64_t n_valid = s_start[RS_RADIX - 1];
   const int64_t chunk = ceil_div(ceil_div(n_valid, (int64_t)gridDim.x), 4) * 4;
@@ -303,17 +304,17 @@ static int launch_part_hist(hipStream_t st, const U *is, const T *vs, int64_t n,
                             int64_t H, void *scratch, size_t scratch_bytes) {
   constexpr int shift = hist_part_shift<T>();
   const int64_t tiles = rs_num_tiles(n);
-  const size_t rs_bytes = hist_align(rs_scratch_bytes(tiles, 1));
+  const size_t rs_bytes = hist_align(rs_scratch_bytes(tiles));
   const size_t is_bytes = hist_align((size_t)n * sizeof(U));
   if (scratch_bytes < rs_bytes + is_bytes + (size_t)n * sizeof(T)) return FA_ESCRATCH;
   if (!is_aligned(scratch, 256)) return FA_EALIGN;
   U *pis = (U *)((char *)scratch + rs_bytes);
   T *pvs = (T *)((char *)scratch + rs_bytes + is_bytes);
-  RsScratch sc = rs_carve(scratch, tiles, 1);
+  RsScratch sc = rs_carve(scratch, tiles);
   DigitBinRange<U> fn{(uint64_t)H, shift};
-  int rc = rs_prepare<U>(st, is, n, fn, 1, sc);
+  int rc = rs_prepare(st, sc);
   if (rc != 0) return rc;
-  rc = rs_pass<U, (int)sizeof(T)>(st, is, pis, vs, pvs, n, fn, 0, sc);
+  rc = rs_pass<U, (int)sizeof(T)>(st, is, pis, vs, pvs, n, fn, 0, 1u, sc);
   if (rc != 0) return rc;
   auto kernel = seghist_part_kernel<T, Op, U>;
   static bool raised = false;
@@ -324,7 +325,7 @@ static int launch_part_hist(hipStream_t st, const U *is, const T *vs, int64_t n,
     raised = true;
   }
   hipLaunchKernelGGL(kernel, dim3(hist_num_cus()), dim3(HIST_BLOCK), HIST_LDS_BYTES, st, pis, pvs,
-                     sc.gbase, dest, H, shift);
+                     sc.offsets, sc.tiles, dest, H, shift);
   return launch_status();
 }
 
@@ -339,7 +340,7 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
     return launch_lds_hist<T, Op, int32_t>(st, (const int32_t *)is, (const T *)vs, n, (T *)dest, H);
   }
   const int64_t part_limit = (int64_t)255 << hist_part_shift<T>();
-  if (H <= part_limit && n < ((int64_t)1 << 30)) {
+  if (H <= part_limit && n < ((int64_t)1 << 31)) {
     if (is64)
       return launch_part_hist<T, Op, uint64_t>(st, (const uint64_t *)is, (const T *)vs, n,
                                                (T *)dest, H, scratch, scratch_bytes);
@@ -365,7 +366,7 @@ extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int6
   const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)es);
   const int64_t part_limit = (int64_t)255 << (es == 4 ? 15 : 14);
   if (H <= lds_limit || H > part_limit) return 256;
-  return hist_align(rs_scratch_bytes(rs_num_tiles(n), 1)) +
+  return hist_align(rs_scratch_bytes(rs_num_tiles(n))) +
          hist_align((size_t)n * (is64 ? 8 : 4)) + (size_t)n * es + 256;
 }
 
