@@ -10,13 +10,14 @@
 //     128x128 sub-tile as 4x4 MFMA tiles of 32x32 (256 accumulator registers);
 //   * f16/bf16 use v_mfma_f32_32x32x16, f32 uses v_mfma_f32_32x32x2;
 //   * A tiles sit in LDS as [m][k] with a 16-byte XOR swizzle so that the
-//     128-bit fragment reads of 8 consecutive rows hit distinct banks;
+//     128-bit fragment reads hit distinct banks;
 //   * B stays row-major [k][n] all the way into LDS; the f16/bf16 fragments
 //     (8 consecutive k for one n) come out of LDS through the transposing read
 //     ds_read_b64_tr_b16, so B is never transposed in memory (the reference
 //     may materialise `transpose B` with map_transpose);
-//   * global loads for tile k+1 are in flight while tile k is multiplied; LDS
-//     is double buffered, one barrier per k-step.
+//   * LDS is double buffered, one barrier per k-step; f16/bf16 tiles go from
+//     global memory straight into LDS (no register staging) while the previous
+//     tile is multiplied, with the MFMA / LDS-read / load order fixed by hand.
 // Shapes that are not multiples of the tile go to a plain LDS-tiled kernel.
 #include "dispatch.hip.h"
 
@@ -54,33 +55,78 @@ constexpr int MM_A_ROW_BYTES = 64;                     // one k-step of a row of
 constexpr int MM_A_TILE_BYTES = MM_BM * MM_A_ROW_BYTES;  // 16 KiB
 
 // ---------------------------------------------------------------- 16-bit inputs
-// k-step: 64 elements, i.e. 128-byte rows of A (eight 16-byte units, XOR
-// swizzled with the low three bits of the row) and 64 rows of B of 256
-// elements, row stride padded by 32 bytes so that the four rows touched by one
-// transposing read fall on different banks.  A step is 64 MFMAs per wave,
-// long enough to hide the HBM/L2 latency of the loads for the next step.
+// k-step: 64 elements.  Tiles travel from global memory straight into LDS
+// (global_load_lds_dwordx4: lane l of a wave deposits 16 bytes at M0 + 16 l, so
+// one instruction fills 1 KiB of LDS and the swizzles below are applied by
+// choosing which global unit each lane fetches):
+//   A: 256 rows of 128 bytes, eight 16-byte units per row; unit u of row m sits
+//      in slot u ^ ((m >> 1) & 7), so the 16 lanes of one phase of a 128-bit
+//      fragment read (16 consecutive rows, one unit) cover all 64 banks once;
+//   B: 64 rows [k] of 512 bytes (256 n), 32 units per row; unit u of row k sits
+//      in slot u ^ ((k & 3) << 2), so the four rows touched by one transposing
+//      read (64 bytes each) fall into different 64-byte bank groups.
+// Nothing is staged in registers, and LDS is double buffered with one barrier
+// per k-step.
 constexpr int MM16_BK = 64;
 constexpr int MM16_A_ROW_BYTES = MM16_BK * 2;
 constexpr int MM16_A_TILE_BYTES = MM_BM * MM16_A_ROW_BYTES;  // 32 KiB
-constexpr int MM16_B_STRIDE = MM_BN * 2 + 32;                // bytes
-constexpr int MM16_B_TILE_BYTES = MM16_BK * MM16_B_STRIDE;
+constexpr int MM16_B_ROW_BYTES = MM_BN * 2;
+constexpr int MM16_B_TILE_BYTES = MM16_BK * MM16_B_ROW_BYTES;  // 32 KiB
 constexpr int MM16_STAGE_BYTES = MM16_A_TILE_BYTES + MM16_B_TILE_BYTES;
-constexpr int MM16_UNITS = 8;  // 16-byte units per thread per operand per step
+// Four waves in a 2 x 2 arrangement, each computing a 128 x 128 sub-tile (4 x 4
+// MFMA tiles, 256 accumulator registers): the arrangement with the least LDS
+// read traffic per MFMA (8 waves as 2 x 4 measured the same speed).
+constexpr int MM16_WAVES_M = 2, MM16_WAVES_N = 2;
+constexpr int MM16_WAVES = MM16_WAVES_M * MM16_WAVES_N;
+constexpr int MM16_THREADS = 64 * MM16_WAVES;
+constexpr int MM16_MT = MM_BM / (MM16_WAVES_M * 32);  // MFMA tiles per wave along m
+constexpr int MM16_NT = MM_BN / (MM16_WAVES_N * 32);  // and along n
+constexpr int MM16_CHUNKS = MM16_A_TILE_BYTES / 1024 / MM16_WAVES;  // 1 KiB loads per wave, per operand
+// The loads of the next tile ride on the first two k16 steps of a tile, which
+// leaves them the other two steps to land before the barrier.
+constexpr int MM16_LOAD_KSTEPS = 2;
 
 __device__ __forceinline__ int a16_swizzled_offset(int m, int unit) {
-  return m * MM16_A_ROW_BYTES + ((unit ^ (m & 7)) << 4);
+  return m * MM16_A_ROW_BYTES + ((unit ^ ((m >> 1) & 7)) << 4);
+}
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N-1>), in order: a
+// loop whose index is a compile-time constant in every iteration.
+template <int N, class F> __device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+// One direct global -> LDS load of 16 bytes per lane.  `lds_addr` (wave
+// uniform) goes to M0; the kernel has no other user of M0.  The compiler does
+// not track this load: the caller waits for vmcnt before the barrier that
+// publishes the tile.
+// The source is a wave-uniform base (scalar registers) plus a 32-bit per-lane
+// byte offset, so the loads of a tile cost no vector registers for addresses.
+__device__ __forceinline__ void load_to_lds_16(const char *uniform_base, uint32_t lane_offset,
+                                               uint32_t lds_addr) {
+  const uint64_t base = (uint64_t)uniform_base;
+  const uint64_t sbase =
+      ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(base >> 32)) << 32) |
+      (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)base);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(
+                   __builtin_amdgcn_readfirstlane(lds_addr)),
+               "v"(lane_offset), "s"(sbase)
+               : "memory");
 }
 
 template <bool BF16>
-__global__ __launch_bounds__(MM_THREADS) void matmul16_kernel(const uint16_t *__restrict__ A,
-                                                              const uint16_t *__restrict__ B,
-                                                              float *__restrict__ C, int M, int N,
-                                                              int K) {
+__global__ __launch_bounds__(MM16_THREADS) void matmul16_kernel(const uint16_t *__restrict__ A,
+                                                                const uint16_t *__restrict__ B,
+                                                                float *__restrict__ C, int M,
+                                                                int N, int K) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / MM16_WAVES_N, wn = wave % MM16_WAVES_N;
   const int64_t batch = blockIdx.z;
   int tile_m, tile_n;
   mm_tile_of_block(tile_m, tile_n);
@@ -89,210 +135,177 @@ __global__ __launch_bounds__(MM_THREADS) void matmul16_kernel(const uint16_t *__
   const uint16_t *Bb = B + batch * (int64_t)K * N;
   float *Cb = C + batch * (int64_t)M * N;
 
-  // This thread's 16-byte units of the A tile and of the B tile: unit i is
-  // 32 rows of A (8 rows of B) below unit 0, so one base address each and
-  // constant strides describe all of them.
-  const int am0 = tid >> 3, au = tid & 7;
-  const int bk0 = tid >> 5, bu = tid & 31;
-  // Addresses are a block-uniform base (scalar registers) plus one 32-bit
-  // per-thread byte offset, which keeps the 16 loads of a step off the vector
-  // register budget.
-  const char *a_base = reinterpret_cast<const char *>(Ab + (int64_t)bm * K);
-  const char *b_base = reinterpret_cast<const char *>(Bb + bn);
-  const uint32_t a_toff = (uint32_t)(am0 * K + au * 8) * 2u;
-  const uint32_t b_toff = (uint32_t)(bk0 * N + bu * 8) * 2u;
-  const int64_t a_src_step = (int64_t)32 * K * 2;  // bytes between units
-  const int64_t b_src_step = (int64_t)8 * N * 2;
-  const int a_dst0 = a16_swizzled_offset(am0, au);  // (am0 + 32 i) & 7 == am0 & 7
-  const int b_dst0 = MM16_A_TILE_BYTES + bk0 * MM16_B_STRIDE + bu * 16;
-  constexpr int a_dst_step = 32 * MM16_A_ROW_BYTES;
-  constexpr int b_dst_step = 8 * MM16_B_STRIDE;
+  // Loads.  Chunk c of the A tile is rows 8c..8c+7 (1 KiB of LDS), chunk c of
+  // the B tile is rows 2c, 2c+1.  Wave w moves chunks w, w + WAVES, ...; since
+  // WAVES is even the swizzle term of a lane's row does not depend on the
+  // chunk, so a lane's chunks differ by a constant stride in global memory.
+  static_assert(MM16_WAVES % 2 == 0, "swizzle terms assume an even chunk stride");
+  const int a_r = lane >> 3, a_slot = lane & 7;
+  const int a_unit = a_slot ^ (((wave & 1) << 2) | (a_r >> 1));  // ((8 w + a_r) >> 1) & 7
+  const int b_r = lane >> 5, b_slot = lane & 31;
+  const int b_unit = b_slot ^ ((((wave & 1) << 1) | b_r) << 2);  // ((2 w + b_r) & 3) << 2
+  const char *a_src = reinterpret_cast<const char *>(Ab + (int64_t)(bm + wave * 8) * K);
+  const char *b_src = reinterpret_cast<const char *>(Bb + (int64_t)(wave * 2) * N + bn);
+  const uint32_t a_lane = (uint32_t)(a_r * K * 2 + a_unit * 16);  // K, N < 2^27 elements
+  const uint32_t b_lane = (uint32_t)(b_r * N * 2 + b_unit * 16);
+  const int64_t a_chunk_step = (int64_t)MM16_WAVES * 8 * K * 2;
+  const int64_t b_chunk_step = (int64_t)MM16_WAVES * 2 * N * 2;
+  const int64_t b_tile_step = (int64_t)MM16_BK * N * 2;
+  const uint32_t lds_base =
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
+  const uint32_t a_dst = lds_base + wave * 1024;
+  const uint32_t b_dst = lds_base + MM16_A_TILE_BYTES + wave * 1024;
+  // Load j of a tile: even j moves a chunk of A, odd j a chunk of B.
+  auto fetch_one = [&](int kt, int stage, int j) __attribute__((always_inline)) {
+    const int i = j >> 1;
+    if ((j & 1) == 0)
+      load_to_lds_16(a_src + (int64_t)kt * (MM16_BK * 2) + i * a_chunk_step, a_lane,
+                     a_dst + stage * MM16_STAGE_BYTES + i * (MM16_WAVES * 1024));
+    else
+      load_to_lds_16(b_src + (int64_t)kt * b_tile_step + i * b_chunk_step, b_lane,
+                     b_dst + stage * MM16_STAGE_BYTES + i * (MM16_WAVES * 1024));
+  };
 
-  f32x16 acc[4][4];
+  f32x16 acc[MM16_MT][MM16_NT];
 #pragma unroll
-  for (int i = 0; i < 4; i++)
+  for (int i = 0; i < MM16_MT; i++)
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < MM16_NT; j++)
 #pragma unroll
       for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
-  const int KT = K / MM16_BK;
-#pragma unroll
-  for (int i = 0; i < MM16_UNITS; i++) {
-    *reinterpret_cast<uint4 *>(lds + a_dst0 + i * a_dst_step) =
-        *reinterpret_cast<const uint4 *>(a_base + i * a_src_step + a_toff);
-    *reinterpret_cast<uint4 *>(lds + b_dst0 + i * b_dst_step) =
-        *reinterpret_cast<const uint4 *>(b_base + i * b_src_step + b_toff);
-  }
-  __syncthreads();
-
   // Fragment addresses inside a stage (k16 step 0; later steps add constants).
-  const int a_row = wm * 128 + (lane & 31);  // + mt * 32
-  const int a_half = lane >> 5;              // which 8 of the 16 k of a step
-  int b_frag[4];                             // [n-tile], first of the two transposing reads
+  const int a_row = wm * (MM16_MT * 32) + (lane & 31);  // + mt * 32
+  const int a_half = lane >> 5;                         // which 8 of the 16 k of a step
+  int b_frag[MM16_NT];  // [n-tile], first of the two transposing reads
   {
+    // Lane r of a group of 16 supplies the 8 bytes at row kbase + r/4, columns
+    // n0 + 4 (r%4) .. +3; the read hands lane j the k-column it needs.
     const int r = lane & 15;
-    const int kbase = (lane >> 5) * 8 + (r >> 2);
+    const int kbase = (lane >> 5) * 8 + (r >> 2);  // kbase & 3 == r >> 2 in every step
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++) {
-      const int n0 = wn * 128 + nt * 32 + ((lane >> 4) & 1) * 16 + 4 * (r & 3);
-      b_frag[nt] = MM16_A_TILE_BYTES + kbase * MM16_B_STRIDE + n0 * 2;
+    for (int nt = 0; nt < MM16_NT; nt++) {
+      const int n0 = wn * (MM16_NT * 32) + nt * 32 + ((lane >> 4) & 1) * 16 + 4 * (r & 3);
+      const int unit = (n0 >> 3) ^ ((r >> 2) << 2);
+      b_frag[nt] = MM16_A_TILE_BYTES + kbase * MM16_B_ROW_BYTES + unit * 16 + (n0 & 7) * 2;
     }
   }
 
-  auto multiply = [&](const unsigned char *stage) {
-#pragma unroll
-    for (int ks = 0; ks < MM16_BK / 16; ks++) {
-      uint4 af[4], bf[4];
-#pragma unroll
-      for (int mt = 0; mt < 4; mt++)
-        af[mt] = *reinterpret_cast<const uint4 *>(
-            stage + a16_swizzled_offset(a_row + mt * 32, ks * 2 + a_half));
-#pragma unroll
-      for (int nt = 0; nt < 4; nt++) {
-        const unsigned char *p = stage + b_frag[nt] + ks * 16 * MM16_B_STRIDE;
-        const i16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (i16x4 __attribute__((address_space(3))) *)(p));
-        const i16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (i16x4 __attribute__((address_space(3))) *)(p + 4 * MM16_B_STRIDE));
-        uint2 l2 = bit_cast<uint2>(lo), h2 = bit_cast<uint2>(hi);
-        bf[nt] = make_uint4(l2.x, l2.y, h2.x, h2.y);
-      }
-#pragma unroll
-      for (int mt = 0; mt < 4; mt++)
-#pragma unroll
-        for (int nt = 0; nt < 4; nt++) {
-          if constexpr (BF16) {
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                bit_cast<bf16x8>(af[mt]), bit_cast<bf16x8>(bf[nt]), acc[mt][nt], 0, 0, 0);
-          } else {
-            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                bit_cast<f16x8>(af[mt]), bit_cast<f16x8>(bf[nt]), acc[mt][nt], 0, 0, 0);
-          }
-        }
+  // A k16 step is MT*NT MFMAs, walked n-tile by n-tile.  Its instruction order
+  // is fixed by hand (a scheduling barrier after every MFMA):
+  //   * after each of the first MT + 2 NT MFMAs one LDS read of the next step's
+  //     fragments is issued (fragments are double buffered), in the order the
+  //     next step consumes them: B0, A0..A(MT-1), B1, B2, ...  The last reads
+  //     are needed only late in the next step, so no MFMA waits on a read that
+  //     was issued just before it;
+  //   * after every second MFMA of the first steps one load of the next tile is
+  //     issued.  Loads are spread out because a wave that issues many of them
+  //     back to back stalls until the memory pipeline has taken them, with its
+  //     SIMD's MFMA unit idle meanwhile.
+  constexpr int KSTEPS = MM16_BK / 16;
+  constexpr int MFMAS = MM16_MT * MM16_NT, READS = MM16_MT + 2 * MM16_NT;
+  static_assert(READS <= MFMAS, "one LDS read follows one MFMA");
+  constexpr int LOADS = 2 * MM16_CHUNKS;  // per wave and tile
+  static_assert(LOADS % MM16_LOAD_KSTEPS == 0, "loads divide evenly over the steps");
+  constexpr int LOADS_PER_STEP = LOADS / MM16_LOAD_KSTEPS;
+  static_assert(MFMAS % LOADS_PER_STEP == 0, "loads divide evenly over the MFMAs");
+  constexpr int MFMAS_PER_LOAD = MFMAS / LOADS_PER_STEP;
+  struct Frags {
+    uint4 a[MM16_MT];
+    uint4 b[MM16_NT];  // .xy: k 0..3|8..11 of the step, .zw: k 4..7|12..15 (one read each)
+  };
+  auto read_b_half = [&](const unsigned char *stage, int ks, int nt,
+                         int half) __attribute__((always_inline)) -> uint2 {
+    const unsigned char *p =
+        stage + b_frag[nt] + (ks * 16 + half * 4) * MM16_B_ROW_BYTES;
+    return bit_cast<uint2>(__builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (i16x4 __attribute__((address_space(3))) *)(p)));
+  };
+  // Read number `idx` of a step, in consumption order.
+  auto issue_read = [&](const unsigned char *stage, int ks, int idx,
+                        Frags &f) __attribute__((always_inline)) {
+    if (idx < 2) {
+      const uint2 h = read_b_half(stage, ks, 0, idx);
+      if (idx == 0) f.b[0].x = h.x, f.b[0].y = h.y;
+      else f.b[0].z = h.x, f.b[0].w = h.y;
+    } else if (idx < 2 + MM16_MT) {
+      const int mt = idx - 2;
+      f.a[mt] = *reinterpret_cast<const uint4 *>(
+          stage + a16_swizzled_offset(a_row + mt * 32, ks * 2 + a_half));
+    } else {
+      const int j = idx - 2 - MM16_MT, nt = 1 + (j >> 1);
+      const uint2 h = read_b_half(stage, ks, nt, j & 1);
+      if ((j & 1) == 0) f.b[nt].x = h.x, f.b[nt].y = h.y;
+      else f.b[nt].z = h.x, f.b[nt].w = h.y;
     }
   };
+  auto k16_step = [&](const unsigned char *stage, int ks, const Frags &cur, Frags &next,
+                      int next_kt, int next_stage, auto fetch) __attribute__((always_inline)) {
+    static_for<MFMAS>([&](auto ic) __attribute__((always_inline)) {
+      constexpr int i = decltype(ic)::value;
+      constexpr int nt = i / MM16_MT, mt = i % MM16_MT;
+      const uint4 bfrag = cur.b[nt];
+      if constexpr (BF16) {
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            bit_cast<bf16x8>(cur.a[mt]), bit_cast<bf16x8>(bfrag), acc[mt][nt], 0, 0, 0);
+      } else {
+        acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+            bit_cast<f16x8>(cur.a[mt]), bit_cast<f16x8>(bfrag), acc[mt][nt], 0, 0, 0);
+      }
+      if (ks + 1 < KSTEPS && i < READS) issue_read(stage, ks + 1, i, next);
+      if constexpr (decltype(fetch)::value)
+        if (ks < MM16_LOAD_KSTEPS && i % MFMAS_PER_LOAD == MFMAS_PER_LOAD - 1)
+        fetch_one(next_kt, next_stage, ks * LOADS_PER_STEP + i / MFMAS_PER_LOAD);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  auto multiply = [&](const unsigned char *stage, int next_kt, int next_stage,
+                      auto fetch) __attribute__((always_inline)) {
+    Frags f0, f1;
+    static_for<READS>([&](auto ic) __attribute__((always_inline)) { issue_read(stage, 0, decltype(ic)::value, f0); });
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks += 2) {
+      k16_step(stage, ks, f0, f1, next_kt, next_stage, fetch);
+      k16_step(stage, ks + 1, f1, f0, next_kt, next_stage, fetch);
+    }
+  };
+  // All of this wave's loads have landed, then all waves': the tile is public.
+  auto publish = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+  };
 
-  // Steady state.  Two register sets hold the tiles that are in flight from
-  // HBM/L2: while tile kt is multiplied out of LDS, tile kt+1 (requested one
-  // step earlier) is parked in the other LDS stage and tile kt+2 is requested.
-  // A load therefore has two multiply steps (128 MFMAs per wave) to arrive.
-  // The staged tiles are individual registers on purpose: as arrays carried
-  // around the loop they were kept in scratch memory by the compiler.
-  static_assert(MM16_UNITS == 8, "the staging code below is written out for 8 units");
-  uint4 pa0, pa1, pa2, pa3, pa4, pa5, pa6, pa7, pb0, pb1, pb2, pb3, pb4, pb5, pb6, pb7, qa0, qa1, qa2, qa3, qa4, qa5, qa6, qa7, qb0, qb1, qb2, qb3, qb4, qb5, qb6, qb7;
-#define MM16_KOFF(T) const int64_t koff_ = (int64_t)((T) > KT - 1 ? KT - 1 : (T)) * MM16_BK * 2
-#define MM16_FETCH_P(T) \
-  do { \
-    MM16_KOFF(T); \
-    pa0 = *reinterpret_cast<const uint4 *>(a_base + (0 * a_src_step + koff_) + a_toff); \
-    pb0 = *reinterpret_cast<const uint4 *>(b_base + (0 * b_src_step + koff_ * N) + b_toff); \
-    pa1 = *reinterpret_cast<const uint4 *>(a_base + (1 * a_src_step + koff_) + a_toff); \
-    pb1 = *reinterpret_cast<const uint4 *>(b_base + (1 * b_src_step + koff_ * N) + b_toff); \
-    pa2 = *reinterpret_cast<const uint4 *>(a_base + (2 * a_src_step + koff_) + a_toff); \
-    pb2 = *reinterpret_cast<const uint4 *>(b_base + (2 * b_src_step + koff_ * N) + b_toff); \
-    pa3 = *reinterpret_cast<const uint4 *>(a_base + (3 * a_src_step + koff_) + a_toff); \
-    pb3 = *reinterpret_cast<const uint4 *>(b_base + (3 * b_src_step + koff_ * N) + b_toff); \
-    pa4 = *reinterpret_cast<const uint4 *>(a_base + (4 * a_src_step + koff_) + a_toff); \
-    pb4 = *reinterpret_cast<const uint4 *>(b_base + (4 * b_src_step + koff_ * N) + b_toff); \
-    pa5 = *reinterpret_cast<const uint4 *>(a_base + (5 * a_src_step + koff_) + a_toff); \
-    pb5 = *reinterpret_cast<const uint4 *>(b_base + (5 * b_src_step + koff_ * N) + b_toff); \
-    pa6 = *reinterpret_cast<const uint4 *>(a_base + (6 * a_src_step + koff_) + a_toff); \
-    pb6 = *reinterpret_cast<const uint4 *>(b_base + (6 * b_src_step + koff_ * N) + b_toff); \
-    pa7 = *reinterpret_cast<const uint4 *>(a_base + (7 * a_src_step + koff_) + a_toff); \
-    pb7 = *reinterpret_cast<const uint4 *>(b_base + (7 * b_src_step + koff_ * N) + b_toff); \
-  } while (0)
-#define MM16_FETCH_Q(T) \
-  do { \
-    MM16_KOFF(T); \
-    qa0 = *reinterpret_cast<const uint4 *>(a_base + (0 * a_src_step + koff_) + a_toff); \
-    qb0 = *reinterpret_cast<const uint4 *>(b_base + (0 * b_src_step + koff_ * N) + b_toff); \
-    qa1 = *reinterpret_cast<const uint4 *>(a_base + (1 * a_src_step + koff_) + a_toff); \
-    qb1 = *reinterpret_cast<const uint4 *>(b_base + (1 * b_src_step + koff_ * N) + b_toff); \
-    qa2 = *reinterpret_cast<const uint4 *>(a_base + (2 * a_src_step + koff_) + a_toff); \
-    qb2 = *reinterpret_cast<const uint4 *>(b_base + (2 * b_src_step + koff_ * N) + b_toff); \
-    qa3 = *reinterpret_cast<const uint4 *>(a_base + (3 * a_src_step + koff_) + a_toff); \
-    qb3 = *reinterpret_cast<const uint4 *>(b_base + (3 * b_src_step + koff_ * N) + b_toff); \
-    qa4 = *reinterpret_cast<const uint4 *>(a_base + (4 * a_src_step + koff_) + a_toff); \
-    qb4 = *reinterpret_cast<const uint4 *>(b_base + (4 * b_src_step + koff_ * N) + b_toff); \
-    qa5 = *reinterpret_cast<const uint4 *>(a_base + (5 * a_src_step + koff_) + a_toff); \
-    qb5 = *reinterpret_cast<const uint4 *>(b_base + (5 * b_src_step + koff_ * N) + b_toff); \
-    qa6 = *reinterpret_cast<const uint4 *>(a_base + (6 * a_src_step + koff_) + a_toff); \
-    qb6 = *reinterpret_cast<const uint4 *>(b_base + (6 * b_src_step + koff_ * N) + b_toff); \
-    qa7 = *reinterpret_cast<const uint4 *>(a_base + (7 * a_src_step + koff_) + a_toff); \
-    qb7 = *reinterpret_cast<const uint4 *>(b_base + (7 * b_src_step + koff_ * N) + b_toff); \
-  } while (0)
-#define MM16_PARK_P(STAGE) \
-  do { \
-    unsigned char *dst_ = lds + (STAGE)*MM16_STAGE_BYTES; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 0 * a_dst_step) = pa0; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 0 * b_dst_step) = pb0; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 1 * a_dst_step) = pa1; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 1 * b_dst_step) = pb1; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 2 * a_dst_step) = pa2; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 2 * b_dst_step) = pb2; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 3 * a_dst_step) = pa3; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 3 * b_dst_step) = pb3; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 4 * a_dst_step) = pa4; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 4 * b_dst_step) = pb4; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 5 * a_dst_step) = pa5; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 5 * b_dst_step) = pb5; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 6 * a_dst_step) = pa6; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 6 * b_dst_step) = pb6; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 7 * a_dst_step) = pa7; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 7 * b_dst_step) = pb7; \
-  } while (0)
-#define MM16_PARK_Q(STAGE) \
-  do { \
-    unsigned char *dst_ = lds + (STAGE)*MM16_STAGE_BYTES; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 0 * a_dst_step) = qa0; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 0 * b_dst_step) = qb0; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 1 * a_dst_step) = qa1; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 1 * b_dst_step) = qb1; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 2 * a_dst_step) = qa2; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 2 * b_dst_step) = qb2; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 3 * a_dst_step) = qa3; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 3 * b_dst_step) = qb3; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 4 * a_dst_step) = qa4; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 4 * b_dst_step) = qb4; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 5 * a_dst_step) = qa5; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 5 * b_dst_step) = qb5; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 6 * a_dst_step) = qa6; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 6 * b_dst_step) = qb6; \
-    *reinterpret_cast<uint4 *>(dst_ + a_dst0 + 7 * a_dst_step) = qa7; \
-    *reinterpret_cast<uint4 *>(dst_ + b_dst0 + 7 * b_dst_step) = qb7; \
-  } while (0)
-  MM16_FETCH_P(1);
+  const int KT = K / MM16_BK;
+#pragma unroll
+  for (int j = 0; j < LOADS; j++) fetch_one(0, 0, j);
+  publish();
+  // While tile kt is multiplied out of one stage, tile kt+1 streams into the
+  // other, which every wave finished reading before the previous barrier.
+  // The tile after the last one is the last one again (loaded, never used),
+  // which keeps the loop free of special cases.
+  constexpr std::true_type with_fetch{};
   for (int kt = 0; kt + 1 < KT; kt += 2) {
-    MM16_FETCH_Q(kt + 2);
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(lds);  // tile kt sits in stage 0
-    __builtin_amdgcn_sched_barrier(0);
-    MM16_PARK_P(1);
-    __syncthreads();
-    MM16_FETCH_P(kt + 3);
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(lds + MM16_STAGE_BYTES);  // tile kt+1
-    __builtin_amdgcn_sched_barrier(0);
-    if (kt + 2 < KT) MM16_PARK_Q(0);
-    __syncthreads();
+    multiply(lds, kt + 1, 1, with_fetch);
+    publish();
+    multiply(lds + MM16_STAGE_BYTES, kt + 2 < KT ? kt + 2 : KT - 1, 0, with_fetch);
+    publish();
   }
-#undef MM16_KOFF
-#undef MM16_FETCH_P
-#undef MM16_FETCH_Q
-#undef MM16_PARK_P
-#undef MM16_PARK_Q
-  if (KT & 1) multiply(lds);  // odd count: the last tile was parked in stage 0
+  if (KT & 1) {
+    multiply(lds, KT - 1, 1, with_fetch);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // no load outlives the wave
+  }
 
   // C fragment: element e of lane l is row (e/4)*8 + (l/32)*4 + e%4, column l%32.
 #pragma unroll
-  for (int mt = 0; mt < 4; mt++)
+  for (int mt = 0; mt < MM16_MT; mt++)
 #pragma unroll
-    for (int nt = 0; nt < 4; nt++)
+    for (int nt = 0; nt < MM16_NT; nt++)
 #pragma unroll
       for (int e = 0; e < 16; e++) {
-        const int row = bm + wm * 128 + mt * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
-        const int col = bn + wn * 128 + nt * 32 + (lane & 31);
+        const int row =
+            bm + wm * (MM16_MT * 32) + mt * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
+        const int col = bn + wn * (MM16_NT * 32) + nt * 32 + (lane & 31);
         Cb[(int64_t)row * N + col] = acc[mt][nt][e];
       }
 }
@@ -520,13 +533,13 @@ extern "C" int fa_matmul(fa_stream_t stream, fa_dtype in_t, const void *A, const
       static bool raised = false;
       if (!raised) { rc = raise_lds(matmul16_kernel<false>, 2 * MM16_STAGE_BYTES); raised = rc == 0; }
       if (rc) return rc;
-      hipLaunchKernelGGL((matmul16_kernel<false>), grid, dim3(MM_THREADS), 2 * MM16_STAGE_BYTES, st,
+      hipLaunchKernelGGL((matmul16_kernel<false>), grid, dim3(MM16_THREADS), 2 * MM16_STAGE_BYTES, st,
                          (const uint16_t *)A, (const uint16_t *)B, C, (int)M, (int)N, (int)K);
     } else {
       static bool raised = false;
       if (!raised) { rc = raise_lds(matmul16_kernel<true>, 2 * MM16_STAGE_BYTES); raised = rc == 0; }
       if (rc) return rc;
-      hipLaunchKernelGGL((matmul16_kernel<true>), grid, dim3(MM_THREADS), 2 * MM16_STAGE_BYTES, st,
+      hipLaunchKernelGGL((matmul16_kernel<true>), grid, dim3(MM16_THREADS), 2 * MM16_STAGE_BYTES, st,
                          (const uint16_t *)A, (const uint16_t *)B, C, (int)M, (int)N, (int)K);
     }
     return launch_status();
