@@ -149,6 +149,11 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="segscan_add_f32_2p26")
+    ap.add_argument("--prewarm-seconds", type=float, default=0.5,
+                    help="untimed passes before the W warm-up steps, until this much time has "
+                         "passed: the GPU leaves its idle power state only after a few hundred "
+                         "milliseconds of work, and a short MFMA run measured before that reads "
+                         "up to 40%% slow")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -167,6 +172,11 @@ def main() -> None:
     w = make_workload(args.workload, ctx)
     step = w["step"]
 
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < args.prewarm_seconds:
+        for _ in range(10):
+            step()
+        ctx.sync()
     for _ in range(args.warmup):
         step()
     ctx.sync()

@@ -15,7 +15,8 @@
 //     fence separates value and status.  8-byte element types use two such
 //     words (low and high half), accepted only when both carry the same status;
 //   * descriptors carry a launch epoch, so no kernel clears them between calls;
-//   * the look-back window is a full 64-lane wave.
+//   * the look-back window is a full 64-lane wave with several descriptors per
+//     lane.
 #include "dispatch.hip.h"
 
 namespace fa {
@@ -49,6 +50,11 @@ template <class T> constexpr int scan_rows() { return sizeof(T) == 4 ? FA_SCAN_R
 constexpr int SCAN_WAVES = FA_SCAN_WAVES;
 constexpr int SCAN_BLOCK = SCAN_WAVES * WAVE;
 static_assert(SCAN_WAVES >= 4, "the irregular reduction runs four searches on four waves");
+
+// Descriptors per lane in a look-back window.  Measured on 2^26 f32: 1 -> 99 us,
+// 2 -> 103 us, 4 -> 109 us; the nearest published prefix is normally within 64
+// tiles, and a wider window only adds loads to the round trip.
+constexpr int SCAN_LB = 1;
 
 constexpr uint32_t ST_X = 0;  // nothing published
 constexpr uint32_t ST_A = 1;  // aggregate of the tile
@@ -141,6 +147,8 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   __shared__ uint32_t s_pf;
   __shared__ uint32_t s_bits[MODE == MODE_SEGRED ? TILE / 32 : 1];
   __shared__ int64_t s_bounds[4];
+  // Flag bytes of the tile, one contiguous chunk per wave (segmented scans).
+  __shared__ __align__(16) uint32_t s_flags[(SEG && MODE == MODE_SCAN) ? TILE / 4 : 4];
   // MODE_SEGRED keeps the scanned tile in dynamic LDS (TILE elements).
   extern __shared__ __align__(16) unsigned char s_dyn[];
   T *s_vals = reinterpret_cast<T *>(s_dyn);
@@ -162,6 +170,31 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   const int64_t t0 = tile * TILE;
   const int64_t wbase = t0 + (int64_t)wave * WCHUNK;
 
+  // ---- flags: a wave's chunk has WCHUNK consecutive flag bytes.  They are
+  //      fetched with 16 bytes per lane (a few wide loads instead of one narrow
+  //      load per row) and handed to the lanes that own them through LDS.
+  bool flags_staged = false;
+  if constexpr (SEG && MODE == MODE_SCAN) {
+    constexpr int FB = WCHUNK / WAVE;  // flag bytes per lane
+    static_assert(FB == 8 || FB % 16 == 0, "flag bytes per lane: one 8-byte or whole 16-byte loads");
+    flags_staged = wbase + WCHUNK <= n && ((uintptr_t)flags & 15u) == 0;
+    if (flags_staged) {
+      unsigned char *wf = reinterpret_cast<unsigned char *>(s_flags) + wave * WCHUNK;
+      const uint8_t *src = flags + wbase;
+      if constexpr (FB == 8) {
+        using V2 = __attribute__((ext_vector_type(2))) uint32_t;
+        *reinterpret_cast<V2 *>(wf + lane * 8) =
+            __builtin_nontemporal_load(reinterpret_cast<const V2 *>(src + lane * 8));
+      } else {
+        using V4 = __attribute__((ext_vector_type(4))) uint32_t;
+#pragma unroll
+        for (int j = 0; j < FB / 16; j++)
+          *reinterpret_cast<V4 *>(wf + j * (WAVE * 16) + lane * 16) = __builtin_nontemporal_load(
+              reinterpret_cast<const V4 *>(src + j * (WAVE * 16) + lane * 16));
+      }
+    }
+  }
+
   // ---- load: row r of a wave is 64 lanes x 16 bytes of consecutive memory.
   T x[SCAN_ROWS][VEC];
   uint32_t fm[SCAN_ROWS];
@@ -174,14 +207,16 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
 #pragma unroll
       for (int e = 0; e < VEC; e++) x[r][e] = v.e[e];
       if constexpr (SEG && MODE == MODE_SCAN) {
-        if constexpr (VEC == 4) {
-          const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint32_t *>(flags + idx));
+        if (!flags_staged) {
+          if constexpr (VEC == 4) {
+            const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint32_t *>(flags + idx));
 #pragma unroll
-          for (int e = 0; e < 4; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
-        } else {
-          const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint16_t *>(flags + idx));
+            for (int e = 0; e < 4; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+          } else {
+            const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint16_t *>(flags + idx));
 #pragma unroll
-          for (int e = 0; e < 2; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+            for (int e = 0; e < 2; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+          }
         }
       }
     } else {
@@ -192,6 +227,21 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
         if constexpr (SEG && MODE == MODE_SCAN) {
           if (in && flags[idx + e] != 0) fm[r] |= 1u << e;
         }
+      }
+    }
+  }
+  if constexpr (SEG && MODE == MODE_SCAN) {
+    if (flags_staged) {
+      // Same wave wrote the chunk: LDS operations of a wave complete in order.
+      __builtin_amdgcn_wave_barrier();
+      const unsigned char *wf = reinterpret_cast<const unsigned char *>(s_flags) + wave * WCHUNK;
+#pragma unroll
+      for (int r = 0; r < SCAN_ROWS; r++) {
+        uint32_t w;
+        if constexpr (VEC == 4) w = *reinterpret_cast<const uint32_t *>(wf + (r * WAVE + lane) * 4);
+        else w = *reinterpret_cast<const uint16_t *>(wf + (r * WAVE + lane) * 2);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
       }
     }
   }
@@ -294,17 +344,46 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
       const bool self_contained = SEG && bt.f;
       if (lane == 0)
         desc_publish<T>(desc, tile, epoch, self_contained ? ST_P : ST_A, bt.f, bt.v);
-      int64_t j = tile - 1;
+      // The window is SCAN_LB descriptors per lane, 64 * SCAN_LB tiles.
+      int64_t j = tile - 1;  // newest tile of the window
       while (true) {
-        const int64_t idx = j - (WAVE - 1) + lane;
-        uint32_t st = ST_P, fl = 0u;
-        T v = Op::identity();
-        if (idx >= 0) {
-          while (!desc_read<T>(desc, idx, epoch, st, fl, v)) __builtin_amdgcn_s_sleep(1);
+        const int64_t first_idx = j - (int64_t)(WAVE * SCAN_LB - 1) + (int64_t)lane * SCAN_LB;
+        // Fold this lane's descriptors in tile order; one with a published
+        // prefix (or, in a segmented scan, a segment start) restarts the fold.
+        // All descriptors of the lane are requested before any is examined, so
+        // a window costs one round trip however many the lane holds.
+        uint32_t st[SCAN_LB], fl[SCAN_LB];
+        T v[SCAN_LB];
+        bool ok[SCAN_LB];
+#pragma unroll
+        for (int k = 0; k < SCAN_LB; k++) {
+          st[k] = ST_P;
+          fl[k] = 0u;
+          v[k] = Op::identity();
+          ok[k] = first_idx + k < 0 || desc_read<T>(desc, first_idx + k, epoch, st[k], fl[k], v[k]);
         }
-        const bool term = (st == ST_P) || (SEG && fl);
+#pragma unroll
+        for (int k = 0; k < SCAN_LB; k++) {
+          while (!ok[k]) {
+            __builtin_amdgcn_s_sleep(1);
+            ok[k] = desc_read<T>(desc, first_idx + k, epoch, st[k], fl[k], v[k]);
+          }
+        }
+        Pair part = {Op::identity(), 0u};
+        bool term = false;
+#pragma unroll
+        for (int k = 0; k < SCAN_LB; k++) {
+          const Pair e = {v[k], SEG ? fl[k] : 0u};
+          if (st[k] == ST_P) {
+            part = e;
+          } else {
+            if constexpr (SEG) part = seg_apply<T, Op>(part, e);
+            else part.v = Op::apply(part.v, v[k]);
+          }
+          term = term || (st[k] == ST_P) || (SEG && fl[k]);
+        }
         const uint64_t mask = __ballot(term);
-        Pair mine = {v, SEG ? fl : 0u};
+        Pair mine = part;
         if (mask) {
           const int first = 63 - __builtin_clzll(mask);
           if (lane < first) {
@@ -323,7 +402,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
           acc.v = Op::apply(win.v, acc.v);
         }
         if (mask) break;
-        j -= WAVE;
+        j -= WAVE * SCAN_LB;
       }
       if (lane == 0 && !self_contained) {
         Pair inc;
