@@ -52,36 +52,85 @@ static inline int rs_prepare(hipStream_t st, const RsScratch &sc) {
   return fa_replicate((fa_stream_t)st, 4, sc.lookback, (int64_t)(sc.lookback_bytes / 4), 0);
 }
 
-// counts[d][tile] = number of keys of the tile whose digit is d.
+// counts[d][tile] = number of keys of the tile whose digit is d.  A block
+// counts RS_HIST_TILES consecutive tiles, so that what it writes for a digit
+// is a run of RS_HIST_TILES counts (one 32-byte store) instead of single
+// 4-byte stores 4*num_tiles bytes apart, and the keys of the next tile are in
+// flight while the current one is counted.
+constexpr int RS_HIST_TILES = 8;
+
 template <class K, class DigitFn>
 __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__ keys, int64_t n,
                                                            DigitFn fn, int pass, uint32_t *counts,
                                                            int64_t num_tiles) {
   constexpr int VEC = 16 / sizeof(K);
+  constexpr int ROWS = RS_KPT / VEC;
   __shared__ uint32_t h[RS_WAVES][RS_RADIX];
   for (int i = threadIdx.x; i < RS_WAVES * RS_RADIX; i += RS_BLOCK) (&h[0][0])[i] = 0u;
-  __syncthreads();
   const int wave = threadIdx.x / WAVE;
-  const int64_t base = (int64_t)blockIdx.x * RS_TILE;
-  const int64_t end = base + RS_TILE < n ? base + RS_TILE : n;
+  const int64_t tile0 = (int64_t)blockIdx.x * RS_HIST_TILES;
+  const int tiles_here =
+      (int)(num_tiles - tile0 < RS_HIST_TILES ? num_tiles - tile0 : RS_HIST_TILES);
+  uint32_t c[RS_HIST_TILES];  // thread d < 256: count of digit d per tile
 #pragma unroll
-  for (int r = 0; r < RS_KPT / VEC; r++) {
-    const int64_t idx = base + ((int64_t)r * RS_BLOCK + threadIdx.x) * VEC;
-    if (idx + VEC <= end) {
-      const Vec16<K> v = load_vec16(keys + idx);
+  for (int t = 0; t < RS_HIST_TILES; t++) c[t] = 0u;
+
+  // Full tiles are fetched one tile ahead; the last tile of the input may be
+  // ragged and is read element-wise.
+  Vec16<K> cur[ROWS], nxt[ROWS];
+  auto full = [&](int t) { return t < tiles_here && (tile0 + t + 1) * RS_TILE <= n; };
+  auto fetch = [&](int t, Vec16<K>(&v)[ROWS]) {
+    const int64_t base = (tile0 + t) * RS_TILE;
 #pragma unroll
-      for (int e = 0; e < VEC; e++) atomicAdd(&h[wave][fn(v.e[e], pass)], 1u);
-    } else {
-      for (int e = 0; e < VEC; e++)
-        if (idx + e < end) atomicAdd(&h[wave][fn(keys[idx + e], pass)], 1u);
+    for (int r = 0; r < ROWS; r++)
+      v[r] = load_vec16(keys + base + ((int64_t)r * RS_BLOCK + threadIdx.x) * VEC);
+  };
+  if (full(0)) fetch(0, cur);
+  __syncthreads();
+#pragma unroll
+  for (int t = 0; t < RS_HIST_TILES; t++) {
+    if (t < tiles_here) {  // uniform
+      const bool is_full = full(t);
+      if (full(t + 1)) fetch(t + 1, nxt);
+      if (is_full) {
+#pragma unroll
+        for (int r = 0; r < ROWS; r++)
+#pragma unroll
+          for (int e = 0; e < VEC; e++) atomicAdd(&h[wave][fn(cur[r].e[e], pass)], 1u);
+      } else {
+        const int64_t base = (tile0 + t) * RS_TILE;
+        for (int r = 0; r < ROWS; r++)
+          for (int e = 0; e < VEC; e++) {
+            const int64_t idx = base + ((int64_t)r * RS_BLOCK + threadIdx.x) * VEC + e;
+            if (idx < n) atomicAdd(&h[wave][fn(keys[idx], pass)], 1u);
+          }
+      }
+      __syncthreads();
+      if (threadIdx.x < RS_RADIX) {  // sum the waves' counters and clear them
+        uint32_t sum = 0;
+#pragma unroll
+        for (int w = 0; w < RS_WAVES; w++) {
+          sum += h[w][threadIdx.x];
+          h[w][threadIdx.x] = 0u;
+        }
+        c[t] = sum;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < ROWS; r++) cur[r] = nxt[r];
     }
   }
-  __syncthreads();
   if (threadIdx.x < RS_RADIX) {
-    uint32_t c = 0;
+    uint32_t *dst = counts + (int64_t)threadIdx.x * num_tiles + tile0;
+    if (tiles_here == RS_HIST_TILES && (num_tiles & 3) == 0) {
+      static_assert(RS_HIST_TILES == 8, "two 16-byte stores per digit");
+      reinterpret_cast<uint4 *>(dst)[0] = make_uint4(c[0], c[1], c[2], c[3]);
+      reinterpret_cast<uint4 *>(dst)[1] = make_uint4(c[4], c[5], c[6], c[7]);
+    } else {
 #pragma unroll
-    for (int w = 0; w < RS_WAVES; w++) c += h[w][threadIdx.x];
-    counts[(int64_t)threadIdx.x * num_tiles + blockIdx.x] = c;
+      for (int t = 0; t < RS_HIST_TILES; t++)
+        if (t < tiles_here) dst[t] = c[t];
+    }
   }
 }
 
@@ -256,7 +305,8 @@ static int rs_pass(hipStream_t st, const K *kin, K *kout, const void *vin, void 
     if (e != hipSuccess) return (int)e;
     raised = true;
   }
-  hipLaunchKernelGGL((rs_hist_kernel<K, DigitFn>), dim3((unsigned)sc.tiles), dim3(RS_BLOCK), 0, st,
+  hipLaunchKernelGGL((rs_hist_kernel<K, DigitFn>),
+                     dim3((unsigned)ceil_div(sc.tiles, (int64_t)RS_HIST_TILES)), dim3(RS_BLOCK), 0, st,
                      kin, n, fn, pass, sc.counts, sc.tiles);
   int rc = launch_status();
   if (rc != 0) return rc;
