@@ -143,6 +143,20 @@ def make_workload(name: str, ctx):
     return w
 
 
+# HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same
+# counters on a 256 MiB copy); the runs and their commands are in profiles/<kernel>_<workload>.txt.
+MEASURED_TRAFFIC_BYTES = {
+    "segscan_add_f32_2p26": 606.0e6,
+    "scan_add_f32_2p26": 539.3e6,
+    "reduce_add_f32_2p26": 268.5e6,
+    "segred_add_f32_2p26": 275.1e6,
+    "hist_add_i32_H256_uniform_2p27": 1074.2e6,
+    "hist_add_i32_H65536_uniform_2p27": 1107.6e6,
+    "hist_add_i32_H4194304_uniform_2p27": 4229.0e6,
+    "sort_u32_2p26": 4088.4e6,
+}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -245,7 +259,8 @@ def main() -> None:
         "config": {"workload": w["describe"], "name": args.workload,
                    "algorithmic_bytes_per_step" if w["bound"] == "hbm" else "flop_per_step": work},
         "roofline": {"bound": w["bound"], "achieved": round(achieved, 3), "peak": peak,
-                     "unit": unit, "frac": round(achieved / peak, 4), "traffic": None,
+                     "unit": unit, "frac": round(achieved / peak, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "kernel": w["kernel"], "kernel_us": round(kernel_us, 3)},
         "cpu_baseline": cpu,
     }
