@@ -1,5 +1,4 @@
-// SegScan for gfx950: single-pass scan with decoupled look-back, plus the
-// irregular segmented reduction that shares its machinery.
+// SegScan for gfx950: single-pass scan with decoupled look-back.
 //
 // What is computed follows src/Futhark/CodeGen/ImpGen/GPU/SegScan/SinglePass.hs
 // (dynamic tile ids :443-461, tile aggregate/prefix publication with status
@@ -49,7 +48,6 @@ namespace fa {
 template <class T> constexpr int scan_rows() { return sizeof(T) == 4 ? FA_SCAN_ROWS4 : FA_SCAN_ROWS8; }
 constexpr int SCAN_WAVES = FA_SCAN_WAVES;
 constexpr int SCAN_BLOCK = SCAN_WAVES * WAVE;
-static_assert(SCAN_WAVES >= 4, "the irregular reduction runs four searches on four waves");
 
 // Descriptors per lane in a look-back window.  Measured on 2^26 f32: 1 -> 99 us,
 // 2 -> 103 us, 4 -> 109 us; the nearest published prefix is normally within 64
@@ -104,36 +102,11 @@ __device__ __forceinline__ bool desc_read(const uint64_t *desc, int64_t tile, ui
   return true;
 }
 
-// First index i in [0,m] for which pred(i) holds, pred monotone (false..true);
-// a 64-ary search run by one whole wave.
-template <class Pred>
-__device__ __forceinline__ int64_t wave_search_first(int64_t m, int lane, Pred pred) {
-  int64_t lo = 0, hi = m;
-  while (hi > lo) {
-    const int64_t span = hi - lo;
-    const int64_t step = (span + WAVE - 1) / WAVE;
-    const int64_t p = lo + (int64_t)lane * step;
-    const bool t = (p < hi) ? pred(p) : true;
-    const uint64_t mask = __ballot(t);
-    const int L = mask ? __builtin_ctzll(mask) : WAVE;
-    if (L == 0) return lo;
-    const int64_t nhi = lo + (int64_t)L * step;
-    lo = lo + (int64_t)(L - 1) * step + 1;
-    hi = nhi < hi ? nhi : hi;
-  }
-  return lo;
-}
-
-enum { MODE_SCAN = 0, MODE_SEGRED = 1 };
-
-// MODE_SCAN  : out[n], flags optional (SEG), EXCL selects the exclusive form.
-// MODE_SEGRED: flags are derived from `offsets`; out[m] receives the scanned
-//              value at the last element of each segment (ne for empty ones).
-template <class T, class Op, bool SEG, bool EXCL, int MODE>
+// out[n]; flags optional (SEG); EXCL selects the exclusive form.
+template <class T, class Op, bool SEG, bool EXCL>
 __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
     const T *__restrict__ xs, const uint8_t *__restrict__ flags, int64_t n, T *__restrict__ out,
-    uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles,
-    const int64_t *__restrict__ offsets, const int64_t *__restrict__ lens, int64_t m) {
+    uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles) {
   constexpr int VEC = Vec16<T>::N;
   constexpr int SCAN_ROWS = scan_rows<T>();
   constexpr int WCHUNK = SCAN_ROWS * WAVE * VEC;
@@ -145,22 +118,14 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   __shared__ uint32_t s_wf[SCAN_WAVES];
   __shared__ T s_pv;
   __shared__ uint32_t s_pf;
-  __shared__ uint32_t s_bits[MODE == MODE_SEGRED ? TILE / 32 : 1];
-  __shared__ int64_t s_bounds[4];
   // Flag bytes of the tile, one contiguous chunk per wave (segmented scans).
-  __shared__ __align__(16) uint32_t s_flags[(SEG && MODE == MODE_SCAN) ? TILE / 4 : 4];
-  // MODE_SEGRED keeps the scanned tile in dynamic LDS (TILE elements).
-  extern __shared__ __align__(16) unsigned char s_dyn[];
-  T *s_vals = reinterpret_cast<T *>(s_dyn);
+  __shared__ __align__(16) uint32_t s_flags[SEG ? TILE / 4 : 4];
 
   if (threadIdx.x == 0) {
     const uint32_t t = atomicAdd(ticket, 1u);
     s_tile = (int64_t)t;
     // The last ticket of this launch has been drawn: rearm for the next one.
     if ((int64_t)t == num_tiles - 1) st_relaxed_u32(ticket, 0u);
-  }
-  if constexpr (MODE == MODE_SEGRED) {
-    for (int i = threadIdx.x; i < TILE / 32; i += SCAN_BLOCK) s_bits[i] = 0u;
   }
   __syncthreads();
   // Tile and wave numbers are the same in all lanes; say so to the compiler.
@@ -174,7 +139,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   //      fetched with 16 bytes per lane (a few wide loads instead of one narrow
   //      load per row) and handed to the lanes that own them through LDS.
   bool flags_staged = false;
-  if constexpr (SEG && MODE == MODE_SCAN) {
+  if constexpr (SEG) {
     constexpr int FB = WCHUNK / WAVE;  // flag bytes per lane
     static_assert(FB == 8 || FB % 16 == 0, "flag bytes per lane: one 8-byte or whole 16-byte loads");
     flags_staged = wbase + WCHUNK <= n && ((uintptr_t)flags & 15u) == 0;
@@ -206,7 +171,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
       Vec16<T> v = FA_SCAN_LOAD(xs + idx);
 #pragma unroll
       for (int e = 0; e < VEC; e++) x[r][e] = v.e[e];
-      if constexpr (SEG && MODE == MODE_SCAN) {
+      if constexpr (SEG) {
         if (!flags_staged) {
           if constexpr (VEC == 4) {
             const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint32_t *>(flags + idx));
@@ -224,13 +189,13 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
       for (int e = 0; e < VEC; e++) {
         const bool in = idx + e < n;
         x[r][e] = in ? xs[idx + e] : Op::identity();
-        if constexpr (SEG && MODE == MODE_SCAN) {
+        if constexpr (SEG) {
           if (in && flags[idx + e] != 0) fm[r] |= 1u << e;
         }
       }
     }
   }
-  if constexpr (SEG && MODE == MODE_SCAN) {
+  if constexpr (SEG) {
     if (flags_staged) {
       // Same wave wrote the chunk: LDS operations of a wave complete in order.
       __builtin_amdgcn_wave_barrier();
@@ -243,42 +208,6 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
 #pragma unroll
         for (int e = 0; e < VEC; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
       }
-    }
-  }
-
-  // ---- irregular reduction: find the segments that start / end in this tile
-  //      and turn their start offsets into flag bits.
-  int64_t e_first = 0, e_last = 0;
-  if constexpr (MODE == MODE_SEGRED) {
-    const int64_t t1 = (t0 + TILE < n) ? t0 + TILE : n;
-    int64_t r;
-    if (wave == 0) {
-      r = wave_search_first(m, lane, [&](int64_t i) { return offsets[i] >= t0; });
-    } else if (wave == 1) {
-      r = wave_search_first(m, lane, [&](int64_t i) { return offsets[i] >= t1; });
-    } else if (wave == 2) {
-      r = (tile == 0) ? 0
-                      : wave_search_first(
-                            m, lane, [&](int64_t i) { return offsets[i] + lens[i] > t0; });
-    } else if (wave == 3) {
-      r = wave_search_first(m, lane, [&](int64_t i) { return offsets[i] + lens[i] > t1; });
-    } else {
-      r = 0;
-    }
-    if (lane == 0 && wave < 4) s_bounds[wave] = r;
-    __syncthreads();
-    const int64_t s_first = s_bounds[0], s_last = s_bounds[1];
-    e_first = s_bounds[2];
-    e_last = s_bounds[3];
-    for (int64_t i = s_first + threadIdx.x; i < s_last; i += SCAN_BLOCK) {
-      const int64_t p = offsets[i] - t0;
-      if ((uint64_t)p < (uint64_t)TILE) atomicOr(&s_bits[p >> 5], 1u << (p & 31));
-    }
-    __syncthreads();
-#pragma unroll
-    for (int r2 = 0; r2 < SCAN_ROWS; r2++) {
-      const int p = wave * WCHUNK + (r2 * WAVE + lane) * VEC;
-      fm[r2] = (s_bits[p >> 5] >> (p & 31)) & ((1u << VEC) - 1u);
     }
   }
 
@@ -442,28 +371,13 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
       prev = incl;
     }
 
-    if constexpr (MODE == MODE_SCAN) {
-      const int64_t idx = wbase + (int64_t)(r * WAVE + lane) * VEC;
-      if (idx + VEC <= n) {
-        FA_SCAN_STORE(out + idx, o);
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; e++)
-          if (idx + e < n) out[idx + e] = o.e[e];
-      }
+    const int64_t idx = wbase + (int64_t)(r * WAVE + lane) * VEC;
+    if (idx + VEC <= n) {
+      FA_SCAN_STORE(out + idx, o);
     } else {
-      const int p = wave * WCHUNK + (r * WAVE + lane) * VEC;
 #pragma unroll
-      for (int e = 0; e < VEC; e++) s_vals[p + e] = o.e[e];
-    }
-  }
-
-  if constexpr (MODE == MODE_SEGRED) {
-    __syncthreads();
-    for (int64_t i = e_first + threadIdx.x; i < e_last; i += SCAN_BLOCK) {
-      const int64_t len = lens[i];
-      const int64_t p = offsets[i] + len - 1 - t0;
-      out[i] = (len == 0 || (uint64_t)p >= (uint64_t)TILE) ? Op::identity() : s_vals[p];
+      for (int e = 0; e < VEC; e++)
+        if (idx + e < n) out[idx + e] = o.e[e];
     }
   }
 }
@@ -487,9 +401,8 @@ static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int6
   uint64_t *desc = (uint64_t *)((char *)scratch + SCAN_HEADER_BYTES);
   const dim3 grid((unsigned)tiles), block(SCAN_BLOCK);
 #define FA_LAUNCH(SEGV, EXV)                                                              \
-  hipLaunchKernelGGL((segscan_kernel<T, Op, SEGV, EXV, MODE_SCAN>), grid, block, 0, s,   \
-                     (const T *)xs, flags, n, (T *)out, ticket, desc, epoch, tiles,       \
-                     (const int64_t *)nullptr, (const int64_t *)nullptr, (int64_t)0)
+  hipLaunchKernelGGL((segscan_kernel<T, Op, SEGV, EXV>), grid, block, 0, s, (const T *)xs, \
+                     flags, n, (T *)out, ticket, desc, epoch, tiles)
   if (flags) {
     if (exclusive) FA_LAUNCH(true, true);
     else FA_LAUNCH(true, false);
@@ -498,49 +411,6 @@ static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int6
     else FA_LAUNCH(false, false);
   }
 #undef FA_LAUNCH
-  return launch_status();
-}
-
-template <class T>
-__global__ void fill_kernel(T *dst, int64_t n, T v) {
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += (int64_t)gridDim.x * blockDim.x)
-    dst[i] = v;
-}
-
-template <class T, class Op>
-static int launch_segred_irregular(hipStream_t s, const void *vs, int64_t n,
-                                   const int64_t *offsets, const int64_t *lens, int64_t m,
-                                   void *out, void *scratch, size_t scratch_bytes,
-                                   uint32_t epoch) {
-  if (m == 0) return 0;
-  if (n == 0) {
-    // Every segment is empty.
-    int grid = (int)(ceil_div(m, 256) < 4096 ? ceil_div(m, 256) : 4096);
-    hipLaunchKernelGGL((fill_kernel<T>), dim3(grid), dim3(256), 0, s, (T *)out, m,
-                       Op::identity());
-    return launch_status();
-  }
-  const int64_t tiles = scan_num_tiles<T>(n);
-  if (scratch_bytes < SCAN_HEADER_BYTES + (size_t)tiles * SCAN_DESC_BYTES) return FA_ESCRATCH;
-  if (!is_aligned(vs, 16) || !is_aligned(scratch, 16) || !is_aligned(offsets, 8) ||
-      !is_aligned(lens, 8))
-    return FA_EALIGN;
-  if (tiles > INT32_MAX) return FA_EINVAL;
-  uint32_t *ticket = (uint32_t *)scratch;
-  uint64_t *desc = (uint64_t *)((char *)scratch + SCAN_HEADER_BYTES);
-  auto kernel = segscan_kernel<T, Op, true, false, MODE_SEGRED>;
-  const size_t lds = (size_t)scan_tile_elems<T>() * sizeof(T);
-  static bool lds_limit_raised = false;  // per instantiation
-  if (!lds_limit_raised) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    lds_limit_raised = true;
-  }
-  hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(SCAN_BLOCK), lds, s, (const T *)vs,
-                     (const uint8_t *)nullptr, n, (T *)out, ticket, desc, epoch, tiles, offsets,
-                     lens, m);
   return launch_status();
 }
 
@@ -563,18 +433,5 @@ extern "C" int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op, const void *
   if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xs, flags, n, exclusive, out, scratch,
-                      scratch_bytes, epoch);
-}
-
-extern "C" int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op, const void *vs,
-                                   int64_t n, const int64_t *offsets, const int64_t *lens,
-                                   int64_t m, void *out, void *scratch, size_t scratch_bytes,
-                                   uint32_t epoch) {
-  if (n < 0 || m < 0 || (m > 0 && (offsets == nullptr || lens == nullptr || out == nullptr)) ||
-      (n > 0 && m > 0 && (vs == nullptr || scratch == nullptr)))
-    return FA_EINVAL;
-  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
-  FA_DISPATCH_TYPE_OP(launch_segred_irregular, t, op, s, vs, n, offsets, lens, m, out, scratch,
                       scratch_bytes, epoch);
 }

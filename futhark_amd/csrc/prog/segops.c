@@ -266,19 +266,24 @@ static int do_segred(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
                      const char *entry) {
   const int64_t m = offsets->shape[0], n = vs->shape[0];
   if (lens->shape[0] != m) return bad_sizes(ctx, entry);
-  uint32_t epoch = 0;
-  void *scratch = rts_scan_scratch(ctx, fa_segscan_scratch_bytes(t, n), &epoch);
-  if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
   struct fut_array *res = out_array(ctx, m * (int64_t)es, 1, &m, "segred.out");
   if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
-  struct rts_event *ev = rts_kernel_begin(
-      ctx, "segred_irregular",
-      rts_msgprintf("{\"n\":%lld,\"segments\":%lld}", (long long)n, (long long)m));
-  int code = fa_segred_irregular(ctx->stream, t, op, vs->mem.mem, n,
-                                 (const int64_t *)offsets->mem.mem,
-                                 (const int64_t *)lens->mem.mem, m, res->mem.mem, scratch,
-                                 ctx->scan_scratch_bytes, epoch);
-  int err = rts_kernel_end(ctx, ev, "segred_irregular", code);
+  /* Plain workspace from the pool; not the look-back scratch of the scans,
+     whose contents must stay valid descriptors. */
+  struct memblock_device scratch = {0};
+  int err = rts_memblock_alloc(ctx, &scratch, (int64_t)fa_segred_irregular_scratch_bytes(t, n),
+                               "segred.scratch");
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "segred_irregular",
+        rts_msgprintf("{\"n\":%lld,\"segments\":%lld}", (long long)n, (long long)m));
+    int code = fa_segred_irregular(ctx->stream, t, op, vs->mem.mem, n,
+                                   (const int64_t *)offsets->mem.mem,
+                                   (const int64_t *)lens->mem.mem, m, res->mem.mem, scratch.mem,
+                                   (size_t)scratch.size);
+    err = rts_kernel_end(ctx, ev, "segred_irregular", code);
+  }
+  rts_memblock_unref(ctx, &scratch, "segred.scratch");
   if (err != 0) {
     drop_array(ctx, res);
     return err;

@@ -94,8 +94,8 @@ int fa_segred_regular(fa_stream_t stream, fa_dtype t, fa_op op,
  *   unsegmented case).
  *
  * scratch protocol: the buffer must have been zero-filled once when it was
- * allocated; after that it may be passed to any number of fa_segscan /
- * fa_segred_irregular calls provided `epoch` is strictly larger on every call
+ * allocated; after that it may be passed to any number of fa_segscan calls
+ * provided `epoch` is strictly larger on every call
  * (1 <= epoch < 2^28; zero-fill again before wrapping).  Tile descriptors
  * carry the epoch, so no per-call clearing kernel is needed. */
 size_t fa_segscan_scratch_bytes(fa_dtype t, int64_t n);
@@ -105,13 +105,16 @@ int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op,
 
 /* Irregular segmented reduction (Pass/Flatten/Builtins.hs:582-602):
  *   out[i] = lens[i] == 0 ? ne : segscan(flags-from-offsets, vs)[offsets[i]+lens[i]-1]
- * computed without materialising the scan.  offsets must be non-decreasing,
- * within [0,n].  Same scratch protocol as fa_segscan. */
+ * computed without materialising the scan.  Segments must be in order and
+ * disjoint (offsets non-decreasing, offsets[i] + lens[i] <= offsets[i+1], all
+ * within [0,n]); elements between segments are ignored.  `scratch` is plain
+ * workspace of fa_segred_irregular_scratch_bytes(t, n) bytes, 16-byte aligned;
+ * its contents on entry do not matter. */
+size_t fa_segred_irregular_scratch_bytes(fa_dtype t, int64_t n);
 int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op,
                         const void *vs, int64_t n,
                         const int64_t *offsets, const int64_t *lens, int64_t m,
-                        void *out, void *scratch, size_t scratch_bytes,
-                        uint32_t epoch);
+                        void *out, void *scratch, size_t scratch_bytes);
 
 /* ----------------------------------------------------------------- SegHist
  * `reduce_by_index dest op ne is vs` (prelude/soacs.fut:132-146): for every i

@@ -117,6 +117,27 @@ def test_segred_irregular(ctx, t, op):
                 assert np.array_equal(got, oracle.segred(op, t, offsets, lens, xs)), (n, mean)
 
 
+def test_segred_gaps_and_unit_segments(ctx):
+    """Elements between segments are ignored; segments of one element; a segment
+    that spans hundreds of tiles next to short ones."""
+    rng = np.random.default_rng(7)
+    n = 3_000_017
+    xs = rng.integers(-1000, 1000, n).astype(np.int64)
+    # unit segments with gaps of varying width, then one very long segment, then a tail gap
+    starts = np.cumsum(rng.integers(1, 9, 20000)).astype(np.int64)
+    lens = np.ones_like(starts)
+    long_start = int(starts[-1]) + 5
+    offsets = np.concatenate([starts, [long_start, n - 40]]).astype(np.int64)
+    lens = np.concatenate([lens, [n - 100 - long_start, 30]]).astype(np.int64)
+    o, l, v = ctx.new("i64_1d", offsets), ctx.new("i64_1d", lens), ctx.new("i64_1d", xs)
+    for op in ("add", "max"):
+        out = ctx.call(f"segred_{op}_i64", ["i64_1d"], o, l, v)
+        assert np.array_equal(out.values(), oracle.segred(op, "i64", offsets, lens, xs)), op
+        out.free()
+    for h in (o, l, v):
+        h.free()
+
+
 def test_segred_all_empty_and_no_segments(ctx):
     o = ctx.new("i64_1d", np.zeros(4, np.int64)); l = ctx.new("i64_1d", np.zeros(4, np.int64))
     v = ctx.new("f32_1d", np.zeros(0, np.float32))
