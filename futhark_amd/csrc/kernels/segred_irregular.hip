@@ -7,8 +7,8 @@
 // reference materialises the whole scan; here nothing of it reaches memory, and
 // no block waits for another one:
 //   1. segred_bounds_kernel finds, for every tile boundary, the first segment
-//      that starts at or after it and the first that ends after it (one 64-ary
-//      wave search each; segments are in order, so both are monotone);
+//      that starts at or after it and the first that ends after it (every
+//      segment marks the boundaries it owns; segments are in order);
 //   2. segred_tiles_kernel scans every 16 KiB tile on its own (start flags from
 //      `offsets` as an LDS bitmap, DPP wave scans, scanned tile kept in LDS),
 //      writes the result of every segment that lies inside the tile, and leaves
@@ -39,49 +39,72 @@ struct SriTileRec {
   uint64_t has_start;  // nonzero if a segment starts in the tile
 };
 
-// First index i in [0,m] for which pred(i) holds, pred monotone (false..true);
-// a 64-ary search run by one whole wave.
-template <class Pred>
-__device__ __forceinline__ int64_t sri_wave_search_first(int64_t m, int lane, Pred pred) {
-  int64_t lo = 0, hi = m;
-  while (hi > lo) {
-    const int64_t span = hi - lo;
-    const int64_t step = (span + WAVE - 1) / WAVE;
-    const int64_t p = lo + (int64_t)lane * step;
-    const bool t = (p < hi) ? pred(p) : true;
-    const uint64_t mask = __ballot(t);
-    const int L = mask ? __builtin_ctzll(mask) : WAVE;
-    if (L == 0) return lo;
-    const int64_t nhi = lo + (int64_t)L * step;
-    lo = lo + (int64_t)(L - 1) * step + 1;
-    hi = nhi < hi ? nhi : hi;
-  }
-  return lo;
-}
-
 // bounds[2t]   = first segment with offsets[i] >= p_t,
 // bounds[2t+1] = first segment with offsets[i] + lens[i] > p_t (0 for t == 0, so
-//                that empty segments at position 0 belong to tile 0),
+//                that empty segments at position 0 belong to tile 0; m for the
+//                last boundary),
 // for p_t = min(t * tile_elems, n), t = 0..num_tiles.
+//
+// Computed from the segments' side: thread i (0..m, m standing for a sentinel
+// segment at infinity) owns the boundaries between its predecessor's start
+// (end) and its own, and writes its index there.  Starts and ends are
+// non-decreasing, so every boundary has exactly one owner.  A segment that
+// spans many tiles hands its boundaries to the whole wave.
+__device__ __forceinline__ void sri_mark(int64_t *bounds, int which, int64_t t_lo, int64_t t_hi,
+                                         int64_t value, int lane) {
+  const int64_t count = t_hi - t_lo + 1;
+  if (count > 0 && count <= 4) {
+    for (int64_t t = t_lo; t <= t_hi; t++) bounds[2 * t + which] = value;
+  }
+  uint64_t wide = __ballot(count > 4);
+  while (wide) {
+    const int src = __builtin_ctzll(wide);
+    wide &= wide - 1;
+    const int64_t lo = read_lane(t_lo, src), hi = read_lane(t_hi, src);
+    const int64_t v = read_lane(value, src);
+    for (int64_t t = lo + lane; t <= hi; t += WAVE) bounds[2 * t + which] = v;
+  }
+}
+
 static __global__ __launch_bounds__(256) void segred_bounds_kernel(
     const int64_t *__restrict__ offsets, const int64_t *__restrict__ lens, int64_t m, int64_t n,
     int64_t tile_elems, int64_t num_tiles, int64_t *__restrict__ bounds) {
   const int lane = lane_id();
-  const int64_t job = (int64_t)blockIdx.x * (256 / WAVE) + threadIdx.x / WAVE;
-  if (job >= 2 * (num_tiles + 1)) return;
-  const int64_t t = job >> 1;
-  const int64_t p = t * tile_elems < n ? t * tile_elems : n;
-  int64_t r;
-  if ((job & 1) == 0) {
-    r = sri_wave_search_first(m, lane, [&](int64_t i) { return offsets[i] >= p; });
-  } else if (t == 0) {
-    r = 0;
-  } else if (t == num_tiles) {
-    r = m;  // every remaining segment (empty ones at position n included) ends by n
-  } else {
-    r = sri_wave_search_first(m, lane, [&](int64_t i) { return offsets[i] + lens[i] > p; });
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const bool live = i <= m;  // whole waves stay in the loops of sri_mark
+  const int64_t inf = INT64_MAX / 2;
+  int64_t s_prev = -1, s_here = inf, e_prev = 0, e_here = inf;
+  if (live) {
+    if (i > 0) {
+      s_prev = offsets[i - 1];
+      e_prev = s_prev + lens[i - 1];
+    }
+    if (i < m) {
+      s_here = offsets[i];
+      e_here = s_here + lens[i];
+    }
   }
-  if (lane == 0) bounds[job] = r;
+  // Interior boundaries are t = 0..num_tiles-1 at p_t = t * tile_elems.
+  // Starts: s_prev < p_t <= s_here.
+  {
+    const int64_t t_lo = s_prev < 0 ? 0 : s_prev / tile_elems + 1;
+    int64_t t_hi = s_here / tile_elems;
+    if (t_hi > num_tiles - 1) t_hi = num_tiles - 1;
+    sri_mark(bounds, 0, live ? t_lo : 1, live ? t_hi : 0, i, lane);
+    if (live && s_prev < n && n <= s_here) bounds[2 * num_tiles] = i;  // p = n
+  }
+  // Ends: e_prev <= p_t < e_here, t >= 1.
+  {
+    int64_t t_lo = (e_prev + tile_elems - 1) / tile_elems;
+    if (t_lo < 1) t_lo = 1;
+    int64_t t_hi = e_here >= 1 ? (e_here - 1) / tile_elems : -1;
+    if (t_hi > num_tiles - 1) t_hi = num_tiles - 1;
+    sri_mark(bounds, 1, live ? t_lo : 1, live ? t_hi : 0, i, lane);
+    if (i == 0) {
+      bounds[1] = 0;
+      bounds[2 * num_tiles + 1] = m;
+    }
+  }
 }
 
 template <class T> __device__ __forceinline__ uint64_t sri_bits(T v) {
@@ -293,8 +316,7 @@ static int launch_segred_irregular(hipStream_t s, const void *vs, int64_t n,
   if (tiles > INT32_MAX) return FA_EINVAL;
   int64_t *bounds = (int64_t *)scratch;
   SriTileRec *recs = (SriTileRec *)((char *)scratch + (size_t)(tiles + 1) * 16);
-  const int64_t jobs = 2 * (tiles + 1);
-  hipLaunchKernelGGL(segred_bounds_kernel, dim3((unsigned)ceil_div(jobs, (int64_t)(256 / WAVE))),
+  hipLaunchKernelGGL(segred_bounds_kernel, dim3((unsigned)ceil_div(m + 1, (int64_t)256)),
                      dim3(256), 0, s, offsets, lens, m, n, tile_elems, tiles, bounds);
   hipLaunchKernelGGL((segred_tiles_kernel<T, Op>), dim3((unsigned)tiles), dim3(SRI_BLOCK), 0, s,
                      (const T *)vs, n, offsets, lens, (const int64_t *)bounds, (T *)out, recs);
