@@ -143,6 +143,44 @@ def make_workload(name: str, ctx):
     return w
 
 
+def run_via_server(name: str, steps: int, warmup: int):
+    """`futhark bench` protocol: restore inputs once, then time `call` (entry + sync, as the
+    server measures it: rts/c/server.h:386-391) with the result freed between runs."""
+    import tempfile
+    from futhark_amd import datagen as dg
+    from futhark_amd import values as fv
+    from futhark_amd.server import Server
+
+    kind, op, t, sz = name.split("_")
+    n = 1 << int(sz[2:])
+    if kind in ("segscan", "segred"):
+        offsets, lens, flags = dg.segments(32, n, 1024)
+        xs = dg.uniform_f32(33, n) if t == "f32" else dg.uniform_int(34, n, -(1 << 20), 1 << 20, np.int64)
+        if kind == "segscan":
+            arrays, types = [flags, xs], ["[]u8", f"[]{t}"]
+        else:
+            arrays, types = [offsets, lens, xs], ["[]i64", "[]i64", f"[]{t}"]
+    elif kind in ("scan", "reduce"):
+        xs = dg.uniform_f32(17, n) if t == "f32" else dg.uniform_int(16, n, -1000, 1000)
+        arrays, types = [xs], [f"[]{t}"]
+    else:
+        raise SystemExit("--via-server covers scan/reduce/segscan/segred workloads")
+    names = [f"in{i}" for i in range(len(arrays))]
+    with tempfile.TemporaryDirectory() as d, Server() as srv:
+        path = f"{d}/inputs.bin"
+        fv.write_binary(path, arrays)
+        srv.cmd("restore", path, *[w for pair in zip(names, types) for w in pair])
+        runtimes = []
+        for i in range(warmup + steps):
+            us = srv.call(f"{kind}_{op}_{t}", "out", *names)
+            srv.cmd("free", "out")
+            if i >= warmup:
+                runtimes.append(us)
+    return {"entry": f"{kind}_{op}_{t}", "runs": steps,
+            "runtime_us_mean": round(float(np.mean(runtimes)), 1),
+            "runtime_us_min": int(np.min(runtimes))}
+
+
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same
 # counters on a 256 MiB copy); the runs and their commands are in profiles/<kernel>_<workload>.txt.
 MEASURED_TRAFFIC_BYTES = {
@@ -168,6 +206,11 @@ def main() -> None:
                          "passed: the GPU leaves its idle power state only after a few hundred "
                          "milliseconds of work, and a short MFMA run measured before that reads "
                          "up to 40%% slow")
+    ap.add_argument("--via-server", action="store_true",
+                    help="additionally drive the same workload through futhark_amd/bin/"
+                         "segops-server the way `futhark bench` does (values restored from a "
+                         "binary data file, K `call`s) and report the runtimes the server prints; "
+                         "scan/reduce/segscan/segred workloads only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -239,6 +282,10 @@ def main() -> None:
                "sample": f"{reps} passes of the full workload with the futhark-multicore-style "
                          f"restatement in oracle/multicore.c ({t_cpu:.1f} s)"}
 
+    server = None
+    if args.via_server:
+        server = run_via_server(args.workload, args.steps, args.warmup)
+
     if args.calibrate_copy:
         import ctypes as C
         from futhark_amd import lib_path
@@ -264,6 +311,8 @@ def main() -> None:
                      "kernel": w["kernel"], "kernel_us": round(kernel_us, 3)},
         "cpu_baseline": cpu,
     }
+    if server is not None:
+        out["server"] = server
     print(json.dumps(out))
     ctx.close()
 

@@ -2,6 +2,8 @@
 
   futhark_amd/lib/libfuthark_amd_kernels.so   HIP kernels for gfx950 + C ABI (hipcc)
   futhark_amd/lib/libsegops.so                C runtime + `segops` program API (gcc)
+  futhark_amd/lib/libfuthark_amd_values.so    Futhark value reader/writer (gcc)
+  futhark_amd/bin/segops-server               server executable of the program (gcc)
   oracle/liboracle.so                         CPU oracle and CPU baseline (gcc)
 
 Run as `python -m futhark_amd.build` or through `__graft_entry__.build()`.
@@ -84,6 +86,26 @@ def build_host() -> Path:
     return out
 
 
+def build_server() -> Path:
+    """The value reader/writer as a library of its own (tools and tests bind it)
+    and the server executable, which needs nothing but the public API."""
+    OBJ.mkdir(parents=True, exist_ok=True)
+    bindir = PKG / "bin"
+    bindir.mkdir(parents=True, exist_ok=True)
+    server_flags = ["-O2", "-std=c99", "-fPIC", "-Wall", "-Wextra", f"-I{ROOT / 'include'}",
+                    f"-I{CSRC / 'server'}"]
+    values_obj = OBJ / "server_values.o"
+    _run(["gcc", *server_flags, "-c", str(CSRC / "server" / "values.c"), "-o", str(values_obj)])
+    _run(["gcc", "-shared", "-o", str(LIB / "libfuthark_amd_values.so"), str(values_obj), "-lm"])
+    server_obj = OBJ / "server_server.o"
+    _run(["gcc", *server_flags, "-c", str(CSRC / "server" / "server.c"), "-o", str(server_obj)])
+    out = bindir / "segops-server"
+    _run(["gcc", "-o", str(out), str(server_obj), str(values_obj), f"-L{LIB}", "-lsegops",
+          "-lfuthark_amd_kernels", f"-L{ROCM / 'lib'}", "-lamdhip64", "-lm",
+          "-Wl,-rpath,$ORIGIN/../lib", f"-Wl,-rpath,{ROCM / 'lib'}"])
+    return out
+
+
 def build_oracle() -> Path:
     _run(["make", "-C", str(ROOT / "oracle"), "-s"])
     return ROOT / "oracle" / "liboracle.so"
@@ -92,9 +114,11 @@ def build_oracle() -> Path:
 def build_all() -> None:
     build_kernels()
     build_host()
+    build_server()
     build_oracle()
 
 
 if __name__ == "__main__":
     build_all()
-    print("built:", *(str(p) for p in sorted(LIB.glob("*.so"))), ROOT / "oracle" / "liboracle.so")
+    print("built:", *(str(p) for p in sorted(LIB.glob("*.so"))), PKG / "bin" / "segops-server",
+          ROOT / "oracle" / "liboracle.so")

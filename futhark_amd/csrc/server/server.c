@@ -1,0 +1,1019 @@
+/* segops-server: the line-oriented server executable of the `segops` program
+ * (docs/server-protocol.rst), i.e. what `futhark hip --server segops.fut` would
+ * give `futhark bench/test/autotune` to talk to.  It sits entirely on the public
+ * C API of libsegops.so (include/segops.h) plus the value reader/writer of
+ * values.c.  Command set, replies and error texts follow rts/c/server.h
+ * (dispatcher :1447-1535, call :344-403, restore/store :405-480); the program
+ * has no sum types and its only records are the pair results of the by-key
+ * sorts.
+ *
+ * Variables hold either a scalar (stored inline) or a pointer to a library
+ * array; records hold the variables of their fields. */
+#define _POSIX_C_SOURCE 200809L
+#include <ctype.h>
+#include <errno.h>
+#include <getopt.h>
+#include <inttypes.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <time.h>
+
+#include "segops.h"
+#include "futhark_amd_values.h"
+
+/* ------------------------------------------------------------------ types */
+
+enum kind { K_PRIMITIVE, K_ARRAY, K_RECORD };
+
+struct stype;
+typedef void *(*arr_new_fn)(struct futhark_context *, const void *, const int64_t *);
+typedef int (*arr_free_fn)(struct futhark_context *, void *);
+typedef int (*arr_values_fn)(struct futhark_context *, void *, void *);
+typedef const int64_t *(*arr_shape_fn)(struct futhark_context *, void *);
+typedef int (*arr_index_fn)(struct futhark_context *, void *, void *, const int64_t *);
+
+struct stype {
+  const char *name; /* Futhark syntax without sizes: "f32", "[]f32", "([]u32, []i32)" */
+  enum kind kind;
+  const char *prim; /* element (or scalar) type name for values.c */
+  int rank;
+  arr_new_fn arr_new;
+  arr_free_fn arr_free;
+  arr_values_fn arr_values;
+  arr_shape_fn arr_shape;
+  arr_index_fn arr_index;
+  int num_fields; /* records */
+  const char *field_names[2];
+  const char *field_types[2];
+};
+
+/* Uniform-signature shims over the per-type array API. */
+#define ARRAY_SHIMS_1D(N, CT)                                                                \
+  static void *new_##N##_1d(struct futhark_context *c, const void *d, const int64_t *s) {    \
+    return futhark_new_##N##_1d(c, (const CT *)d, s[0]);                                     \
+  }                                                                                          \
+  static int index_##N##_1d(struct futhark_context *c, void *o, void *a, const int64_t *i) { \
+    return futhark_index_##N##_1d(c, (CT *)o, a, i[0]);                                      \
+  }
+#define ARRAY_SHIMS_2D(N, CT)                                                                \
+  static void *new_##N##_2d(struct futhark_context *c, const void *d, const int64_t *s) {    \
+    return futhark_new_##N##_2d(c, (const CT *)d, s[0], s[1]);                               \
+  }                                                                                          \
+  static int index_##N##_2d(struct futhark_context *c, void *o, void *a, const int64_t *i) { \
+    return futhark_index_##N##_2d(c, (CT *)o, a, i[0], i[1]);                                \
+  }
+#define ARRAY_SHIMS_3D(N, CT)                                                                \
+  static void *new_##N##_3d(struct futhark_context *c, const void *d, const int64_t *s) {    \
+    return futhark_new_##N##_3d(c, (const CT *)d, s[0], s[1], s[2]);                         \
+  }                                                                                          \
+  static int index_##N##_3d(struct futhark_context *c, void *o, void *a, const int64_t *i) { \
+    return futhark_index_##N##_3d(c, (CT *)o, a, i[0], i[1], i[2]);                          \
+  }
+#define ARRAY_SHIMS_COMMON(N, R)                                                             \
+  static int free_##N##_##R(struct futhark_context *c, void *a) {                            \
+    return futhark_free_##N##_##R(c, a);                                                     \
+  }                                                                                          \
+  static int values_##N##_##R(struct futhark_context *c, void *a, void *o) {                 \
+    return futhark_values_##N##_##R(c, a, o);                                                \
+  }                                                                                          \
+  static const int64_t *shape_##N##_##R(struct futhark_context *c, void *a) {                \
+    return futhark_shape_##N##_##R(c, a);                                                    \
+  }
+#define A1(N, CT) ARRAY_SHIMS_1D(N, CT) ARRAY_SHIMS_COMMON(N, 1d)
+#define A2(N, CT) ARRAY_SHIMS_2D(N, CT) ARRAY_SHIMS_COMMON(N, 2d)
+#define A3(N, CT) ARRAY_SHIMS_3D(N, CT) ARRAY_SHIMS_COMMON(N, 3d)
+A1(i32, int32_t) A1(i64, int64_t) A1(u8, uint8_t) A1(u32, uint32_t) A1(u64, uint64_t)
+A1(f32, float) A1(f64, double)
+A2(i32, int32_t) A2(i64, int64_t) A2(f32, float) A2(f64, double)
+A3(f32, float) A3(f16, uint16_t) A3(u16, uint16_t)
+
+#define PRIM(N) {N, K_PRIMITIVE, N, 0, NULL, NULL, NULL, NULL, NULL, 0, {0}, {0}}
+#define ARR(NAME, P, R, N, S) \
+  {NAME, K_ARRAY, P, R, new_##N##_##S, free_##N##_##S, values_##N##_##S, shape_##N##_##S, \
+   index_##N##_##S, 0, {0}, {0}}
+#define PAIR(NAME, T0, T1) \
+  {NAME, K_RECORD, NULL, 0, NULL, NULL, NULL, NULL, NULL, 2, {"0", "1"}, {T0, T1}}
+
+static const struct stype types[] = {
+    PRIM("i32"), PRIM("i64"), PRIM("f32"), PRIM("f64"),
+    ARR("[]i32", "i32", 1, i32, 1d), ARR("[]i64", "i64", 1, i64, 1d),
+    ARR("[]u8", "u8", 1, u8, 1d), ARR("[]u32", "u32", 1, u32, 1d),
+    ARR("[]u64", "u64", 1, u64, 1d), ARR("[]f32", "f32", 1, f32, 1d),
+    ARR("[]f64", "f64", 1, f64, 1d),
+    ARR("[][]i32", "i32", 2, i32, 2d), ARR("[][]i64", "i64", 2, i64, 2d),
+    ARR("[][]f32", "f32", 2, f32, 2d), ARR("[][]f64", "f64", 2, f64, 2d),
+    ARR("[][][]f32", "f32", 3, f32, 3d), ARR("[][][]f16", "f16", 3, f16, 3d),
+    ARR("[][][]u16", "u16", 3, u16, 3d),
+    PAIR("([]u32, []i32)", "[]u32", "[]i32"), PAIR("([]u64, []i32)", "[]u64", "[]i32"),
+};
+#define NUM_TYPES ((int)(sizeof(types) / sizeof(types[0])))
+
+static const struct stype *find_type(const char *name) {
+  for (int i = 0; i < NUM_TYPES; i++)
+    if (strcmp(types[i].name, name) == 0) return &types[i];
+  return NULL;
+}
+
+/* ----------------------------------------------------------------- values */
+
+struct variable;
+struct value {
+  const struct stype *type;
+  union {
+    int32_t i32;
+    int64_t i64;
+    float f32;
+    double f64;
+    unsigned char bytes[8];
+    void *arr;
+    struct variable *fields[2]; /* records own anonymous variables */
+  } u;
+};
+
+struct variable {
+  char *name; /* NULL for the anonymous fields of a record */
+  struct value value;
+  struct variable *next;
+};
+
+/* ------------------------------------------------------------ entry points */
+
+typedef int (*entry_fn)(struct futhark_context *, struct value *out, struct value **ins);
+
+struct entry {
+  const char *name;
+  entry_fn f;
+  const char *out_type;
+  int out_unique;
+  int num_ins;
+  const char *in_types[3];
+  int in_consumed[3];
+  const char *tuning_params[3]; /* NULL terminated */
+};
+
+#define ARRP(v) ((v)->u.arr)
+#define SEGOP_ENTRY_FNS(OP, T, CT)                                                             \
+  static int e_reduce_##OP##_##T(struct futhark_context *c, struct value *o,                   \
+                                 struct value **i) {                                           \
+    return futhark_entry_reduce_##OP##_##T(c, (CT *)o->u.bytes, ARRP(i[0]));                   \
+  }                                                                                            \
+  static int e_scan_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) { \
+    return futhark_entry_scan_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,             \
+                                         ARRP(i[0]));                                          \
+  }                                                                                            \
+  static int e_exscan_##OP##_##T(struct futhark_context *c, struct value *o,                   \
+                                 struct value **i) {                                           \
+    return futhark_entry_exscan_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,           \
+                                           ARRP(i[0]));                                        \
+  }                                                                                            \
+  static int e_segscan_##OP##_##T(struct futhark_context *c, struct value *o,                  \
+                                  struct value **i) {                                          \
+    return futhark_entry_segscan_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,          \
+                                            ARRP(i[0]), ARRP(i[1]));                           \
+  }                                                                                            \
+  static int e_segred_##OP##_##T(struct futhark_context *c, struct value *o,                   \
+                                 struct value **i) {                                           \
+    return futhark_entry_segred_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,           \
+                                           ARRP(i[0]), ARRP(i[1]), ARRP(i[2]));                \
+  }                                                                                            \
+  static int e_segreduce_##OP##_##T(struct futhark_context *c, struct value *o,                \
+                                    struct value **i) {                                        \
+    return futhark_entry_segreduce_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,        \
+                                              ARRP(i[0]));                                     \
+  }                                                                                            \
+  static int e_hist_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) { \
+    return futhark_entry_hist_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,             \
+                                         i[0]->u.i64, ARRP(i[1]), ARRP(i[2]));                 \
+  }                                                                                            \
+  static int e_rbi_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) {  \
+    return futhark_entry_rbi_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr, ARRP(i[0]),  \
+                                        ARRP(i[1]), ARRP(i[2]));                               \
+  }
+#define SEGOP_ENTRY_FNS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(SEGOP_ENTRY_FNS, T, CT)
+FUTHARK_FOR_EACH_NUM_TYPE(SEGOP_ENTRY_FNS_FOR_TYPE)
+
+static int e_bmm_f32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_bmm_f32(c, (struct futhark_f32_3d **)&o->u.arr, ARRP(i[0]), ARRP(i[1]));
+}
+static int e_bmm_f16(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_bmm_f16(c, (struct futhark_f32_3d **)&o->u.arr, ARRP(i[0]), ARRP(i[1]));
+}
+static int e_bmm_bf16(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_bmm_bf16(c, (struct futhark_f32_3d **)&o->u.arr, ARRP(i[0]), ARRP(i[1]));
+}
+static int e_matmul_f32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_matmul_f32(c, (struct futhark_f32_2d **)&o->u.arr, ARRP(i[0]),
+                                  ARRP(i[1]));
+}
+static int e_radix_sort_u32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_radix_sort_u32(c, (struct futhark_u32_1d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_radix_sort_u64(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_radix_sort_u64(c, (struct futhark_u64_1d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_radix_sort_pairs_u32_i32(struct futhark_context *c, struct value *o,
+                                      struct value **i) {
+  return futhark_entry_radix_sort_pairs_u32_i32(
+      c, (struct futhark_u32_1d **)&o->u.fields[0]->value.u.arr,
+      (struct futhark_i32_1d **)&o->u.fields[1]->value.u.arr, ARRP(i[0]), ARRP(i[1]));
+}
+static int e_radix_sort_pairs_u64_i32(struct futhark_context *c, struct value *o,
+                                      struct value **i) {
+  return futhark_entry_radix_sort_pairs_u64_i32(
+      c, (struct futhark_u64_1d **)&o->u.fields[0]->value.u.arr,
+      (struct futhark_i32_1d **)&o->u.fields[1]->value.u.arr, ARRP(i[0]), ARRP(i[1]));
+}
+static int e_transpose_f32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_transpose_f32(c, (struct futhark_f32_2d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_iota_i64(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_iota_i64(c, (struct futhark_i64_1d **)&o->u.arr, i[0]->u.i64);
+}
+static int e_replicate_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_replicate_i32(c, (struct futhark_i32_1d **)&o->u.arr, i[0]->u.i64,
+                                     i[1]->u.i32);
+}
+
+#define HIST_PARAM "segops.hist_lds_bins_max"
+#define SEGRED_PARAM "segops.segred_small_threshold"
+#define SEGOP_ENTRY_ROWS(OP, T, CT)                                                             \
+  {"reduce_" #OP "_" #T, e_reduce_##OP##_##T, #T, 1, 1, {"[]" #T}, {0}, {NULL}},                \
+  {"scan_" #OP "_" #T, e_scan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {NULL}},               \
+  {"exscan_" #OP "_" #T, e_exscan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {NULL}},           \
+  {"segscan_" #OP "_" #T, e_segscan_##OP##_##T, "[]" #T, 1, 2, {"[]u8", "[]" #T}, {0}, {NULL}}, \
+  {"segred_" #OP "_" #T, e_segred_##OP##_##T, "[]" #T, 1, 3, {"[]i64", "[]i64", "[]" #T},       \
+   {0}, {NULL}},                                                                                \
+  {"segreduce_" #OP "_" #T, e_segreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0},            \
+   {SEGRED_PARAM, NULL}},                                                                       \
+  {"hist_" #OP "_" #T, e_hist_##OP##_##T, "[]" #T, 1, 3, {"i64", "[]i32", "[]" #T}, {0},        \
+   {HIST_PARAM, NULL}},                                                                         \
+  {"rbi_" #OP "_" #T, e_rbi_##OP##_##T, "[]" #T, 1, 3, {"[]" #T, "[]i32", "[]" #T}, {1, 0, 0},  \
+   {HIST_PARAM, NULL}},
+#define SEGOP_ENTRY_ROWS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(SEGOP_ENTRY_ROWS, T, CT)
+
+static const struct entry entries[] = {
+    FUTHARK_FOR_EACH_NUM_TYPE(SEGOP_ENTRY_ROWS_FOR_TYPE)
+    {"bmm_f32", e_bmm_f32, "[][][]f32", 1, 2, {"[][][]f32", "[][][]f32"}, {0}, {NULL}},
+    {"bmm_f16", e_bmm_f16, "[][][]f32", 1, 2, {"[][][]f16", "[][][]f16"}, {0}, {NULL}},
+    {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {NULL}},
+    {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {NULL}},
+    {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {NULL}},
+    {"radix_sort_u64", e_radix_sort_u64, "[]u64", 1, 1, {"[]u64"}, {0}, {NULL}},
+    {"radix_sort_pairs_u32_i32", e_radix_sort_pairs_u32_i32, "([]u32, []i32)", 1, 2,
+     {"[]u32", "[]i32"}, {0}, {NULL}},
+    {"radix_sort_pairs_u64_i32", e_radix_sort_pairs_u64_i32, "([]u64, []i32)", 1, 2,
+     {"[]u64", "[]i32"}, {0}, {NULL}},
+    {"transpose_f32", e_transpose_f32, "[][]f32", 1, 1, {"[][]f32"}, {0}, {NULL}},
+    {"iota_i64", e_iota_i64, "[]i64", 1, 1, {"i64"}, {0}, {NULL}},
+    {"replicate_i32", e_replicate_i32, "[]i32", 1, 2, {"i64", "i32"}, {0}, {NULL}},
+};
+#define NUM_ENTRIES ((int)(sizeof(entries) / sizeof(entries[0])))
+
+static const struct entry *find_entry(const char *name) {
+  for (int i = 0; i < NUM_ENTRIES; i++)
+    if (strcmp(entries[i].name, name) == 0) return &entries[i];
+  return NULL;
+}
+
+/* ----------------------------------------------------------------- server */
+
+struct server {
+  struct futhark_context_config *cfg;
+  struct futhark_context *ctx;
+  struct variable *vars;
+};
+
+static void reply_ok(void) {
+  printf("%%%%%% OK\n");
+  fflush(stdout);
+}
+
+/* After this marker everything up to the next OK is the error message. */
+static void reply_failure(const char *fmt, ...) {
+  printf("%%%%%% FAILURE\n");
+  if (fmt != NULL) {
+    va_list ap;
+    va_start(ap, fmt);
+    vprintf(fmt, ap);
+    va_end(ap);
+  }
+}
+
+static void report_context_error(struct server *s, int err) {
+  if (err == 0) return;
+  reply_failure(NULL);
+  char *msg = futhark_context_get_error(s->ctx);
+  if (msg != NULL) puts(msg);
+  free(msg);
+}
+
+static struct variable *find_var(struct server *s, const char *name) {
+  for (struct variable *v = s->vars; v != NULL; v = v->next)
+    if (strcmp(v->name, name) == 0) return v;
+  return NULL;
+}
+
+static struct variable *alloc_var(const char *name, const struct stype *t) {
+  struct variable *v = calloc(1, sizeof *v);
+  if (v == NULL) abort();
+  v->name = name ? strdup(name) : NULL;
+  v->value.type = t;
+  if (t->kind == K_RECORD)
+    for (int i = 0; i < t->num_fields; i++)
+      v->value.u.fields[i] = alloc_var(NULL, find_type(t->field_types[i]));
+  return v;
+}
+
+/* NULL if the name is taken. */
+static struct variable *create_var(struct server *s, const char *name, const struct stype *t) {
+  if (find_var(s, name) != NULL) return NULL;
+  struct variable *v = alloc_var(name, t);
+  v->next = s->vars;
+  s->vars = v;
+  return v;
+}
+
+static void release_value(struct server *s, struct value *val) {
+  const struct stype *t = val->type;
+  if (t->kind == K_ARRAY) {
+    if (val->u.arr != NULL) t->arr_free(s->ctx, val->u.arr);
+    val->u.arr = NULL;
+  } else if (t->kind == K_RECORD) {
+    for (int i = 0; i < t->num_fields; i++) {
+      if (val->u.fields[i] == NULL) continue;
+      release_value(s, &val->u.fields[i]->value);
+      free(val->u.fields[i]);
+      val->u.fields[i] = NULL;
+    }
+  }
+}
+
+static void drop_var(struct server *s, struct variable *v, int release) {
+  for (struct variable **p = &s->vars; *p != NULL; p = &(*p)->next)
+    if (*p == v) {
+      *p = v->next;
+      break;
+    }
+  if (release) {
+    release_value(s, &v->value);
+  } else if (v->value.type->kind == K_RECORD) {
+    for (int i = 0; i < v->value.type->num_fields; i++) free(v->value.u.fields[i]);
+  }
+  free(v->name);
+  free(v);
+}
+
+static int count_args(char **args) {
+  int n = 0;
+  while (args[n] != NULL) n++;
+  return n;
+}
+
+/* A missing argument ends the server, as in the reference (get_arg,
+ * rts/c/server.h:296-308). */
+static const char *need_arg(char **args, int i) {
+  for (int k = 0; k <= i; k++)
+    if (args[k] == NULL) {
+      fprintf(stderr, "Insufficient command args.\n");
+      exit(1);
+    }
+  return args[i];
+}
+
+static int64_t now_usec(void) {
+  struct timespec ts;
+  clock_gettime(CLOCK_MONOTONIC, &ts);
+  return (int64_t)ts.tv_sec * 1000000 + ts.tv_nsec / 1000;
+}
+
+static void cmd_call(struct server *s, char **args) {
+  const char *name = need_arg(args, 0);
+  const char *out_name = need_arg(args, 1);
+  const struct entry *e = find_entry(name);
+  if (e == NULL) {
+    reply_failure("Unknown entry point: %s\n", name);
+    return;
+  }
+  struct value *ins[3] = {0};
+  for (int i = 0; i < e->num_ins; i++) {
+    const char *in_name = need_arg(args, 2 + i);
+    struct variable *v = find_var(s, in_name);
+    if (v == NULL) {
+      reply_failure("Unknown variable: %s\n", in_name);
+      return;
+    }
+    if (strcmp(v->value.type->name, e->in_types[i]) != 0) {
+      reply_failure("Wrong input type.  Expected %s, got %s.\n", e->in_types[i],
+                    v->value.type->name);
+      return;
+    }
+    ins[i] = &v->value;
+  }
+  struct variable *out = create_var(s, out_name, find_type(e->out_type));
+  if (out == NULL) {
+    reply_failure("Variable already exists: %s\n", out_name);
+    return;
+  }
+  const int64_t t0 = now_usec();
+  int err = e->f(s->ctx, &out->value, ins);
+  err |= futhark_context_sync(s->ctx);
+  const int64_t t1 = now_usec();
+  printf("runtime: %lld\n", (long long)(t1 - t0));
+  report_context_error(s, err);
+  if (err != 0) drop_var(s, out, 0); /* the outputs were left untouched */
+}
+
+/* Reads one value of type t from f into val (val->type already set). */
+static int restore_value(struct server *s, FILE *f, struct value *val) {
+  const struct stype *t = val->type;
+  if (t->kind == K_RECORD) {
+    for (int i = 0; i < t->num_fields; i++)
+      if (restore_value(s, f, &val->u.fields[i]->value) != 0) return 1;
+    return 0;
+  }
+  int64_t shape[FV_MAX_RANK];
+  void *data = NULL;
+  if (fv_read_binary(f, fv_primtype(t->prim), t->rank, shape, &data, NULL, 0) != 0) return 1;
+  int rc = 0;
+  if (t->kind == K_PRIMITIVE) {
+    memcpy(val->u.bytes, data, (size_t)fv_primtype(t->prim)->size);
+  } else {
+    val->u.arr = t->arr_new(s->ctx, data, shape);
+    if (val->u.arr == NULL) rc = 1;
+    /* The copy to the device is asynchronous and reads `data`. */
+    if (rc == 0 && futhark_context_sync(s->ctx) != 0) rc = 1;
+  }
+  free(data);
+  return rc;
+}
+
+static void cmd_restore(struct server *s, char **args) {
+  const char *fname = need_arg(args, 0);
+  FILE *f = fopen(fname, "rb");
+  if (f == NULL) {
+    reply_failure("Failed to open %s: %s\n", fname, strerror(errno));
+    return;
+  }
+  int bad = 0, values = 0;
+  for (int i = 1; args[i] != NULL; i += 2, values++) {
+    const char *vname = args[i];
+    const char *tname = need_arg(args, i + 1);
+    const struct stype *t = find_type(tname);
+    if (t == NULL) {
+      bad = 1;
+      reply_failure("Unknown type: %s\n", tname);
+      break;
+    }
+    struct variable *v = create_var(s, vname, t);
+    if (v == NULL) {
+      bad = 1;
+      reply_failure("Variable already exists: %s\n", vname);
+      break;
+    }
+    errno = 0;
+    if (restore_value(s, f, &v->value) != 0) {
+      bad = 1;
+      reply_failure("Failed to restore variable %s.\n"
+                    "Possibly malformed data in %s (errno: %s)\n",
+                    vname, fname, strerror(errno));
+      drop_var(s, v, 1);
+      break;
+    }
+  }
+  if (!bad && fv_end_of_input(f) != 0)
+    reply_failure("Expected EOF after reading %d values from %s\n", values, fname);
+  fclose(f);
+  if (!bad) report_context_error(s, futhark_context_sync(s->ctx));
+}
+
+static int store_value(struct server *s, FILE *f, struct value *val) {
+  const struct stype *t = val->type;
+  if (t->kind == K_RECORD) {
+    for (int i = 0; i < t->num_fields; i++)
+      if (store_value(s, f, &val->u.fields[i]->value) != 0) return 1;
+    return 0;
+  }
+  const struct fv_primtype *p = fv_primtype(t->prim);
+  if (t->kind == K_PRIMITIVE) return fv_write_binary(f, p, 0, NULL, val->u.bytes);
+  const int64_t *shape = t->arr_shape(s->ctx, val->u.arr);
+  size_t count = 1;
+  for (int i = 0; i < t->rank; i++) count *= (size_t)shape[i];
+  void *host = malloc(count * (size_t)p->size + 1);
+  if (host == NULL) return 1;
+  int rc = t->arr_values(s->ctx, val->u.arr, host);
+  rc |= futhark_context_sync(s->ctx);
+  if (rc == 0) rc = fv_write_binary(f, p, t->rank, shape, host);
+  free(host);
+  return rc;
+}
+
+static void cmd_store(struct server *s, char **args) {
+  const char *fname = need_arg(args, 0);
+  FILE *f = fopen(fname, "wb");
+  if (f == NULL) {
+    reply_failure("Failed to open %s: %s\n", fname, strerror(errno));
+    return;
+  }
+  for (int i = 1; args[i] != NULL; i++) {
+    struct variable *v = find_var(s, args[i]);
+    if (v == NULL) {
+      reply_failure("Unknown variable: %s\n", args[i]);
+      break;
+    }
+    if (store_value(s, f, &v->value) != 0) {
+      report_context_error(s, 1);
+      break;
+    }
+  }
+  fclose(f);
+}
+
+static void cmd_free(struct server *s, char **args) {
+  for (int i = 0; args[i] != NULL; i++) {
+    struct variable *v = find_var(s, args[i]);
+    if (v == NULL) {
+      reply_failure("Unknown variable: %s\n", args[i]);
+      return;
+    }
+    drop_var(s, v, 1);
+  }
+}
+
+static void cmd_rename(struct server *s, char **args) {
+  const char *oldname = need_arg(args, 0), *newname = need_arg(args, 1);
+  struct variable *v = find_var(s, oldname);
+  if (v == NULL) {
+    reply_failure("Unknown variable: %s\n", oldname);
+    return;
+  }
+  if (find_var(s, newname) != NULL) {
+    reply_failure("Variable already exists: %s\n", newname);
+    return;
+  }
+  free(v->name);
+  v->name = strdup(newname);
+}
+
+static void cmd_inputs(char **args) {
+  const struct entry *e = find_entry(need_arg(args, 0));
+  if (e == NULL) {
+    reply_failure("Unknown entry point: %s\n", args[0]);
+    return;
+  }
+  for (int i = 0; i < e->num_ins; i++)
+    printf("%s%s\n", e->in_consumed[i] ? "*" : "", e->in_types[i]);
+}
+
+static void cmd_output(char **args) {
+  const struct entry *e = find_entry(need_arg(args, 0));
+  if (e == NULL) {
+    reply_failure("Unknown entry point: %s\n", args[0]);
+    return;
+  }
+  printf("%s%s\n", e->out_unique ? "*" : "", e->out_type);
+}
+
+static void cmd_report(struct server *s) {
+  char *report = futhark_context_report(s->ctx);
+  if (report != NULL) {
+    puts(report);
+  } else {
+    reply_failure("Failed to produce profiling report.\n");
+  }
+  free(report);
+}
+
+static void cmd_set_tuning_param(struct server *s, char **args) {
+  const char *param = need_arg(args, 0), *val_s = need_arg(args, 1);
+  const size_t val = (size_t)strtoull(val_s, NULL, 10);
+  if (futhark_context_config_set_tuning_param(s->cfg, param, val) != 0)
+    reply_failure("Failed to set tuning parameter %s to %ld\n", param, (long)val);
+}
+
+static void cmd_tuning_params(char **args) {
+  const struct entry *e = find_entry(need_arg(args, 0));
+  if (e == NULL) {
+    reply_failure("Unknown entry point: %s\n", args[0]);
+    return;
+  }
+  for (int i = 0; i < 3 && e->tuning_params[i] != NULL; i++) {
+    const char *cls = "";
+    for (int k = 0; k < futhark_get_tuning_param_count(); k++)
+      if (strcmp(futhark_get_tuning_param_name(k), e->tuning_params[i]) == 0)
+        cls = futhark_get_tuning_param_class(k);
+    printf("%s %s\n", e->tuning_params[i], cls);
+  }
+}
+
+static void cmd_tuning_param_class(char **args) {
+  const char *param = need_arg(args, 0);
+  for (int k = 0; k < futhark_get_tuning_param_count(); k++)
+    if (strcmp(futhark_get_tuning_param_name(k), param) == 0) {
+      printf("%s\n", futhark_get_tuning_param_class(k));
+      return;
+    }
+  reply_failure("Unknown tuning parameter: %s\n", param);
+}
+
+static void cmd_kind(char **args) {
+  const struct stype *t = find_type(need_arg(args, 0));
+  if (t == NULL) {
+    reply_failure("Unknown type: %s\n", args[0]);
+    return;
+  }
+  puts(t->kind == K_PRIMITIVE ? "primitive" : t->kind == K_ARRAY ? "array" : "record");
+}
+
+static const struct stype *array_type_arg(char **args) {
+  const struct stype *t = find_type(need_arg(args, 0));
+  if (t == NULL || t->kind != K_ARRAY) {
+    reply_failure("Not an array type\n");
+    return NULL;
+  }
+  return t;
+}
+
+static void cmd_shape(struct server *s, char **args) {
+  struct variable *v = find_var(s, need_arg(args, 0));
+  if (v == NULL) {
+    reply_failure("Unknown variable: %s\n", args[0]);
+    return;
+  }
+  if (v->value.type->kind != K_ARRAY) {
+    reply_failure("Not an array type\n");
+    return;
+  }
+  const int64_t *shape = v->value.type->arr_shape(s->ctx, v->value.u.arr);
+  for (int i = 0; i < v->value.type->rank; i++) printf("%lld\n", (long long)shape[i]);
+}
+
+/* Parses a whole decimal integer. */
+static int parse_i64(const char *s, int64_t *out) {
+  char *end;
+  errno = 0;
+  const long long v = strtoll(s, &end, 10);
+  if (errno != 0 || end == s || *end != 0) return 1;
+  *out = v;
+  return 0;
+}
+
+static void cmd_new_array(struct server *s, char **args) {
+  const char *to = need_arg(args, 0);
+  const struct stype *t = find_type(need_arg(args, 1));
+  if (find_var(s, to) != NULL) {
+    reply_failure("Variable already exists: %s\n", to);
+    return;
+  }
+  if (t == NULL || t->kind != K_ARRAY) {
+    reply_failure("Not an array type\n");
+    return;
+  }
+  const int num_args = count_args(args + 2);
+  if (num_args < t->rank) {
+    reply_failure("Expected %d dimensions, but got %d.\n", t->rank, num_args);
+    return;
+  }
+  int64_t shape[FV_MAX_RANK], count = 1;
+  for (int i = 0; i < t->rank; i++) {
+    if (parse_i64(args[2 + i], &shape[i]) != 0 || shape[i] < 0) {
+      reply_failure("Invalid size `%s` of dimension %d.\n", args[2 + i], i + 1);
+      return;
+    }
+    count *= shape[i];
+  }
+  if (count != num_args - t->rank) {
+    reply_failure("Expected %d values, but got %d.\n", (int)count, num_args - t->rank);
+    return;
+  }
+  const struct fv_primtype *p = fv_primtype(t->prim);
+  unsigned char *host = malloc((size_t)count * (size_t)p->size + 1);
+  if (host == NULL) {
+    reply_failure("Out of memory.\n");
+    return;
+  }
+  for (int64_t i = 0; i < count; i++) {
+    const char *vn = args[2 + t->rank + i];
+    struct variable *v = find_var(s, vn);
+    if (v == NULL) {
+      reply_failure("Unknown variable: %s\n", vn);
+      free(host);
+      return;
+    }
+    if (v->value.type->kind != K_PRIMITIVE || strcmp(v->value.type->prim, t->prim) != 0) {
+      reply_failure("Value %d mismatch: expected type %s, got %s\n", (int)i, t->prim,
+                    v->value.type->name);
+      free(host);
+      return;
+    }
+    memcpy(host + (size_t)i * (size_t)p->size, v->value.u.bytes, (size_t)p->size);
+  }
+  struct variable *out = create_var(s, to, t);
+  out->value.u.arr = t->arr_new(s->ctx, host, shape);
+  int err = out->value.u.arr == NULL;
+  err |= futhark_context_sync(s->ctx);
+  free(host);
+  report_context_error(s, err);
+  if (err != 0) drop_var(s, out, 1);
+}
+
+static void cmd_index(struct server *s, char **args) {
+  const char *to = need_arg(args, 0);
+  struct variable *from = find_var(s, need_arg(args, 1));
+  if (from == NULL) {
+    reply_failure("Unknown variable: %s\n", args[1]);
+    return;
+  }
+  const struct stype *t = from->value.type;
+  if (t->kind != K_ARRAY) {
+    reply_failure("Not an array type\n");
+    return;
+  }
+  int64_t idx[FV_MAX_RANK];
+  for (int i = 0; i < t->rank; i++) {
+    if (args[2 + i] == NULL) {
+      reply_failure("%d indices expected but %d values provided.\n", t->rank, i);
+      return;
+    }
+    if (parse_i64(args[2 + i], &idx[i]) != 0) {
+      reply_failure("Invalid index `%s` on dimension %d.\n", args[2 + i], i + 1);
+      return;
+    }
+  }
+  struct variable *out = create_var(s, to, find_type(t->prim));
+  if (out == NULL) {
+    reply_failure("Variable already exists: %s\n", to);
+    return;
+  }
+  int err = t->arr_index(s->ctx, out->value.u.bytes, from->value.u.arr, idx);
+  err |= futhark_context_sync(s->ctx);
+  report_context_error(s, err);
+  if (err != 0) drop_var(s, out, 0);
+}
+
+static void cmd_fields(char **args) {
+  const struct stype *t = find_type(need_arg(args, 0));
+  if (t == NULL || t->kind != K_RECORD) {
+    reply_failure("Not a record type\n");
+    return;
+  }
+  for (int i = 0; i < t->num_fields; i++) printf("%s %s\n", t->field_names[i], t->field_types[i]);
+}
+
+/* The library's public API has no way to take a second reference to an
+ * array, so a projected field is a copy made through host memory. */
+static void cmd_project(struct server *s, char **args) {
+  const char *to = need_arg(args, 0);
+  struct variable *from = find_var(s, need_arg(args, 1));
+  const char *field = need_arg(args, 2);
+  if (from == NULL) {
+    reply_failure("Unknown variable: %s\n", args[1]);
+    return;
+  }
+  const struct stype *t = from->value.type;
+  if (t->kind != K_RECORD) {
+    reply_failure("Not a record type\n");
+    return;
+  }
+  int fi = -1;
+  for (int i = 0; i < t->num_fields; i++)
+    if (strcmp(t->field_names[i], field) == 0) fi = i;
+  if (fi < 0) {
+    reply_failure("No such field\n");
+    return;
+  }
+  if (find_var(s, to) != NULL) {
+    reply_failure("Variable already exists: %s\n", to);
+    return;
+  }
+  struct value *src = &from->value.u.fields[fi]->value;
+  const struct stype *ft = src->type;
+  const struct fv_primtype *p = fv_primtype(ft->prim);
+  const int64_t *shape = ft->arr_shape(s->ctx, src->u.arr);
+  size_t count = 1;
+  for (int i = 0; i < ft->rank; i++) count *= (size_t)shape[i];
+  void *host = malloc(count * (size_t)p->size + 1);
+  if (host == NULL) {
+    reply_failure("Out of memory.\n");
+    return;
+  }
+  int err = ft->arr_values(s->ctx, src->u.arr, host);
+  err |= futhark_context_sync(s->ctx);
+  struct variable *out = create_var(s, to, ft);
+  if (err == 0) {
+    out->value.u.arr = ft->arr_new(s->ctx, host, shape);
+    err = out->value.u.arr == NULL;
+    err |= futhark_context_sync(s->ctx);
+  }
+  free(host);
+  report_context_error(s, err);
+  if (err != 0) drop_var(s, out, 1);
+}
+
+static char *next_word(char **line) {
+  char *p = *line;
+  while (isspace((unsigned char)*p)) p++;
+  if (*p == 0) return NULL;
+  char *word;
+  if (*p == '"') {
+    word = ++p;
+    while (*p != 0 && *p != '"') p++;
+    if (*p != '"') return NULL; /* unterminated quote ends the line */
+  } else {
+    word = p;
+    while (*p != 0 && !isspace((unsigned char)*p)) p++;
+  }
+  if (*p != 0) {
+    *p = 0;
+    *line = p + 1;
+  } else {
+    *line = p;
+  }
+  return word;
+}
+
+#define MAX_WORDS 1000
+
+static void process_line(struct server *s, char *line) {
+  static char *words[MAX_WORDS + 1];
+  int n = 0;
+  while ((words[n] = next_word(&line)) != NULL) {
+    if (++n == MAX_WORDS) {
+      fprintf(stderr, "Line too long.\n");
+      exit(1);
+    }
+  }
+  const char *cmd = words[0];
+  char **args = words + 1;
+  if (cmd == NULL) {
+    reply_failure("Empty line\n");
+  } else if (strcmp(cmd, "call") == 0) {
+    cmd_call(s, args);
+  } else if (strcmp(cmd, "restore") == 0) {
+    cmd_restore(s, args);
+  } else if (strcmp(cmd, "store") == 0) {
+    cmd_store(s, args);
+  } else if (strcmp(cmd, "free") == 0) {
+    cmd_free(s, args);
+  } else if (strcmp(cmd, "rename") == 0) {
+    cmd_rename(s, args);
+  } else if (strcmp(cmd, "inputs") == 0) {
+    cmd_inputs(args);
+  } else if (strcmp(cmd, "output") == 0) {
+    cmd_output(args);
+  } else if (strcmp(cmd, "clear") == 0) {
+    report_context_error(s, futhark_context_clear_caches(s->ctx));
+  } else if (strcmp(cmd, "pause_profiling") == 0) {
+    futhark_context_pause_profiling(s->ctx);
+  } else if (strcmp(cmd, "unpause_profiling") == 0) {
+    futhark_context_unpause_profiling(s->ctx);
+  } else if (strcmp(cmd, "report") == 0) {
+    cmd_report(s);
+  } else if (strcmp(cmd, "set_tuning_param") == 0) {
+    cmd_set_tuning_param(s, args);
+  } else if (strcmp(cmd, "tuning_params") == 0) {
+    cmd_tuning_params(args);
+  } else if (strcmp(cmd, "tuning_param_class") == 0) {
+    cmd_tuning_param_class(args);
+  } else if (strcmp(cmd, "attributes") == 0) {
+    if (find_entry(need_arg(args, 0)) == NULL) reply_failure("Unknown entry point: %s\n", args[0]);
+  } else if (strcmp(cmd, "kind") == 0) {
+    cmd_kind(args);
+  } else if (strcmp(cmd, "type") == 0) {
+    struct variable *v = find_var(s, need_arg(args, 0));
+    if (v == NULL) reply_failure("Unknown variable: %s\n", args[0]);
+    else puts(v->value.type->name);
+  } else if (strcmp(cmd, "shape") == 0) {
+    cmd_shape(s, args);
+  } else if (strcmp(cmd, "elemtype") == 0) {
+    const struct stype *t = array_type_arg(args);
+    if (t != NULL) puts(t->prim);
+  } else if (strcmp(cmd, "rank") == 0) {
+    const struct stype *t = array_type_arg(args);
+    if (t != NULL) printf("%d\n", t->rank);
+  } else if (strcmp(cmd, "new_array") == 0) {
+    cmd_new_array(s, args);
+  } else if (strcmp(cmd, "index") == 0) {
+    cmd_index(s, args);
+  } else if (strcmp(cmd, "fields") == 0) {
+    cmd_fields(args);
+  } else if (strcmp(cmd, "project") == 0) {
+    cmd_project(s, args);
+  } else if (strcmp(cmd, "entry_points") == 0) {
+    for (int i = 0; i < NUM_ENTRIES; i++) puts(entries[i].name);
+  } else if (strcmp(cmd, "types") == 0) {
+    for (int i = 0; i < NUM_TYPES; i++) puts(types[i].name);
+  } else if (strcmp(cmd, "set") == 0 || strcmp(cmd, "zip") == 0 || strcmp(cmd, "unzip") == 0 ||
+             strcmp(cmd, "new") == 0) {
+    /* In-place array update and record construction: no entry point of this
+     * program takes a record, and no array of records exists. */
+    reply_failure("Command `%s` is not supported by this program.\n", cmd);
+  } else if (strcmp(cmd, "variants") == 0 || strcmp(cmd, "variant") == 0 ||
+             strcmp(cmd, "construct") == 0 || strcmp(cmd, "destruct") == 0) {
+    reply_failure("Not a sum type\n");
+  } else {
+    fprintf(stderr, "Unknown command: %s\n", cmd);
+    exit(1);
+  }
+}
+
+static void usage(const char *prog) {
+  printf("Usage: %s [OPTIONS]...\nOptions:\n\n"
+         "  -D/--debugging     Perform possibly expensive internal correctness checks and "
+         "verbose logging.\n"
+         "  -L/--log           Print various low-overhead logging information while running.\n"
+         "  -P/--profile       Enable the collection of profiling information.\n"
+         "  -h/--help          Print help information and exit.\n"
+         "  --print-params     Print all tuning parameters that can be set with --param or "
+         "--tuning.\n"
+         "  --param NAME=INT   Set a tuning parameter to the given value.\n"
+         "  --tuning FILE      Read tuning parameters (NAME=INT lines) from the indicated file.\n"
+         "  -d/--device NAME   Use the first device whose name contains the given string.\n"
+         "\nFor more information, consult the Futhark User's Guide or the man pages.\n",
+         prog);
+}
+
+static void set_param_or_die(struct futhark_context_config *cfg, const char *assignment) {
+  const char *eq = strchr(assignment, '=');
+  int64_t value;
+  if (eq == NULL || parse_i64(eq + 1, &value) != 0) {
+    fprintf(stderr, "Invalid argument for --param option: %s\n", assignment);
+    exit(1);
+  }
+  char *name = strndup(assignment, (size_t)(eq - assignment));
+  if (futhark_context_config_set_tuning_param(cfg, name, (size_t)value) != 0) {
+    fprintf(stderr, "Unknown parameter: %s\n", name);
+    exit(1);
+  }
+  free(name);
+}
+
+int main(int argc, char **argv) {
+  struct futhark_context_config *cfg = futhark_context_config_new();
+  if (cfg == NULL) abort();
+  static const struct option long_opts[] = {
+      {"debugging", no_argument, NULL, 'D'},   {"log", no_argument, NULL, 'L'},
+      {"profile", no_argument, NULL, 'P'},     {"help", no_argument, NULL, 'h'},
+      {"print-params", no_argument, NULL, 1},  {"param", required_argument, NULL, 2},
+      {"tuning", required_argument, NULL, 3},  {"device", required_argument, NULL, 'd'},
+      {0, 0, 0, 0}};
+  int c;
+  while ((c = getopt_long(argc, argv, ":DLPhd:", long_opts, NULL)) != -1) {
+    switch (c) {
+      case 'D': futhark_context_config_set_debugging(cfg, 1); break;
+      case 'L': futhark_context_config_set_logging(cfg, 1); break;
+      case 'P': futhark_context_config_set_profiling(cfg, 1); break;
+      case 'h': usage(argv[0]); return 0;
+      case 'd': futhark_context_config_set_device(cfg, optarg); break;
+      case 1:
+        for (int i = 0; i < futhark_get_tuning_param_count(); i++)
+          printf("%s (%s)\n", futhark_get_tuning_param_name(i), futhark_get_tuning_param_class(i));
+        return 0;
+      case 2: set_param_or_die(cfg, optarg); break;
+      case 3: {
+        FILE *f = fopen(optarg, "r");
+        if (f == NULL) {
+          fprintf(stderr, "Cannot open %s: %s\n", optarg, strerror(errno));
+          return 1;
+        }
+        char buf[512];
+        while (fgets(buf, sizeof buf, f) != NULL) {
+          buf[strcspn(buf, "\r\n")] = 0;
+          if (buf[0] != 0) set_param_or_die(cfg, buf);
+        }
+        fclose(f);
+        break;
+      }
+      case ':': fprintf(stderr, "Missing argument for option %s\n", argv[optind - 1]); return 1;
+      default: fprintf(stderr, "Unknown option: %s\n", argv[optind - 1]); return 1;
+    }
+  }
+  if (optind < argc) {
+    fprintf(stderr, "Excess non-option: %s\n", argv[optind]);
+    return 1;
+  }
+
+  struct futhark_context *ctx = futhark_context_new(cfg);
+  if (ctx == NULL) abort();
+  futhark_context_set_logging_file(ctx, stdout);
+  char *error = futhark_context_get_error(ctx);
+  if (error != NULL) {
+    fprintf(stderr, "Error during context initialisation:\n%s\n", error);
+    return 1;
+  }
+
+  struct server s = {cfg, ctx, NULL};
+  char *line = NULL;
+  size_t cap = 0;
+  reply_ok();
+  while (getline(&line, &cap, stdin) > 0) {
+    process_line(&s, line);
+    reply_ok();
+  }
+  while (s.vars != NULL) drop_var(&s, s.vars, 1);
+  free(line);
+  futhark_context_free(ctx);
+  futhark_context_config_free(cfg);
+  return 0;
+}

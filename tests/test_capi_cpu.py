@@ -28,6 +28,14 @@ def test_kernel_library_exports_every_declared_launcher():
     assert not missing, missing
 
 
+def test_values_library_exports_every_declared_function():
+    hdr = (ROOT / "include" / "futhark_amd_values.h").read_text()
+    names = set(re.findall(r"\b(fv_\w+)\s*\(", hdr))
+    assert {"fv_read_binary", "fv_write_binary", "fv_write_text", "fv_primtype"} <= names
+    missing = names - _exports(lib_path("libfuthark_amd_values.so"))
+    assert not missing, missing
+
+
 def test_program_library_exports_the_generated_api():
     hdr = (ROOT / "include" / "segops.h").read_text()
     body = "\n".join(l for l in hdr.splitlines() if not l.rstrip().endswith("\\") and "#define" not in l)
