@@ -52,7 +52,10 @@ static inline int rs_prepare(hipStream_t st, const RsScratch &sc) {
   return fa_replicate((fa_stream_t)st, 4, sc.lookback, (int64_t)(sc.lookback_bytes / 4), 0);
 }
 
-// counts[d][tile] = number of keys of the tile whose digit is d.  A block
+// counts[d][tile] = number of keys of the tile whose digit is d.  The kernel
+// runs at the rate of LDS atomics (about one per nanosecond chip-wide, 72 us
+// per 2^26 keys); spreading each counter over 32 bank-private columns made no
+// difference, so the limit is the atomic unit and not bank conflicts.  A block
 // counts RS_HIST_TILES consecutive tiles, so that what it writes for a digit
 // is a run of RS_HIST_TILES counts (one 32-byte store) instead of single
 // 4-byte stores 4*num_tiles bytes apart, and the keys of the next tile are in
