@@ -83,15 +83,43 @@ template <class T, int Scope> struct AtomicUpdate<T, OpMin<T>, Scope> {
   }
 };
 
-// Update of a destination cell in HBM.  Float max/min use a compare-and-swap
-// loop on the operator itself, so that a NaN already in `dest` is replaced the
-// way fmax/fmin replace it (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:844-905).
+// Update of a bin in LDS.  For max and min the cell is read first and the
+// atomic issued only if the value would change it: bins are monotone, so a
+// stale read can only cause a redundant atomic, and after the first few
+// elements of a bin almost no update changes it (LDS atomics run at about a
+// quarter of the rate of LDS reads).  NaN values never change a bin (fmax/fmin
+// ignore them), and bins start from the identity, so they never hold NaN.
+template <class T, class Op>
+__device__ __forceinline__ void lds_update(T *p, T v) {
+  if constexpr (std::is_same<Op, OpAdd<T>>::value) {
+    AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(p, v);
+  } else {
+    const T cur = *reinterpret_cast<volatile T *>(p);
+    const bool changes = std::is_same<Op, OpMax<T>>::value ? (v > cur) : (v < cur);
+    if (changes) AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(p, v);
+  }
+}
+
+// Update of a destination cell in HBM.  For float max/min the integer view is
+// enough (one atomic without return) unless the cell holds a NaN, which fmax
+// and fmin replace by the other operand
+// (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:844-905 uses a compare-and-swap loop
+// on the operator for every update).  Nothing here ever writes a NaN, so a cell
+// seen without one never holds one later; a cell seen with one goes through a
+// compare-and-swap loop on the operator itself.
 template <class T, class Op>
 __device__ __forceinline__ void global_update(T *p, T v) {
   constexpr bool float_minmax = !std::is_integral<T>::value && !std::is_same<Op, OpAdd<T>>::value;
   if constexpr (float_minmax) {
     using U = typename SameSizeInt<T>::U;
     U *q = reinterpret_cast<U *>(p);
+    // An ordinary load is enough for the NaN test: a stale value can only be an
+    // earlier one, i.e. show a NaN that is gone by now, never hide one.
+    const T seen = *reinterpret_cast<const volatile T *>(p);
+    if (seen == seen) {
+      AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_AGENT>::apply(p, v);
+      return;
+    }
     U old = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     while (true) {
       const T want = Op::apply(bit_cast<T>(old), v);
@@ -153,7 +181,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
   auto update = [&](int64_t bin, T v) {
     const int64_t r = bin - lo;
     if ((uint64_t)r < (uint64_t)nb)
-      AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(&sh[((int)r << log2_copies) + copy], v);
+      lds_update<T, Op>(&sh[((int)r << log2_copies) + copy], v);
   };
   if (nb > 0) {
     for (int64_t i = s * HIST_BLOCK + threadIdx.x; i < nvec; i += stride) {
@@ -228,10 +256,10 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
       }
 #pragma unroll
       for (int q = 0; q < 4; q++)
-        AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(&sh[(int)((int64_t)b[q] - bin0)], v[q]);
+        lds_update<T, Op>(&sh[(int)((int64_t)b[q] - bin0)], v[q]);
     }
     for (; i < hi; i += HIST_BLOCK)
-      AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(&sh[(int)((int64_t)pis[i] - bin0)], pvs[i]);
+      lds_update<T, Op>(&sh[(int)((int64_t)pis[i] - bin0)], pvs[i]);
     __syncthreads();
     for (int q = threadIdx.x; q < nb; q += HIST_BLOCK) {
       const T acc = sh[q];
