@@ -138,6 +138,16 @@ def make_workload(name: str, ctx):
             ctx.call(f"bmm_{t}", ["f32_3d"], a, bb).free()
         w.update(step=step, flops=2 * b * m * m * m, kernel="segmap_matmul", dtype=t, bound="mfma",
                  keep=[a, bb], describe=f"batched matmul b={b} M=N=K={m}, {t} in, f32 accumulate")
+    elif name.startswith("transpose_"):
+        # transpose_f32_8192x8192
+        _, t, shape = name.split("_")
+        rows, cols = (int(x) for x in shape.split("x"))
+        x = ctx.new("f32_2d", dg.uniform_f32(90, rows * cols).reshape(rows, cols))
+
+        def step():
+            ctx.call("transpose_f32", ["f32_2d"], x).free()
+        w.update(step=step, bytes=2 * rows * cols * 4, kernel="map_transpose_4b", dtype=t, bound="hbm",
+                 keep=[x], describe=f"transpose of [{rows}][{cols}]{t} (map_transpose_4b)")
     else:
         raise SystemExit(f"unknown workload {name}")
     return w

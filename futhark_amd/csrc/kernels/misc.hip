@@ -1,7 +1,6 @@
 // Builtin data-movement kernels: replicate, iota, copy and the batched 2-D
-// transpose.  They stand where the reference keeps builtin#replicate_* /
-// builtin#iota_* (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:1274-1436) and
-// map_transpose_{1,2,4,8}b (rts/opencl/transpose.cl, dispatch rts/c/gpu.h:333-461).
+// copy.  They stand where the reference keeps builtin#replicate_* /
+// builtin#iota_* (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:1274-1436).
 #include "dispatch.hip.h"
 
 namespace fa {
@@ -40,48 +39,11 @@ __global__ void copy_tail_kernel(uint8_t *dst, const uint8_t *src, int64_t from,
   if (i < n) dst[i] = src[i];
 }
 
-// dst[b][j][i] = src[b][i][j].  A 64x64 tile goes through LDS; rows are padded
-// by one element so that the column reads fall on distinct banks.  Both the
-// global reads and the global writes of a wave touch 64 consecutive elements.
-template <class T>
-__global__ __launch_bounds__(256) void transpose_kernel(T *__restrict__ dst,
-                                                        const T *__restrict__ src, int64_t rows,
-                                                        int64_t cols) {
-  constexpr int TS = 64;
-  __shared__ T tile[TS][TS + 1];
-  const int64_t b = blockIdx.z;
-  const int64_t r0 = (int64_t)blockIdx.y * TS, c0 = (int64_t)blockIdx.x * TS;
-  const T *s = src + b * rows * cols;
-  T *d = dst + b * rows * cols;
-  const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;  // 64 x 4
-#pragma unroll 4
-  for (int i = ty; i < TS; i += 4) {
-    const int64_t r = r0 + i, c = c0 + tx;
-    if (r < rows && c < cols) tile[i][tx] = s[r * cols + c];
-  }
-  __syncthreads();
-#pragma unroll 4
-  for (int i = ty; i < TS; i += 4) {
-    const int64_t c = c0 + i, r = r0 + tx;
-    if (r < rows && c < cols) d[c * rows + r] = tile[tx][i];
-  }
-}
-
 static int grid_for(int64_t n, int per_block) {
   int64_t g = ceil_div(n, per_block);
   if (g < 1) g = 1;
   if (g > 256 * 16) g = 256 * 16;
   return (int)g;
-}
-
-template <class T>
-static int launch_transpose(hipStream_t s, void *dst, const void *src, int64_t batch,
-                            int64_t rows, int64_t cols) {
-  const int64_t gx = ceil_div(cols, 64), gy = ceil_div(rows, 64);
-  if (gx > INT32_MAX || gy > 65535 || batch > 65535) return FA_EINVAL;
-  hipLaunchKernelGGL((transpose_kernel<T>), dim3((unsigned)gx, (unsigned)gy, (unsigned)batch),
-                     dim3(256), 0, s, (T *)dst, (const T *)src, rows, cols);
-  return launch_status();
 }
 
 }  // namespace fa
@@ -135,21 +97,6 @@ extern "C" int fa_copy(fa_stream_t stream, void *dst, const void *src, size_t by
                        (const uint8_t *)src, nvec * 16, (int64_t)bytes);
   }
   return launch_status();
-}
-
-extern "C" int fa_map_transpose(fa_stream_t stream, int elem_bytes, void *dst, const void *src,
-                                int64_t batch, int64_t rows, int64_t cols) {
-  if (batch < 0 || rows < 0 || cols < 0) return FA_EINVAL;
-  if (batch * rows * cols == 0) return 0;
-  if (dst == nullptr || src == nullptr) return FA_EINVAL;
-  hipStream_t s = (hipStream_t)stream;
-  switch (elem_bytes) {
-    case 1: return launch_transpose<uint8_t>(s, dst, src, batch, rows, cols);
-    case 2: return launch_transpose<uint16_t>(s, dst, src, batch, rows, cols);
-    case 4: return launch_transpose<uint32_t>(s, dst, src, batch, rows, cols);
-    case 8: return launch_transpose<uint64_t>(s, dst, src, batch, rows, cols);
-    default: return FA_ENOTSUP;
-  }
 }
 
 extern "C" int fa_version(void) { return 1000; }

@@ -155,10 +155,25 @@ int fa_matmul(fa_stream_t stream, fa_dtype in_t,
 
 /* ------------------------------------------------ builtin data movement
  * Batched 2-D transpose: dst[b][j][i] = src[b][i][j], src : [batch][rows][cols].
- * Replaces: map_transpose_{1,2,4,8}b (rts/opencl/transpose.cl). */
+ * Replaces: map_transpose_{1,2,4,8}b and their low_height / low_width / small /
+ * large variants (rts/opencl/transpose.cl, chosen in rts/c/gpu.h:333-461). */
 int fa_map_transpose(fa_stream_t stream, int elem_bytes,
                      void *dst, const void *src,
                      int64_t batch, int64_t rows, int64_t cols);
+
+/* Copy between two index functions over the same shape:
+ *   dst[dst_offset + sum_k i_k*dst_strides[k]] = src[src_offset + sum_k i_k*src_strides[k]]
+ * for every index (i_0..i_{rank-1}) of `shape`; offsets and strides count
+ * elements of elem_bytes (1, 2, 4, 8) bytes, strides may be negative,
+ * rank <= 8.  The regions must not overlap.  The copy runs as a flat device
+ * copy, as a batched transpose or element by element, decided as the reference
+ * decides (rts/c/copy.h:55-190; lmad_copy_gpu2gpu_{1,2,4,8}b,
+ * rts/c/gpu.h:484-586); *path, if not NULL, says which. */
+enum { FA_LMAD_NOTHING = 0, FA_LMAD_FLAT = 1, FA_LMAD_TRANSPOSE = 2, FA_LMAD_GENERAL = 3 };
+int fa_lmad_copy(fa_stream_t stream, int elem_bytes,
+                 void *dst, int64_t dst_offset, const int64_t *dst_strides,
+                 const void *src, int64_t src_offset, const int64_t *src_strides,
+                 const int64_t *shape, int rank, int *path);
 
 /* Fill n elements of elem_bytes (1,2,4,8) each with the given bit pattern.
  * Replaces: builtin#replicate_* (ImpGen/GPU/Base.hs:1274-1350). */

@@ -169,6 +169,20 @@ def transpose_f32(x):
     return out
 
 
+def lmad_copy(dst, dst_offset, dst_strides, src, src_offset, src_strides, shape):
+    """In place on the flat numpy buffer `dst` (same dtype as `src`); strides in elements."""
+    assert dst.dtype == src.dtype and dst.flags.c_contiguous and src.flags.c_contiguous
+    r = len(shape)
+    I64 = C.c_int64 * max(r, 1)
+    fn = lib().orc_lmad_copy
+    fn.restype = None
+    fn.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p,
+                   C.c_void_p, C.c_int]
+    fn(dst.itemsize, _p(dst), dst_offset, I64(*dst_strides), _p(src), src_offset,
+       I64(*src_strides), I64(*shape), r)
+    return dst
+
+
 # ---- futhark-multicore-style CPU baseline (oracle/multicore.c) -------------
 def mc_threads() -> int:
     return int(lib().mc_num_threads())

@@ -291,6 +291,29 @@ void orc_radix_sort(const void *keys, void *keys_out, const void *vals, void *va
 }
 
 /* --------------------------------------------------------- data movement */
+/* LMAD copy, element by element in row-major index order: what the reference's
+ * generic copy does (rts/c/copy.h:35-53, lmad_copy_elements), for elements of
+ * any size.  Offsets and strides count elements. */
+static void orc_lmad_rec(int r, uint8_t *dst, const int64_t *dst_strides, const uint8_t *src,
+                         const int64_t *src_strides, const int64_t *shape, int64_t es) {
+  if (r == 0) {
+    memcpy(dst, src, (size_t)es);
+    return;
+  }
+  for (int64_t i = 0; i < shape[0]; i++)
+    orc_lmad_rec(r - 1, dst + i * dst_strides[0] * es, dst_strides + 1,
+                 src + i * src_strides[0] * es, src_strides + 1, shape + 1, es);
+}
+
+void orc_lmad_copy(int elem_bytes, void *dst, int64_t dst_offset, const int64_t *dst_strides,
+                   const void *src, int64_t src_offset, const int64_t *src_strides,
+                   const int64_t *shape, int rank) {
+  for (int i = 0; i < rank; i++)
+    if (shape[i] == 0) return;
+  orc_lmad_rec(rank, (uint8_t *)dst + dst_offset * elem_bytes, dst_strides,
+               (const uint8_t *)src + src_offset * elem_bytes, src_strides, shape, elem_bytes);
+}
+
 void orc_transpose_f32(const float *in, float *out, int64_t rows, int64_t cols) {
   for (int64_t i = 0; i < rows; i++)
     for (int64_t j = 0; j < cols; j++) out[j * rows + i] = in[i * cols + j];
