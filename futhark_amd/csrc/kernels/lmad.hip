@@ -111,6 +111,47 @@ __global__ __launch_bounds__(256) void transpose_tile_kernel(T *__restrict__ dst
   }
 }
 
+// The same tile with 16 bytes per lane on both global sides (V = 16 / sizeof(T)
+// elements): a lane loads V consecutive elements of a source row, and stores V
+// consecutive elements of a destination row, which it gathers from V source
+// rows of the LDS tile.  Needs rows and cols that are multiples of V and
+// 16-byte aligned bases.
+template <class T>
+__global__ __launch_bounds__(256) void transpose_tile_vec_kernel(T *__restrict__ dst,
+                                                                 const T *__restrict__ src,
+                                                                 int64_t rows, int64_t cols) {
+  constexpr int TS = 64;
+  constexpr int V = 16 / sizeof(T);
+  constexpr int LANES = TS / V;         // lanes across one tile row
+  constexpr int STEP = 256 / LANES;     // tile rows covered per pass
+  __shared__ T tile[TS][TS + 1];
+  const int64_t b = blockIdx.z;
+  const int64_t r0 = (int64_t)blockIdx.y * TS, c0 = (int64_t)blockIdx.x * TS;
+  const T *s = src + b * rows * cols;
+  T *d = dst + b * rows * cols;
+  const int tx = threadIdx.x % LANES, ty = threadIdx.x / LANES;
+#pragma unroll
+  for (int i = ty; i < TS; i += STEP) {
+    const int64_t r = r0 + i, c = c0 + tx * V;
+    if (r < rows && c < cols) {
+      const Vec16<T> v = load_vec16(s + r * cols + c);
+#pragma unroll
+      for (int e = 0; e < V; e++) tile[i][tx * V + e] = v.e[e];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = ty; i < TS; i += STEP) {
+    const int64_t c = c0 + i, r = r0 + tx * V;  // destination row c, columns r..r+V-1
+    if (r < rows && c < cols) {
+      Vec16<T> v;
+#pragma unroll
+      for (int e = 0; e < V; e++) v.e[e] = tile[tx * V + e][i];
+      store_vec16(d + c * rows + r, v);
+    }
+  }
+}
+
 template <class T>
 static int launch_map_transpose(hipStream_t st, T *dst, const T *src, int64_t batch, int64_t rows,
                                 int64_t cols) {
@@ -132,8 +173,14 @@ static int launch_map_transpose(hipStream_t st, T *dst, const T *src, int64_t ba
   }
   const int64_t gx = ceil_div(cols, (int64_t)64), gy = ceil_div(rows, (int64_t)64);
   if (gx > INT32_MAX || gy > 65535) return FA_EINVAL;
-  hipLaunchKernelGGL((transpose_tile_kernel<T>), dim3((unsigned)gx, (unsigned)gy, (unsigned)batch),
-                     dim3(256), 0, st, dst, src, rows, cols);
+  const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
+  constexpr int V = 16 / (int)sizeof(T);
+  if (sizeof(T) >= 4 && rows % V == 0 && cols % V == 0 && is_aligned(dst, 16) &&
+      is_aligned(src, 16))
+    hipLaunchKernelGGL((transpose_tile_vec_kernel<T>), grid, dim3(256), 0, st, dst, src, rows,
+                       cols);
+  else
+    hipLaunchKernelGGL((transpose_tile_kernel<T>), grid, dim3(256), 0, st, dst, src, rows, cols);
   return launch_status();
 }
 
