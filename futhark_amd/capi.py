@@ -26,6 +26,11 @@ ARRAY_TYPES = {
     "f16_3d": (np.uint16, 3), "u16_3d": (np.uint16, 3),
 }
 OPS = ("add", "max", "min")
+BITOPS = ("and", "or", "xor")  # integer types only
+
+
+def ops_for(t: str):
+    return OPS + BITOPS if t in ("i32", "i64") else OPS
 
 
 def lib_path(name: str = "libsegops.so") -> Path:
@@ -92,7 +97,7 @@ class Segops:
             sh.argtypes = [vp, vp]
         pp = C.POINTER(vp)
         for t in NUM_TYPES:
-            for op in OPS:
+            for op in ops_for(t):
                 getattr(L, f"futhark_entry_reduce_{op}_{t}").argtypes = [vp, vp, vp]
                 getattr(L, f"futhark_entry_scan_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_exscan_{op}_{t}").argtypes = [vp, pp, vp]

@@ -82,6 +82,26 @@ template <class T> struct OpMin {
   }
 };
 
+// Bitwise operators, integer types only (rts/c/scalar.h:521-534).
+template <class T> struct OpAnd {
+  static_assert(std::is_integral<T>::value, "bitwise and: integers only");
+  static constexpr bool commutative = true;
+  static __host__ __device__ __forceinline__ T identity() { return (T)~(T)0; }
+  static __host__ __device__ __forceinline__ T apply(T a, T b) { return a & b; }
+};
+template <class T> struct OpOr {
+  static_assert(std::is_integral<T>::value, "bitwise or: integers only");
+  static constexpr bool commutative = true;
+  static __host__ __device__ __forceinline__ T identity() { return (T)0; }
+  static __host__ __device__ __forceinline__ T apply(T a, T b) { return a | b; }
+};
+template <class T> struct OpXor {
+  static_assert(std::is_integral<T>::value, "bitwise xor: integers only");
+  static constexpr bool commutative = true;
+  static __host__ __device__ __forceinline__ T identity() { return (T)0; }
+  static __host__ __device__ __forceinline__ T apply(T a, T b) { return a ^ b; }
+};
+
 // ------------------------------------------------------- bit reinterpretation
 
 template <class To, class From>

@@ -12,6 +12,9 @@ using namespace fa;
         case FA_ADD: return FN<int32_t, OpAdd<int32_t>>(__VA_ARGS__);                \
         case FA_MAX: return FN<int32_t, OpMax<int32_t>>(__VA_ARGS__);                \
         case FA_MIN: return FN<int32_t, OpMin<int32_t>>(__VA_ARGS__);                \
+        case FA_AND: return FN<int32_t, OpAnd<int32_t>>(__VA_ARGS__);                \
+        case FA_OR: return FN<int32_t, OpOr<int32_t>>(__VA_ARGS__);                  \
+        case FA_XOR: return FN<int32_t, OpXor<int32_t>>(__VA_ARGS__);                \
         default: return FA_ENOTSUP;                                                  \
       }                                                                              \
     case FA_I64:                                                                     \
@@ -19,6 +22,9 @@ using namespace fa;
         case FA_ADD: return FN<int64_t, OpAdd<int64_t>>(__VA_ARGS__);                \
         case FA_MAX: return FN<int64_t, OpMax<int64_t>>(__VA_ARGS__);                \
         case FA_MIN: return FN<int64_t, OpMin<int64_t>>(__VA_ARGS__);                \
+        case FA_AND: return FN<int64_t, OpAnd<int64_t>>(__VA_ARGS__);                \
+        case FA_OR: return FN<int64_t, OpOr<int64_t>>(__VA_ARGS__);                  \
+        case FA_XOR: return FN<int64_t, OpXor<int64_t>>(__VA_ARGS__);                \
         default: return FA_ENOTSUP;                                                  \
       }                                                                              \
     case FA_U32:                                                                     \
@@ -26,6 +32,9 @@ using namespace fa;
         case FA_ADD: return FN<uint32_t, OpAdd<uint32_t>>(__VA_ARGS__);              \
         case FA_MAX: return FN<uint32_t, OpMax<uint32_t>>(__VA_ARGS__);              \
         case FA_MIN: return FN<uint32_t, OpMin<uint32_t>>(__VA_ARGS__);              \
+        case FA_AND: return FN<uint32_t, OpAnd<uint32_t>>(__VA_ARGS__);              \
+        case FA_OR: return FN<uint32_t, OpOr<uint32_t>>(__VA_ARGS__);                \
+        case FA_XOR: return FN<uint32_t, OpXor<uint32_t>>(__VA_ARGS__);              \
         default: return FA_ENOTSUP;                                                  \
       }                                                                              \
     case FA_U64:                                                                     \
@@ -33,6 +42,9 @@ using namespace fa;
         case FA_ADD: return FN<uint64_t, OpAdd<uint64_t>>(__VA_ARGS__);              \
         case FA_MAX: return FN<uint64_t, OpMax<uint64_t>>(__VA_ARGS__);              \
         case FA_MIN: return FN<uint64_t, OpMin<uint64_t>>(__VA_ARGS__);              \
+        case FA_AND: return FN<uint64_t, OpAnd<uint64_t>>(__VA_ARGS__);              \
+        case FA_OR: return FN<uint64_t, OpOr<uint64_t>>(__VA_ARGS__);                \
+        case FA_XOR: return FN<uint64_t, OpXor<uint64_t>>(__VA_ARGS__);              \
         default: return FA_ENOTSUP;                                                  \
       }                                                                              \
     case FA_F32:                                                                     \

@@ -76,6 +76,21 @@ template <class T, int Scope> struct AtomicUpdate<T, OpMax<T>, Scope> {
     else float_minmax_update<T, Scope, true>(p, v);
   }
 };
+template <class T, int Scope> struct AtomicUpdate<T, OpAnd<T>, Scope> {
+  static __device__ __forceinline__ void apply(T *p, T v) {
+    __hip_atomic_fetch_and(p, v, __ATOMIC_RELAXED, Scope);
+  }
+};
+template <class T, int Scope> struct AtomicUpdate<T, OpOr<T>, Scope> {
+  static __device__ __forceinline__ void apply(T *p, T v) {
+    __hip_atomic_fetch_or(p, v, __ATOMIC_RELAXED, Scope);
+  }
+};
+template <class T, int Scope> struct AtomicUpdate<T, OpXor<T>, Scope> {
+  static __device__ __forceinline__ void apply(T *p, T v) {
+    __hip_atomic_fetch_xor(p, v, __ATOMIC_RELAXED, Scope);
+  }
+};
 template <class T, int Scope> struct AtomicUpdate<T, OpMin<T>, Scope> {
   static __device__ __forceinline__ void apply(T *p, T v) {
     if constexpr (std::is_integral<T>::value) __hip_atomic_fetch_min(p, v, __ATOMIC_RELAXED, Scope);
@@ -91,7 +106,8 @@ template <class T, int Scope> struct AtomicUpdate<T, OpMin<T>, Scope> {
 // ignore them), and bins start from the identity, so they never hold NaN.
 template <class T, class Op>
 __device__ __forceinline__ void lds_update(T *p, T v) {
-  if constexpr (std::is_same<Op, OpAdd<T>>::value) {
+  constexpr bool minmax = std::is_same<Op, OpMax<T>>::value || std::is_same<Op, OpMin<T>>::value;
+  if constexpr (!minmax) {
     AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(p, v);
   } else {
     const T cur = *reinterpret_cast<volatile T *>(p);
@@ -109,7 +125,8 @@ __device__ __forceinline__ void lds_update(T *p, T v) {
 // compare-and-swap loop on the operator itself.
 template <class T, class Op>
 __device__ __forceinline__ void global_update(T *p, T v) {
-  constexpr bool float_minmax = !std::is_integral<T>::value && !std::is_same<Op, OpAdd<T>>::value;
+  constexpr bool float_minmax =
+      !std::is_integral<T>::value && (std::is_same<Op, OpMax<T>>::value || std::is_same<Op, OpMin<T>>::value);
   if constexpr (float_minmax) {
     using U = typename SameSizeInt<T>::U;
     U *q = reinterpret_cast<U *>(p);

@@ -212,7 +212,8 @@ static int bad_sizes(struct futhark_context *ctx, const char *entry) {
 }
 
 static const fa_dtype DT_i32 = FA_I32, DT_i64 = FA_I64, DT_f32 = FA_F32, DT_f64 = FA_F64;
-static const fa_op OP_add = FA_ADD, OP_max = FA_MAX, OP_min = FA_MIN;
+static const fa_op OP_add = FA_ADD, OP_max = FA_MAX, OP_min = FA_MIN, OP_and = FA_AND, OP_or = FA_OR,
+                   OP_xor = FA_XOR;
 
 static int do_reduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es, void *out,
                      const struct fut_array *in) {
@@ -313,6 +314,8 @@ static int do_segreduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_
 static uint64_t neutral_bits(fa_dtype t, fa_op op) {
   union { int32_t i; float f; uint32_t u; } b32;
   union { int64_t i; double f; uint64_t u; } b64;
+  if (op == FA_OR || op == FA_XOR) return 0;
+  if (op == FA_AND) return t == FA_I32 ? 0xffffffffull : ~0ull;
   switch (t) {
     case FA_I32:
       b32.i = op == FA_ADD ? 0 : (op == FA_MAX ? INT32_MIN : INT32_MAX);
@@ -453,6 +456,8 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
 
 #define DEFINE_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(DEFINE_SEGOP_ENTRIES, T, CT)
 FUTHARK_FOR_EACH_NUM_TYPE(DEFINE_FOR_TYPE)
+#define DEFINE_BITOPS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(DEFINE_SEGOP_ENTRIES, T, CT)
+FUTHARK_FOR_EACH_INT_TYPE(DEFINE_BITOPS_FOR_TYPE)
 
 /* ------------------------------------------------------------------ matmul */
 

@@ -193,6 +193,8 @@ struct entry {
   }
 #define SEGOP_ENTRY_FNS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(SEGOP_ENTRY_FNS, T, CT)
 FUTHARK_FOR_EACH_NUM_TYPE(SEGOP_ENTRY_FNS_FOR_TYPE)
+#define SEGOP_BITOP_FNS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(SEGOP_ENTRY_FNS, T, CT)
+FUTHARK_FOR_EACH_INT_TYPE(SEGOP_BITOP_FNS_FOR_TYPE)
 
 static int e_bmm_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_bmm_f32(c, (struct futhark_f32_3d **)&o->u.arr, ARRP(i[0]), ARRP(i[1]));
@@ -252,9 +254,11 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
   {"rbi_" #OP "_" #T, e_rbi_##OP##_##T, "[]" #T, 1, 3, {"[]" #T, "[]i32", "[]" #T}, {1, 0, 0},  \
    {HIST_PARAM, NULL}},
 #define SEGOP_ENTRY_ROWS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(SEGOP_ENTRY_ROWS, T, CT)
+#define SEGOP_BITOP_ROWS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(SEGOP_ENTRY_ROWS, T, CT)
 
 static const struct entry entries[] = {
     FUTHARK_FOR_EACH_NUM_TYPE(SEGOP_ENTRY_ROWS_FOR_TYPE)
+    FUTHARK_FOR_EACH_INT_TYPE(SEGOP_BITOP_ROWS_FOR_TYPE)
     {"bmm_f32", e_bmm_f32, "[][][]f32", 1, 2, {"[][][]f32", "[][][]f32"}, {0}, {NULL}},
     {"bmm_f16", e_bmm_f16, "[][][]f32", 1, 2, {"[][][]f16", "[][][]f16"}, {0}, {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {NULL}},

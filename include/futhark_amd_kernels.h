@@ -50,7 +50,8 @@ typedef enum {
  * Semantics are those of rts/c/scalar.h: two's-complement wrap-around add
  * (scalar.h:29-30), smax/smin (scalar.h:488-503), fmaxf/fminf, i.e. NaN-ignoring
  * (scalar.h:931-934). */
-typedef enum { FA_ADD = 0, FA_MAX = 1, FA_MIN = 2, FA_OP_COUNT } fa_op;
+/* FA_AND, FA_OR, FA_XOR: integer types only (neutral elements -1, 0, 0). */
+typedef enum { FA_ADD = 0, FA_MAX = 1, FA_MIN = 2, FA_AND = 3, FA_OR = 4, FA_XOR = 5, FA_OP_COUNT } fa_op;
 
 #define FA_EINVAL (-1)   /* bad argument (null pointer, negative size, ...) */
 #define FA_ENOTSUP (-2)  /* dtype/op combination not built */

@@ -35,7 +35,9 @@
  *   entry radix_sort_pairs_K_V (keys: []K) (vals: []V) : ([]K, []V)
  *   entry transpose_f32 (xss: [][]f32) : [][]f32 = transpose xss
  *
- * OP in {add, max, min}; NE = 0, T.lowest, T.highest; T in {i32, i64, f32, f64}.
+ * OP in {add, max, min}; NE = 0, T.lowest, T.highest; T in {i32, i64, f32, f64};
+ * for T in {i32, i64} also OP in {and, or, xor} with NE = -1, 0, 0
+ * (tests/hist/{and,or,xor}.fut).
  */
 #ifndef SEGOPS_H
 #define SEGOPS_H
@@ -210,6 +212,13 @@ FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
 
 #define FUTHARK_DECLARE_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(FUTHARK_DECLARE_SEGOP_ENTRIES, T, CT)
 FUTHARK_FOR_EACH_NUM_TYPE(FUTHARK_DECLARE_FOR_TYPE)
+
+/* The same eight entry points for the bitwise operators on the integer types. */
+#define FUTHARK_FOR_EACH_INT_TYPE(X) X(i32, int32_t) X(i64, int64_t)
+#define FUTHARK_FOR_EACH_BITOP(X, T, CT) X(and, T, CT) X(or, T, CT) X(xor, T, CT)
+#define FUTHARK_DECLARE_BITOPS_FOR_TYPE(T, CT) \
+  FUTHARK_FOR_EACH_BITOP(FUTHARK_DECLARE_SEGOP_ENTRIES, T, CT)
+FUTHARK_FOR_EACH_INT_TYPE(FUTHARK_DECLARE_BITOPS_FOR_TYPE)
 
 int futhark_entry_bmm_f32(struct futhark_context *ctx, struct futhark_f32_3d **out0,
                           const struct futhark_f32_3d *in0, const struct futhark_f32_3d *in1);

@@ -108,6 +108,8 @@ NEUTRAL = {
     ("add", "i64"): 0, ("max", "i64"): np.iinfo(np.int64).min, ("min", "i64"): np.iinfo(np.int64).max,
     ("add", "f32"): 0.0, ("max", "f32"): -np.inf, ("min", "f32"): np.inf,
     ("add", "f64"): 0.0, ("max", "f64"): -np.inf, ("min", "f64"): np.inf,
+    ("and", "i32"): -1, ("or", "i32"): 0, ("xor", "i32"): 0,
+    ("and", "i64"): -1, ("or", "i64"): 0, ("xor", "i64"): 0,
 }
 
 

@@ -33,7 +33,10 @@
 #define OPS_INT(T, U, S)                                                        \
   static inline T add_##S(T a, T b) { return (T)((U)a + (U)b); }                \
   static inline T max_##S(T a, T b) { return a < b ? b : a; }                   \
-  static inline T min_##S(T a, T b) { return a < b ? a : b; }
+  static inline T min_##S(T a, T b) { return a < b ? a : b; }                   \
+  static inline T and_##S(T a, T b) { return a & b; }                           \
+  static inline T or_##S(T a, T b) { return a | b; }                            \
+  static inline T xor_##S(T a, T b) { return a ^ b; }
 OPS_INT(int32_t, uint32_t, i32)
 OPS_INT(int64_t, uint64_t, i64)
 static inline float add_f32(float a, float b) { return a + b; }
@@ -50,6 +53,13 @@ static inline double min_f64(double a, double b) { return fmin(a, b); }
 #define NE_add_i64 0
 #define NE_max_i64 INT64_MIN
 #define NE_min_i64 INT64_MAX
+/* bitwise operators: -1, 0, 0 (tests/hist/and.fut:32, or.fut:32, xor.fut:32) */
+#define NE_and_i32 (-1)
+#define NE_or_i32 0
+#define NE_xor_i32 0
+#define NE_and_i64 (-1)
+#define NE_or_i64 0
+#define NE_xor_i64 0
 #define NE_add_f32 0.0f
 #define NE_max_f32 (-INFINITY)
 #define NE_min_f32 (INFINITY)
@@ -128,6 +138,9 @@ static inline double min_f64(double a, double b) { return fmin(a, b); }
 #define DEFINE_LIT_ALL_OPS(S, T) DEFINE_LIT(add, S, T) DEFINE_LIT(max, S, T) DEFINE_LIT(min, S, T)
 DEFINE_LIT_ALL_OPS(i32, int32_t)
 DEFINE_LIT_ALL_OPS(i64, int64_t)
+#define DEFINE_LIT_BITOPS(S, T) DEFINE_LIT(and, S, T) DEFINE_LIT(or, S, T) DEFINE_LIT(xor, S, T)
+DEFINE_LIT_BITOPS(i32, int32_t)
+DEFINE_LIT_BITOPS(i64, int64_t)
 DEFINE_LIT_ALL_OPS(f32, float)
 DEFINE_LIT_ALL_OPS(f64, double)
 

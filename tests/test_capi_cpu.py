@@ -10,7 +10,7 @@ from pathlib import Path
 import pytest
 
 from futhark_amd import Segops, Context, FutharkError, lib_path
-from futhark_amd.capi import ARRAY_TYPES, NUM_TYPES, OPS
+from futhark_amd.capi import ARRAY_TYPES, NUM_TYPES, OPS, ops_for
 
 ROOT = Path(__file__).resolve().parent.parent
 
@@ -44,7 +44,7 @@ def test_program_library_exports_the_generated_api():
         for f in ("new", "new_raw", "free", "values", "index", "values_raw", "shape"):
             declared.add(f"futhark_{f}_{kind}")
     for t in NUM_TYPES:
-        for op in OPS:
+        for op in ops_for(t):
             for e in ("reduce", "scan", "exscan", "segscan", "segred", "segreduce", "hist", "rbi"):
                 declared.add(f"futhark_entry_{e}_{op}_{t}")
     declared = {d for d in declared if not d.endswith("_")}

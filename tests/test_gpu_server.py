@@ -45,7 +45,7 @@ def test_introspection(srv):
     types = srv.cmd("types")
     assert {"i32", "[]f32", "[][]f32", "[][][]f16", "([]u32, []i32)"} <= set(types)
     entries = srv.cmd("entry_points")
-    assert len(entries) == 4 * 3 * 8 + 11 and "segscan_add_f32" in entries
+    assert len(entries) == (4 * 3 + 2 * 3) * 8 + 11 and "segscan_add_f32" in entries
     assert srv.cmd("inputs", "segscan_add_f32") == ["[]u8", "[]f32"]
     assert srv.cmd("output", "segscan_add_f32") == ["*[]f32"]
     assert srv.cmd("inputs", "rbi_add_i32") == ["*[]i32", "[]i32", "[]i32"]

@@ -54,6 +54,26 @@ def test_hist_simple_large_max_min(goldens):
             assert out.tolist() == c["out"]
 
 
+def test_hist_bitwise_operators(goldens):
+    # tests/hist/{and,or,xor,and64,xor64}.fut: neutral elements -1, 0, 0
+    for name in ("hist_and", "hist_or", "hist_xor", "hist_and64", "hist_xor64"):
+        op = name[5:].rstrip("64")
+        t = goldens[name]["type"]
+        for c in goldens[name]["cases"]:
+            out = oracle.hist(op, t, c["n"], c["is"], c["vs"])
+            assert out.tolist() == c["out"], (name, c)
+
+
+def test_bitwise_reductions_and_scans_match_numpy():
+    rng = np.random.default_rng(9)
+    for t, dt in (("i32", np.int32), ("i64", np.int64)):
+        xs = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, 1000, dtype=dt)
+        for op, uf in (("and", np.bitwise_and), ("or", np.bitwise_or), ("xor", np.bitwise_xor)):
+            assert oracle.reduce(op, t, xs) == uf.reduce(xs)
+            assert np.array_equal(oracle.scan(op, t, xs), uf.accumulate(xs))
+        assert oracle.reduce("and", t, xs[:0]) == -1 and oracle.reduce("xor", t, xs[:0]) == 0
+
+
 def test_hist_f32_including_nan(goldens):
     for c in goldens["hist_f32"]["cases"]:
         for variant in ("lit", "f64acc"):
