@@ -1,0 +1,56 @@
+"""Inputs with more than 2^31 elements: every index computation on the path has
+to be 64-bit (the reference sizes everything as i64, ImpGen/GPU/Base.hs).  The
+data follow closed forms, so the expected results need no second pass over
+17 GB on the host: xs[i] = (i mod 7) - 3 sums to 0 over every period, and its
+inclusive scan is P[i mod 7] with P = [-3, -5, -6, -6, -5, -3, 0]."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+N = (1 << 31) + 12345
+P = np.array([-3, -5, -6, -6, -5, -3, 0], np.int32)
+
+
+def _pattern(n):
+    xs = np.empty(n, np.int32)
+    step = 7 * (1 << 22)
+    block = (np.arange(step, dtype=np.int32) % 7 - 3).astype(np.int32)
+    for lo in range(0, n, step):
+        hi = min(lo + step, n)
+        xs[lo:hi] = block[: hi - lo]
+    return xs
+
+
+def test_reduce_and_scans_over_more_than_2p31_elements(ctx):
+    xs = _pattern(N)
+    a = ctx.new("i32_1d", xs)
+    del xs
+    want_sum = int(P[(N - 1) % 7])
+    assert ctx.call("reduce_add_i32", [np.int32], a) == want_sum
+    assert ctx.call("reduce_max_i32", [np.int32], a) == 3
+    out = ctx.call("scan_add_i32", ["i32_1d"], a)
+    got = out.values()
+    out.free()
+    # the far end in full, the rest at two million sampled positions (and the
+    # tile boundaries around 2^31)
+    tail = np.arange(N - (1 << 20), N, dtype=np.int64)
+    assert np.array_equal(got[tail], P[tail % 7])
+    rng = np.random.default_rng(1)
+    idx = np.concatenate([rng.integers(0, N, 2_000_000), np.arange((1 << 31) - 70000, (1 << 31) + 12345)])
+    assert np.array_equal(got[idx], P[idx % 7])
+    del got
+    # segmented: a segment start every 1000 elements; inside a segment the scan
+    # restarts, so the value depends on the position in the segment and the phase
+    flags = np.zeros(N, np.uint8)
+    flags[::1000] = 1
+    f = ctx.new("u8_1d", flags)
+    del flags
+    out = ctx.call("segscan_add_i32", ["i32_1d"], f, a)
+    got = out.values()
+    out.free(); f.free(); a.free()
+    idx = np.concatenate([rng.integers(0, N, 1_000_000), np.arange(N - 5000, N)])
+    start = idx - idx % 1000
+    # sum of xs[start..idx] = S(idx) - S(start - 1), S = the unsegmented scan
+    before = np.where(start > 0, P[(start - 1) % 7], 0)
+    assert np.array_equal(got[idx], P[idx % 7] - before)
