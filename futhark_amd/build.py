@@ -103,6 +103,13 @@ def build_server() -> Path:
     _run(["gcc", "-o", str(out), str(server_obj), str(values_obj), f"-L{LIB}", "-lsegops",
           "-lfuthark_amd_kernels", f"-L{ROCM / 'lib'}", "-lamdhip64", "-lm",
           "-Wl,-rpath,$ORIGIN/../lib", f"-Wl,-rpath,{ROCM / 'lib'}"])
+    # A C program written against the public header only, the way a user of a
+    # generated library writes one (run by tests/test_capi_harness.py).
+    harness = bindir / "capi-harness"
+    _run(["gcc", "-O1", "-std=c99", "-Wall", "-Wextra", f"-I{ROOT / 'include'}",
+          str(ROOT / "tests" / "c" / "capi_harness.c"), "-o", str(harness), f"-L{LIB}", "-lsegops",
+          "-lfuthark_amd_kernels", f"-L{ROCM / 'lib'}", "-lamdhip64", "-lpthread",
+          "-Wl,-rpath,$ORIGIN/../lib", f"-Wl,-rpath,{ROCM / 'lib'}"])
     return out
 
 
