@@ -197,11 +197,13 @@ MEASURED_TRAFFIC_BYTES = {
     "segscan_add_f32_2p26": 606.0e6,
     "scan_add_f32_2p26": 539.3e6,
     "reduce_add_f32_2p26": 268.5e6,
-    "segred_add_f32_2p26": 275.1e6,
+    "segred_add_f32_2p26": 283.3e6,
     "hist_add_i32_H256_uniform_2p27": 1074.2e6,
     "hist_add_i32_H65536_uniform_2p27": 1107.6e6,
     "hist_add_i32_H4194304_uniform_2p27": 4229.0e6,
     "sort_u32_2p26": 4088.4e6,
+    "hist_max_f32_H256_uniform_2p27": 1074.5e6,
+    "transpose_f32_8192x8192": 536.9e6,
 }
 
 
