@@ -90,12 +90,21 @@ def make_workload(name: str, ctx):
         _, op, t, hs, dist, sz = name.split("_")
         n, H = 1 << int(sz[2:]), int(hs[1:])
         is_ = dg.hist_indices(48, n, H, dist)
-        vs = dg.uniform_int(49, n, -1000, 1000) if t == "i32" else dg.uniform_f32(50, n)
+        if t == "f16":
+            vs, es = dg.to_f16_bits(dg.uniform_f32(50, n)), 2
+        elif t[0] == "f":
+            vs = dg.uniform_f32(50, n).astype(np.dtype(f"float{t[1:]}"))
+            es = vs.itemsize
+        else:
+            dt = np.dtype(("int" if t[0] == "i" else "uint") + t[1:])
+            lo, hi = (-1000, 1000) if dt.itemsize >= 4 and t[0] == "i" else (0, 100)
+            vs = dg.uniform_int(49, n, lo, hi).astype(dt)
+            es = dt.itemsize
         i, v = ctx.new("i32_1d", is_), ctx.new(f"{t}_1d", vs)
 
         def step():
             ctx.call(f"hist_{op}_{t}", [f"{t}_1d"], H, i, v).free()
-        w.update(step=step, bytes=n * 8 + 2 * H * 4, kernel="seghist", dtype=t, bound="hbm",
+        w.update(step=step, bytes=n * (4 + es) + 2 * H * es, kernel="seghist", dtype=t, bound="hbm",
                  keep=[i, v], describe=f"hist ({op}) of 2^{sz[2:]} {t} into {H} bins, {dist} i32 "
                                        f"indices, 1% out of range")
         if t == "i32" and op == "add":

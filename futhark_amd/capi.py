@@ -24,13 +24,19 @@ ARRAY_TYPES = {
     "f64_1d": (np.float64, 1), "i32_2d": (np.int32, 2), "i64_2d": (np.int64, 2),
     "f32_2d": (np.float32, 2), "f64_2d": (np.float64, 2), "f32_3d": (np.float32, 3),
     "f16_3d": (np.uint16, 3), "u16_3d": (np.uint16, 3),
+    "i8_1d": (np.int8, 1), "i16_1d": (np.int16, 1), "u16_1d": (np.uint16, 1),
+    "f16_1d": (np.uint16, 1),  # f16 crosses the API as its bits
 }
 OPS = ("add", "max", "min")
 BITOPS = ("and", "or", "xor")  # integer types only
 
 
+# element types that only hist_OP_T and rbi_OP_T exist for
+HIST_ONLY_TYPES = ("i8", "u8", "i16", "u16", "u32", "u64", "f16")
+
+
 def ops_for(t: str):
-    return OPS + BITOPS if t in ("i32", "i64") else OPS
+    return OPS + BITOPS if t[0] in "iu" else OPS
 
 
 def lib_path(name: str = "libsegops.so") -> Path:
@@ -104,6 +110,10 @@ class Segops:
                 getattr(L, f"futhark_entry_segscan_{op}_{t}").argtypes = [vp, pp, vp, vp]
                 getattr(L, f"futhark_entry_segred_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
                 getattr(L, f"futhark_entry_segreduce_{op}_{t}").argtypes = [vp, pp, vp]
+                getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
+                getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
+        for t in HIST_ONLY_TYPES:
+            for op in ops_for(t):
                 getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
                 getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
         for e in ("bmm_f32", "bmm_f16", "bmm_bf16", "matmul_f32"):

@@ -139,6 +139,8 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__
 
 template <int BYTES> struct ValType;
 template <> struct ValType<0> { using T = uint32_t; };
+template <> struct ValType<1> { using T = uint8_t; };
+template <> struct ValType<2> { using T = uint16_t; };
 template <> struct ValType<4> { using T = uint32_t; };
 template <> struct ValType<8> { using T = uint64_t; };
 

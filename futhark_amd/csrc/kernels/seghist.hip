@@ -32,6 +32,31 @@ constexpr int HIST_LDS_BYTES = 128 * 1024;  // bin storage per block
 constexpr int HIST_MAX_RANGES = 4;          // ranges covered by one launch
 constexpr int NUM_XCDS = 8;
 
+// ------------------------------------------------------------ element types
+// Bins of 8- and 16-bit element types are accumulated in LDS as 32-bit cells
+// (integers sign- or zero-extended, f16 as f32): LDS atomics exist for 32 and 64
+// bits only, and src/Futhark/CodeGen/ImpGen/GPU/Base.hs:735-767 with
+// rts/c/atomics8.h / atomics16.h emulates the narrow ones by compare-and-swap on
+// the containing word for every update.  Here only the flush of a bin to the
+// destination does that.  For the integer operators the narrowed wide result
+// equals the narrow evaluation (add wraps modulo 2^8 / 2^16 either way; max,
+// min, and, or, xor commute with the extension); f16 sums are rounded once per
+// block and bin instead of once per element.
+template <class T> struct HistAcc { using A = T; };
+template <> struct HistAcc<int8_t> { using A = int32_t; };
+template <> struct HistAcc<uint8_t> { using A = uint32_t; };
+template <> struct HistAcc<int16_t> { using A = int32_t; };
+template <> struct HistAcc<uint16_t> { using A = uint32_t; };
+template <> struct HistAcc<_Float16> { using A = float; };
+
+template <class Op, class A> struct RebindOp;
+template <class T, class A> struct RebindOp<OpAdd<T>, A> { using type = OpAdd<A>; };
+template <class T, class A> struct RebindOp<OpMax<T>, A> { using type = OpMax<A>; };
+template <class T, class A> struct RebindOp<OpMin<T>, A> { using type = OpMin<A>; };
+template <class T, class A> struct RebindOp<OpAnd<T>, A> { using type = OpAnd<A>; };
+template <class T, class A> struct RebindOp<OpOr<T>, A> { using type = OpOr<A>; };
+template <class T, class A> struct RebindOp<OpXor<T>, A> { using type = OpXor<A>; };
+
 // ------------------------------------------------------------ atomic updates
 // `Scope` is __HIP_MEMORY_SCOPE_WORKGROUP for LDS and _AGENT for HBM.
 
@@ -151,18 +176,57 @@ __device__ __forceinline__ void global_update(T *p, T v) {
   }
 }
 
+// Destination cells narrower than 32 bits: compare-and-swap on the aligned word
+// that contains the cell (rts/c/atomics8.h, atomics16.h do the same); `v` is
+// the block's partial result in the accumulation type.
+template <class T, class OpA, class A>
+__device__ __forceinline__ void global_update_narrow(T *p, A v) {
+  static_assert(sizeof(T) < 4, "narrow cells only");
+  using B = typename std::conditional<sizeof(T) == 1, uint8_t, uint16_t>::type;
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(p);
+  uint32_t *word = reinterpret_cast<uint32_t *>(addr & ~(uintptr_t)3);
+  const int shift = (int)(addr & 3) * 8;
+  const uint32_t mask = (uint32_t)(B)~(B)0 << shift;
+  uint32_t old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  while (true) {
+    const T cur = bit_cast<T>((B)(old >> shift));
+    const T want = (T)OpA::apply((A)cur, v);
+    const uint32_t wbits = (old & ~mask) | ((uint32_t)bit_cast<B>(want) << shift);
+    if (wbits == old) break;
+    if (__hip_atomic_compare_exchange_strong(word, &old, wbits, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT))
+      break;
+  }
+}
+
+// Combines the partial result `acc` of a block into destination cell *p.
+template <class T, class OpA, class A>
+__device__ __forceinline__ void flush_bin(T *p, A acc) {
+  if constexpr (sizeof(T) < 4) global_update_narrow<T, OpA, A>(p, acc);
+  else global_update<T, OpA>(p, acc);
+}
+
 template <class T> __device__ __forceinline__ bool bits_equal(T a, T b) {
   if constexpr (sizeof(T) == 4) return bit_cast<uint32_t>(a) == bit_cast<uint32_t>(b);
   else return bit_cast<uint64_t>(a) == bit_cast<uint64_t>(b);
 }
 
-// Four consecutive elements with 16-byte loads (pointers are 16-byte aligned).
+// Four consecutive elements with the widest loads that fit (src is aligned to
+// 4 * sizeof(E) bytes).
 template <class E> __device__ __forceinline__ void load_elems4(E (&dst)[4], const E *src) {
-  constexpr int NV = (int)(4 * sizeof(E) / 16);
-  uint4 raw[NV];
+  if constexpr (sizeof(E) == 1) {
+    const uint32_t raw = *reinterpret_cast<const uint32_t *>(src);
+    __builtin_memcpy(dst, &raw, 4);
+  } else if constexpr (sizeof(E) == 2) {
+    const uint2 raw = *reinterpret_cast<const uint2 *>(src);
+    __builtin_memcpy(dst, &raw, 8);
+  } else {
+    constexpr int NV = (int)(4 * sizeof(E) / 16);
+    uint4 raw[NV];
 #pragma unroll
-  for (int q = 0; q < NV; q++) raw[q] = reinterpret_cast<const uint4 *>(src)[q];
-  __builtin_memcpy(dst, raw, sizeof(raw));
+    for (int q = 0; q < NV; q++) raw[q] = reinterpret_cast<const uint4 *>(src)[q];
+    __builtin_memcpy(dst, raw, sizeof(raw));
+  }
 }
 
 // ------------------------------------------------------------- LDS histogram
@@ -173,8 +237,10 @@ template <class T, class Op, class I>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
     const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t bin_base,
     int64_t H, int range_bins, int P, int log2_copies) {
+  using A = typename HistAcc<T>::A;
+  using OpA = typename RebindOp<Op, A>::type;
   extern __shared__ __align__(16) unsigned char s_raw[];
-  T *sh = reinterpret_cast<T *>(s_raw);
+  A *sh = reinterpret_cast<A *>(s_raw);
   constexpr int VEC = 4;  // elements per thread per step
 
   const int b = blockIdx.x;
@@ -189,7 +255,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
   const int C = 1 << log2_copies;
   const int cells = nb * C;
 
-  for (int i = threadIdx.x; i < cells; i += HIST_BLOCK) sh[i] = Op::identity();
+  for (int i = threadIdx.x; i < cells; i += HIST_BLOCK) sh[i] = OpA::identity();
   __syncthreads();
 
   const int copy = threadIdx.x & (C - 1);
@@ -198,7 +264,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
   auto update = [&](int64_t bin, T v) {
     const int64_t r = bin - lo;
     if ((uint64_t)r < (uint64_t)nb)
-      lds_update<T, Op>(&sh[((int)r << log2_copies) + copy], v);
+      lds_update<A, OpA>(&sh[((int)r << log2_copies) + copy], (A)v);
   };
   if (nb > 0) {
     for (int64_t i = s * HIST_BLOCK + threadIdx.x; i < nvec; i += stride) {
@@ -218,9 +284,9 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
 
   // Flush: combine the copies of a bin in copy order, skip untouched bins.
   for (int r = threadIdx.x; r < nb; r += HIST_BLOCK) {
-    T acc = sh[r << log2_copies];
-    for (int c = 1; c < C; c++) acc = Op::apply(acc, sh[(r << log2_copies) + c]);
-    if (!bits_equal(acc, Op::identity())) global_update<T, Op>(dest + (lo - bin_base) + r, acc);
+    A acc = sh[r << log2_copies];
+    for (int c = 1; c < C; c++) acc = OpA::apply(acc, sh[(r << log2_copies) + c]);
+    if (!bits_equal(acc, OpA::identity())) flush_bin<T, OpA, A>(dest + (lo - bin_base) + r, acc);
   }
 }
 
@@ -243,8 +309,10 @@ template <class T, class Op, class U>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
     const U *__restrict__ pis, const T *__restrict__ pvs, const uint32_t *__restrict__ offs,
     int64_t num_tiles, T *dest, int64_t H, int shift) {
+  using A = typename HistAcc<T>::A;
+  using OpA = typename RebindOp<Op, A>::type;
   extern __shared__ __align__(16) unsigned char s_raw[];
-  T *sh = reinterpret_cast<T *>(s_raw);
+  A *sh = reinterpret_cast<A *>(s_raw);
   __shared__ uint32_t s_start[RS_RADIX];
   if (threadIdx.x < RS_RADIX) s_start[threadIdx.x] = offs[(int64_t)threadIdx.x * num_tiles];
   __syncthreads();
@@ -260,7 +328,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
     if (lo >= hi) continue;  // uniform over the block
     const int64_t bin0 = (int64_t)r << shift;
     const int nb = (int)((H - bin0) < range_bins ? (H - bin0) : range_bins);
-    for (int i = threadIdx.x; i < nb; i += HIST_BLOCK) sh[i] = Op::identity();
+    for (int i = threadIdx.x; i < nb; i += HIST_BLOCK) sh[i] = OpA::identity();
     __syncthreads();
     int64_t i = lo + threadIdx.x;
     for (; i + 3 * HIST_BLOCK < hi; i += 4 * HIST_BLOCK) {
@@ -273,14 +341,14 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
       }
 #pragma unroll
       for (int q = 0; q < 4; q++)
-        lds_update<T, Op>(&sh[(int)((int64_t)b[q] - bin0)], v[q]);
+        lds_update<A, OpA>(&sh[(int)((int64_t)b[q] - bin0)], (A)v[q]);
     }
     for (; i < hi; i += HIST_BLOCK)
-      lds_update<T, Op>(&sh[(int)((int64_t)pis[i] - bin0)], pvs[i]);
+      lds_update<A, OpA>(&sh[(int)((int64_t)pis[i] - bin0)], (A)pvs[i]);
     __syncthreads();
     for (int q = threadIdx.x; q < nb; q += HIST_BLOCK) {
-      const T acc = sh[q];
-      if (!bits_equal(acc, Op::identity())) global_update<T, Op>(dest + bin0 + q, acc);
+      const A acc = sh[q];
+      if (!bits_equal(acc, OpA::identity())) flush_bin<T, OpA, A>(dest + bin0 + q, acc);
     }
     __syncthreads();
   }
@@ -294,7 +362,9 @@ __global__ __launch_bounds__(256) void seghist_global_kernel(const I *__restrict
   const int64_t stride = (int64_t)gridDim.x * 256;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
     const int64_t bin = (int64_t)is[i];
-    if ((uint64_t)bin < (uint64_t)H) global_update<T, Op>(dest + bin, vs[i]);
+    if ((uint64_t)bin < (uint64_t)H)
+      flush_bin<T, typename RebindOp<Op, typename HistAcc<T>::A>::type, typename HistAcc<T>::A>(
+          dest + bin, (typename HistAcc<T>::A)vs[i]);
   }
 }
 
@@ -313,13 +383,14 @@ static int hist_num_cus() {
 template <class T, class Op, class I>
 static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
                            int64_t H) {
-  const int max_range = HIST_LDS_BYTES / (int)sizeof(T);
+  using A = typename HistAcc<T>::A;
+  const int max_range = HIST_LDS_BYTES / (int)sizeof(A);
   const int P = (int)ceil_div(H, max_range);
   const int range_bins = (int)ceil_div(H, P);
   int log2_copies = 0;
-  while (log2_copies < 5 && (int64_t)range_bins * (2 << log2_copies) * (int64_t)sizeof(T) <= 32 * 1024)
+  while (log2_copies < 5 && (int64_t)range_bins * (2 << log2_copies) * (int64_t)sizeof(A) <= 32 * 1024)
     log2_copies++;
-  const size_t lds = (size_t)range_bins * sizeof(T) << log2_copies;
+  const size_t lds = (size_t)range_bins * sizeof(A) << log2_copies;
   // One block per CU when the range fills LDS, two when two fit.
   const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
   int grid = hist_num_cus() * per_cu;
@@ -339,7 +410,7 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
 }
 
 template <class T> constexpr int hist_part_shift() {
-  return sizeof(T) == 4 ? 15 : 14;  // 128 KiB of bins per range
+  return sizeof(typename HistAcc<T>::A) == 4 ? 15 : 14;  // 128 KiB of bins per range
 }
 
 static size_t hist_align(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -379,7 +450,8 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
                        void *dest, int64_t H, void *scratch, size_t scratch_bytes) {
   if (H == 0 || n == 0) return 0;
   if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
-  const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)sizeof(T));
+  const int64_t lds_limit =
+      (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)sizeof(typename HistAcc<T>::A));
   if (H <= lds_limit) {
     if (is64) return launch_lds_hist<T, Op, int64_t>(st, (const int64_t *)is, (const T *)vs, n, (T *)dest, H);
     return launch_lds_hist<T, Op, int32_t>(st, (const int32_t *)is, (const T *)vs, n, (T *)dest, H);
@@ -406,10 +478,11 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
 
 extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int64_t H) {
   const size_t es = dtype_size(t);
-  if (es != 4 && es != 8) return 0;
+  if (es == 0) return 0;
+  const size_t as = es < 4 ? 4 : es;  // size of the accumulation type
   if (n < 0) n = 0;
-  const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)es);
-  const int64_t part_limit = (int64_t)255 << (es == 4 ? 15 : 14);
+  const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)as);
+  const int64_t part_limit = (int64_t)255 << (as == 4 ? 15 : 14);
   if (H <= lds_limit || H > part_limit) return 256;
   return hist_align(rs_scratch_bytes(rs_num_tiles(n))) +
          hist_align((size_t)n * (is64 ? 8 : 4)) + (size_t)n * es + 256;
@@ -421,14 +494,33 @@ extern "C" int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op, const void *
   if (n < 0 || H < 0 || (H > 0 && dest == nullptr) || (n > 0 && (is == nullptr || vs == nullptr)))
     return FA_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  switch (t) {
-    case FA_I32:
-    case FA_I64:
-    case FA_F32:
-    case FA_F64:
-      break;
-    default:
-      return FA_ENOTSUP;
+#define FA_HIST_NARROW_INT(T)                                                                      \
+  switch (op) {                                                                                    \
+    case FA_ADD: return launch_hist<T, OpAdd<T>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes); \
+    case FA_MAX: return launch_hist<T, OpMax<T>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes); \
+    case FA_MIN: return launch_hist<T, OpMin<T>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes); \
+    case FA_AND: return launch_hist<T, OpAnd<T>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes); \
+    case FA_OR: return launch_hist<T, OpOr<T>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes);  \
+    case FA_XOR: return launch_hist<T, OpXor<T>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes); \
+    default: return FA_ENOTSUP;                                                                    \
   }
+  switch (t) {
+    case FA_I8: FA_HIST_NARROW_INT(int8_t)
+    case FA_U8: FA_HIST_NARROW_INT(uint8_t)
+    case FA_I16: FA_HIST_NARROW_INT(int16_t)
+    case FA_U16: FA_HIST_NARROW_INT(uint16_t)
+    case FA_F16:
+      switch (op) {
+        case FA_ADD: return launch_hist<_Float16, OpAdd<_Float16>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes);
+        case FA_MAX: return launch_hist<_Float16, OpMax<_Float16>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes);
+        case FA_MIN: return launch_hist<_Float16, OpMin<_Float16>>(s, is, is64, vs, n, dest, H, scratch, scratch_bytes);
+        default: return FA_ENOTSUP;
+      }
+    case FA_BF16:
+      return FA_ENOTSUP;
+    default:
+      break;
+  }
+#undef FA_HIST_NARROW_INT
   FA_DISPATCH_TYPE_OP(launch_hist, t, op, s, is, is64, vs, n, dest, H, scratch, scratch_bytes);
 }

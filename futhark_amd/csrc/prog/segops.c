@@ -170,7 +170,11 @@ static int array_index(struct futhark_context *ctx, void *out, struct fut_array 
 
 DEFINE_ARRAY(i32, int32_t, 1)
 DEFINE_ARRAY(i64, int64_t, 1)
+DEFINE_ARRAY(i8, int8_t, 1)
+DEFINE_ARRAY(i16, int16_t, 1)
 DEFINE_ARRAY(u8, uint8_t, 1)
+DEFINE_ARRAY(u16, uint16_t, 1)
+DEFINE_ARRAY(f16, uint16_t, 1)
 DEFINE_ARRAY(u32, uint32_t, 1)
 DEFINE_ARRAY(u64, uint64_t, 1)
 DEFINE_ARRAY(f32, float, 1)
@@ -211,7 +215,9 @@ static int bad_sizes(struct futhark_context *ctx, const char *entry) {
   return 1;
 }
 
-static const fa_dtype DT_i32 = FA_I32, DT_i64 = FA_I64, DT_f32 = FA_F32, DT_f64 = FA_F64;
+static const fa_dtype DT_i32 = FA_I32, DT_i64 = FA_I64, DT_f32 = FA_F32, DT_f64 = FA_F64,
+                      DT_i8 = FA_I8, DT_u8 = FA_U8, DT_i16 = FA_I16, DT_u16 = FA_U16,
+                      DT_u32 = FA_U32, DT_u64 = FA_U64, DT_f16 = FA_F16;
 static const fa_op OP_add = FA_ADD, OP_max = FA_MAX, OP_min = FA_MIN, OP_and = FA_AND, OP_or = FA_OR,
                    OP_xor = FA_XOR;
 
@@ -311,23 +317,30 @@ static int do_segreduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_
   return 0;
 }
 
+/* Bit pattern of the neutral element: 0 for add, or, xor; all ones for and;
+ * T.lowest / T.highest for max / min (prelude/math.fut: the smallest / largest
+ * integer of the type, -inf / +inf for floats). */
 static uint64_t neutral_bits(fa_dtype t, fa_op op) {
-  union { int32_t i; float f; uint32_t u; } b32;
-  union { int64_t i; double f; uint64_t u; } b64;
-  if (op == FA_OR || op == FA_XOR) return 0;
-  if (op == FA_AND) return t == FA_I32 ? 0xffffffffull : ~0ull;
+  union { float f; uint32_t u; } b32;
+  union { double f; uint64_t u; } b64;
+  if (op == FA_ADD || op == FA_OR || op == FA_XOR) return 0;
+  if (op == FA_AND) return ~0ull; /* truncated to the element size by the fill */
+  const int max = op == FA_MAX;
   switch (t) {
-    case FA_I32:
-      b32.i = op == FA_ADD ? 0 : (op == FA_MAX ? INT32_MIN : INT32_MAX);
-      return b32.u;
+    case FA_I8: return (uint8_t)(max ? INT8_MIN : INT8_MAX);
+    case FA_I16: return (uint16_t)(max ? INT16_MIN : INT16_MAX);
+    case FA_I32: return (uint32_t)(max ? INT32_MIN : INT32_MAX);
+    case FA_I64: return (uint64_t)(max ? INT64_MIN : INT64_MAX);
+    case FA_U8: return max ? 0 : UINT8_MAX;
+    case FA_U16: return max ? 0 : UINT16_MAX;
+    case FA_U32: return max ? 0 : UINT32_MAX;
+    case FA_U64: return max ? 0 : UINT64_MAX;
+    case FA_F16: return max ? 0xFC00u : 0x7C00u;
     case FA_F32:
-      b32.f = op == FA_ADD ? 0.0f : (op == FA_MAX ? -__builtin_inff() : __builtin_inff());
+      b32.f = max ? -__builtin_inff() : __builtin_inff();
       return b32.u;
-    case FA_I64:
-      b64.i = op == FA_ADD ? 0 : (op == FA_MAX ? INT64_MIN : INT64_MAX);
-      return b64.u;
     default:
-      b64.f = op == FA_ADD ? 0.0 : (op == FA_MAX ? -__builtin_inf() : __builtin_inf());
+      b64.f = max ? -__builtin_inf() : __builtin_inf();
       return b64.u;
   }
 }
@@ -432,6 +445,9 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }                                                                                           \
+  DEFINE_HIST_ENTRIES(OP, T, CT)
+
+#define DEFINE_HIST_ENTRIES(OP, T, CT)                                                        \
   int futhark_entry_hist_##OP##_##T(struct futhark_context *ctx,                              \
                                     struct futhark_##T##_1d **out0, const int64_t in0,        \
                                     const struct futhark_i32_1d *in1,                         \
@@ -458,6 +474,11 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
 FUTHARK_FOR_EACH_NUM_TYPE(DEFINE_FOR_TYPE)
 #define DEFINE_BITOPS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(DEFINE_SEGOP_ENTRIES, T, CT)
 FUTHARK_FOR_EACH_INT_TYPE(DEFINE_BITOPS_FOR_TYPE)
+#define DEFINE_HIST_ONLY_INT(T, CT)                  \
+  FUTHARK_FOR_EACH_OP(DEFINE_HIST_ENTRIES, T, CT)    \
+  FUTHARK_FOR_EACH_BITOP(DEFINE_HIST_ENTRIES, T, CT)
+FUTHARK_FOR_EACH_HIST_ONLY_INT_TYPE(DEFINE_HIST_ONLY_INT)
+FUTHARK_FOR_EACH_OP(DEFINE_HIST_ENTRIES, f16, uint16_t)
 
 /* ------------------------------------------------------------------ matmul */
 

@@ -86,6 +86,7 @@ struct stype {
 #define A3(N, CT) ARRAY_SHIMS_3D(N, CT) ARRAY_SHIMS_COMMON(N, 3d)
 A1(i32, int32_t) A1(i64, int64_t) A1(u8, uint8_t) A1(u32, uint32_t) A1(u64, uint64_t)
 A1(f32, float) A1(f64, double)
+A1(i8, int8_t) A1(i16, int16_t) A1(u16, uint16_t) A1(f16, uint16_t)
 A2(i32, int32_t) A2(i64, int64_t) A2(f32, float) A2(f64, double)
 A3(f32, float) A3(f16, uint16_t) A3(u16, uint16_t)
 
@@ -102,6 +103,8 @@ static const struct stype types[] = {
     ARR("[]u8", "u8", 1, u8, 1d), ARR("[]u32", "u32", 1, u32, 1d),
     ARR("[]u64", "u64", 1, u64, 1d), ARR("[]f32", "f32", 1, f32, 1d),
     ARR("[]f64", "f64", 1, f64, 1d),
+    ARR("[]i8", "i8", 1, i8, 1d), ARR("[]i16", "i16", 1, i16, 1d),
+    ARR("[]u16", "u16", 1, u16, 1d), ARR("[]f16", "f16", 1, f16, 1d),
     ARR("[][]i32", "i32", 2, i32, 2d), ARR("[][]i64", "i64", 2, i64, 2d),
     ARR("[][]f32", "f32", 2, f32, 2d), ARR("[][]f64", "f64", 2, f64, 2d),
     ARR("[][][]f32", "f32", 3, f32, 3d), ARR("[][][]f16", "f16", 3, f16, 3d),
@@ -183,6 +186,8 @@ struct entry {
     return futhark_entry_segreduce_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,        \
                                               ARRP(i[0]));                                     \
   }                                                                                            \
+  HIST_ENTRY_FNS(OP, T, CT)
+#define HIST_ENTRY_FNS(OP, T, CT)                                                              \
   static int e_hist_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) { \
     return futhark_entry_hist_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,             \
                                          i[0]->u.i64, ARRP(i[1]), ARRP(i[2]));                 \
@@ -195,6 +200,10 @@ struct entry {
 FUTHARK_FOR_EACH_NUM_TYPE(SEGOP_ENTRY_FNS_FOR_TYPE)
 #define SEGOP_BITOP_FNS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(SEGOP_ENTRY_FNS, T, CT)
 FUTHARK_FOR_EACH_INT_TYPE(SEGOP_BITOP_FNS_FOR_TYPE)
+#define HIST_ONLY_INT_FNS(T, CT) \
+  FUTHARK_FOR_EACH_OP(HIST_ENTRY_FNS, T, CT) FUTHARK_FOR_EACH_BITOP(HIST_ENTRY_FNS, T, CT)
+FUTHARK_FOR_EACH_HIST_ONLY_INT_TYPE(HIST_ONLY_INT_FNS)
+FUTHARK_FOR_EACH_OP(HIST_ENTRY_FNS, f16, uint16_t)
 
 static int e_bmm_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_bmm_f32(c, (struct futhark_f32_3d **)&o->u.arr, ARRP(i[0]), ARRP(i[1]));
@@ -249,16 +258,22 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
    {0}, {NULL}},                                                                                \
   {"segreduce_" #OP "_" #T, e_segreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0},            \
    {SEGRED_PARAM, NULL}},                                                                       \
+  HIST_ENTRY_ROWS(OP, T, CT)
+#define HIST_ENTRY_ROWS(OP, T, CT)                                                              \
   {"hist_" #OP "_" #T, e_hist_##OP##_##T, "[]" #T, 1, 3, {"i64", "[]i32", "[]" #T}, {0},        \
    {HIST_PARAM, NULL}},                                                                         \
   {"rbi_" #OP "_" #T, e_rbi_##OP##_##T, "[]" #T, 1, 3, {"[]" #T, "[]i32", "[]" #T}, {1, 0, 0},  \
    {HIST_PARAM, NULL}},
 #define SEGOP_ENTRY_ROWS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(SEGOP_ENTRY_ROWS, T, CT)
 #define SEGOP_BITOP_ROWS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(SEGOP_ENTRY_ROWS, T, CT)
+#define HIST_ONLY_INT_ROWS(T, CT) \
+  FUTHARK_FOR_EACH_OP(HIST_ENTRY_ROWS, T, CT) FUTHARK_FOR_EACH_BITOP(HIST_ENTRY_ROWS, T, CT)
 
 static const struct entry entries[] = {
     FUTHARK_FOR_EACH_NUM_TYPE(SEGOP_ENTRY_ROWS_FOR_TYPE)
     FUTHARK_FOR_EACH_INT_TYPE(SEGOP_BITOP_ROWS_FOR_TYPE)
+    FUTHARK_FOR_EACH_HIST_ONLY_INT_TYPE(HIST_ONLY_INT_ROWS)
+    FUTHARK_FOR_EACH_OP(HIST_ENTRY_ROWS, f16, uint16_t)
     {"bmm_f32", e_bmm_f32, "[][][]f32", 1, 2, {"[][][]f32", "[][][]f32"}, {0}, {NULL}},
     {"bmm_f16", e_bmm_f16, "[][][]f32", 1, 2, {"[][][]f16", "[][][]f16"}, {0}, {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {NULL}},

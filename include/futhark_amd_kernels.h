@@ -42,6 +42,12 @@ typedef enum {
   FA_U64 = 5,
   FA_F16 = 6,  /* IEEE binary16 bits in a uint16_t (docs/c-api.rst:229-233) */
   FA_BF16 = 7, /* bfloat16 bits in a uint16_t: f32 = bits << 16 */
+  /* 8- and 16-bit integers: element types of fa_seghist only (the types
+   * rts/c/atomics8.h and atomics16.h exist for). */
+  FA_I8 = 8,
+  FA_U8 = 9,
+  FA_I16 = 10,
+  FA_U16 = 11,
   FA_DTYPE_COUNT
 } fa_dtype;
 
@@ -123,6 +129,13 @@ int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op,
  * ignored (SegHist.hs:450-458,750-755).  dest is updated in place.
  * Replaces: seghist_local / seghist_global and the SegRed over sub-histograms
  * (SegHist.hs:377-467,576-828,1137-1186).  `is` is i32 (is64 == 0) or i64.
+ * Element types: every integer type of 8 to 64 bits with add, max, min, and,
+ * or, xor; f16, f32, f64 with add, max, min (the table of
+ * src/Futhark/CodeGen/ImpGen/GPU.hs:43-90).  Cells narrower than 32 bits are
+ * updated by compare-and-swap on the aligned 32-bit word that contains them
+ * (rts/c/atomics8.h, atomics16.h), so dest must lie in an allocation that
+ * covers whole words.  f16 sums are accumulated in f32 per block and rounded
+ * when a block combines its bins into dest.
  * scratch: fa_seghist_scratch_bytes() for the same t, is64, n and H; contents
  * need no initialisation (large H partitions the input into it). */
 size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int64_t H);

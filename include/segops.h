@@ -38,6 +38,10 @@
  * OP in {add, max, min}; NE = 0, T.lowest, T.highest; T in {i32, i64, f32, f64};
  * for T in {i32, i64} also OP in {and, or, xor} with NE = -1, 0, 0
  * (tests/hist/{and,or,xor}.fut).
+ * hist_OP_T and rbi_OP_T exist in addition for T in {i8, u8, i16, u16, u32,
+ * u64} with all six operators and for f16 with add, max, min: the element types
+ * whose updates the reference emulates with compare-and-swap, and the unsigned
+ * comparisons (tests/hist/{i8,i16,and8,and16,max8,max16,max,f16}.fut ...).
  */
 #ifndef SEGOPS_H
 #define SEGOPS_H
@@ -159,7 +163,11 @@ void futhark_context_free(struct futhark_context *ctx);
 
 FUTHARK_DECLARE_ARRAY_1D(i32, int32_t)
 FUTHARK_DECLARE_ARRAY_1D(i64, int64_t)
+FUTHARK_DECLARE_ARRAY_1D(i8, int8_t)
+FUTHARK_DECLARE_ARRAY_1D(i16, int16_t)
 FUTHARK_DECLARE_ARRAY_1D(u8, uint8_t)
+FUTHARK_DECLARE_ARRAY_1D(u16, uint16_t)
+FUTHARK_DECLARE_ARRAY_1D(f16, uint16_t) /* f16 crosses the API as its bits */
 FUTHARK_DECLARE_ARRAY_1D(u32, uint32_t)
 FUTHARK_DECLARE_ARRAY_1D(u64, uint64_t)
 FUTHARK_DECLARE_ARRAY_1D(f32, float)
@@ -200,6 +208,9 @@ FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
   int futhark_entry_segreduce_##OP##_##T(struct futhark_context *ctx,                         \
                                          struct futhark_##T##_1d **out0,                      \
                                          const struct futhark_##T##_2d *in0);                 \
+  FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)
+
+#define FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)                                               \
   int futhark_entry_hist_##OP##_##T(struct futhark_context *ctx,                              \
                                     struct futhark_##T##_1d **out0, const int64_t in0,        \
                                     const struct futhark_i32_1d *in1,                         \
@@ -219,6 +230,15 @@ FUTHARK_FOR_EACH_NUM_TYPE(FUTHARK_DECLARE_FOR_TYPE)
 #define FUTHARK_DECLARE_BITOPS_FOR_TYPE(T, CT) \
   FUTHARK_FOR_EACH_BITOP(FUTHARK_DECLARE_SEGOP_ENTRIES, T, CT)
 FUTHARK_FOR_EACH_INT_TYPE(FUTHARK_DECLARE_BITOPS_FOR_TYPE)
+
+/* hist_OP_T and rbi_OP_T alone for the remaining integer types and f16. */
+#define FUTHARK_FOR_EACH_HIST_ONLY_INT_TYPE(X) \
+  X(i8, int8_t) X(u8, uint8_t) X(i16, int16_t) X(u16, uint16_t) X(u32, uint32_t) X(u64, uint64_t)
+#define FUTHARK_DECLARE_HIST_ONLY_INT(T, CT)                  \
+  FUTHARK_FOR_EACH_OP(FUTHARK_DECLARE_HIST_ENTRIES, T, CT)    \
+  FUTHARK_FOR_EACH_BITOP(FUTHARK_DECLARE_HIST_ENTRIES, T, CT)
+FUTHARK_FOR_EACH_HIST_ONLY_INT_TYPE(FUTHARK_DECLARE_HIST_ONLY_INT)
+FUTHARK_FOR_EACH_OP(FUTHARK_DECLARE_HIST_ENTRIES, f16, uint16_t)
 
 int futhark_entry_bmm_f32(struct futhark_context *ctx, struct futhark_f32_3d **out0,
                           const struct futhark_f32_3d *in0, const struct futhark_f32_3d *in1);

@@ -15,7 +15,12 @@ _DIR = Path(__file__).resolve().parent
 _LIB = None
 
 _CT = {"i32": (C.c_int32, np.int32), "i64": (C.c_int64, np.int64),
-       "f32": (C.c_float, np.float32), "f64": (C.c_double, np.float64)}
+       "f32": (C.c_float, np.float32), "f64": (C.c_double, np.float64),
+       # element types of histograms only
+       "i8": (C.c_int8, np.int8), "u8": (C.c_uint8, np.uint8),
+       "i16": (C.c_int16, np.int16), "u16": (C.c_uint16, np.uint16),
+       "u32": (C.c_uint32, np.uint32), "u64": (C.c_uint64, np.uint64),
+       "f16": (C.c_uint16, np.float16)}
 
 
 def lib() -> C.CDLL:
@@ -110,7 +115,12 @@ NEUTRAL = {
     ("add", "f64"): 0.0, ("max", "f64"): -np.inf, ("min", "f64"): np.inf,
     ("and", "i32"): -1, ("or", "i32"): 0, ("xor", "i32"): 0,
     ("and", "i64"): -1, ("or", "i64"): 0, ("xor", "i64"): 0,
+    ("add", "f16"): 0.0, ("max", "f16"): -np.inf, ("min", "f16"): np.inf,
 }
+for _t in ("i8", "u8", "i16", "u16", "u32", "u64"):
+    _ii = np.iinfo(_CT[_t][1])
+    NEUTRAL.update({("add", _t): 0, ("max", _t): _ii.min, ("min", _t): _ii.max,
+                    ("and", _t): _ii.max if _ii.min == 0 else -1, ("or", _t): 0, ("xor", _t): 0})
 
 
 def hist(op: str, t: str, k: int, is_, vs, variant: str = "lit"):
@@ -143,6 +153,17 @@ def widen(bits, kind: str):
     fn.restype = None
     fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
     fn(_p(bits), _p(out), bits.size)
+    return out
+
+
+def narrow_f16(xs):
+    """f32 -> f16, round to nearest even."""
+    xs = _arr(xs, np.float32)
+    out = np.empty(xs.shape, dtype=np.float16)
+    fn = lib().orc_narrow_f16
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+    fn(_p(xs), _p(out), xs.size)
     return out
 
 

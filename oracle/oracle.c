@@ -39,6 +39,14 @@
   static inline T xor_##S(T a, T b) { return a ^ b; }
 OPS_INT(int32_t, uint32_t, i32)
 OPS_INT(int64_t, uint64_t, i64)
+/* the remaining integer types: element types of histograms only
+ * (tests/hist/{i8,i16,and8,and16,max8,max16,min8,min16,or8,or16,xor8,xor16}.fut) */
+OPS_INT(int8_t, uint8_t, i8)
+OPS_INT(uint8_t, uint8_t, u8)
+OPS_INT(int16_t, uint16_t, i16)
+OPS_INT(uint16_t, uint16_t, u16)
+OPS_INT(uint32_t, uint32_t, u32)
+OPS_INT(uint64_t, uint64_t, u64)
 static inline float add_f32(float a, float b) { return a + b; }
 static inline float max_f32(float a, float b) { return fmaxf(a, b); }
 static inline float min_f32(float a, float b) { return fminf(a, b); }
@@ -144,6 +152,25 @@ DEFINE_LIT_BITOPS(i64, int64_t)
 DEFINE_LIT_ALL_OPS(f32, float)
 DEFINE_LIT_ALL_OPS(f64, double)
 
+/* hist / reduce_by_index alone for the other integer types */
+#define DEFINE_RBI(OP, S, T)                                                                   \
+  void orc_rbi_##OP##_##S##_lit(T *dest, int64_t H, const int32_t *is, const T *vs,            \
+                                int64_t n) {                                                   \
+    for (int64_t i = 0; i < n; i++) {                                                          \
+      const int64_t b = (int64_t)is[i];                                                        \
+      if (b >= 0 && b < H) dest[b] = OP##_##S(dest[b], vs[i]);                                 \
+    }                                                                                          \
+  }
+#define DEFINE_RBI_ALL_OPS(S, T)                                                   \
+  DEFINE_RBI(add, S, T) DEFINE_RBI(max, S, T) DEFINE_RBI(min, S, T) DEFINE_RBI(and, S, T) \
+  DEFINE_RBI(or, S, T) DEFINE_RBI(xor, S, T)
+DEFINE_RBI_ALL_OPS(i8, int8_t)
+DEFINE_RBI_ALL_OPS(u8, uint8_t)
+DEFINE_RBI_ALL_OPS(i16, int16_t)
+DEFINE_RBI_ALL_OPS(u16, uint16_t)
+DEFINE_RBI_ALL_OPS(u32, uint32_t)
+DEFINE_RBI_ALL_OPS(u64, uint64_t)
+
 /* ------------------------------- f32 sums accumulated in double (yardstick) */
 float orc_reduce_add_f32_f64acc(const float *xs, int64_t n) {
   double acc = 0.0;
@@ -244,6 +271,61 @@ float orc_f16_to_f32(uint16_t h) {
   memcpy(&f, &bits, 4);
   return f;
 }
+/* f32 -> f16, round to nearest even: what the `half` type of the GPU backends
+ * does on conversion (rts/c/scalar_f16.h:11-60 computes f16 operators in float
+ * and converts back; the table-driven float2halfbits of rts/c/half.h:220-228,
+ * used where there is no native half type, truncates instead). */
+uint16_t orc_f32_to_f16(float f) {
+  uint32_t x;
+  memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7fffffffu;
+  if (x > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((x >> 13) & 0x3ffu)); /* NaN */
+  if (x >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u); /* 65520 and above, inf: to inf */
+  if (x < 0x33000001u) return (uint16_t)sign; /* <= 2^-25: to zero (the tie goes to even) */
+  if (x < 0x38800000u) {                      /* below 2^-14: subnormal result, units of 2^-24 */
+    const int shift = 126 - (int)(x >> 23);   /* 14 .. 24 */
+    const uint32_t man = (x & 0x7fffffu) | 0x800000u;
+    uint32_t r = man >> shift;
+    const uint32_t rem = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (r & 1u))) r++;
+    return (uint16_t)(sign | r);
+  }
+  uint32_t r = (((x >> 23) - 112u) << 10) | ((x >> 13) & 0x3ffu);
+  const uint32_t rem = x & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (r & 1u))) r++; /* a carry runs into the exponent */
+  return (uint16_t)(sign | r);
+}
+void orc_narrow_f16(const float *in, uint16_t *out, int64_t n) {
+  for (int64_t i = 0; i < n; i++) out[i] = orc_f32_to_f16(in[i]);
+}
+/* f16 histograms: operator in float on the widened operands, result stored as
+ * f16 after every update (`lit`); sums accumulated in double and rounded once
+ * per bin (`f64acc`). */
+#define DEFINE_RBI_F16(OP)                                                                  \
+  void orc_rbi_##OP##_f16_lit(uint16_t *dest, int64_t H, const int32_t *is,                 \
+                              const uint16_t *vs, int64_t n) {                              \
+    for (int64_t i = 0; i < n; i++) {                                                       \
+      const int64_t b = (int64_t)is[i];                                                     \
+      if (b >= 0 && b < H)                                                                  \
+        dest[b] = orc_f32_to_f16(OP##_f32(orc_f16_to_f32(dest[b]), orc_f16_to_f32(vs[i]))); \
+    }                                                                                       \
+  }
+DEFINE_RBI_F16(add)
+DEFINE_RBI_F16(max)
+DEFINE_RBI_F16(min)
+void orc_rbi_add_f16_f64acc(uint16_t *dest, int64_t H, const int32_t *is, const uint16_t *vs,
+                            int64_t n) {
+  double *acc = (double *)malloc(sizeof(double) * (size_t)(H > 0 ? H : 1));
+  for (int64_t b = 0; b < H; b++) acc[b] = (double)orc_f16_to_f32(dest[b]);
+  for (int64_t i = 0; i < n; i++) {
+    const int64_t b = (int64_t)is[i];
+    if (b >= 0 && b < H) acc[b] += (double)orc_f16_to_f32(vs[i]);
+  }
+  for (int64_t b = 0; b < H; b++) dest[b] = orc_f32_to_f16((float)acc[b]);
+  free(acc);
+}
+
 float orc_bf16_to_f32(uint16_t h) {
   const uint32_t bits = (uint32_t)h << 16;
   float f;

@@ -64,6 +64,92 @@ def test_hist_bitwise_operators(goldens):
             assert out.tolist() == c["out"], (name, c)
 
 
+NARROW = {"i8": np.int8, "u8": np.uint8, "i16": np.int16, "u16": np.uint16,
+          "u32": np.uint32, "u64": np.uint64}
+
+
+def test_hist_small_integer_types_goldens(goldens):
+    # tests/hist/{i8,i16,and8,and16,or8,or16,xor8,xor16,max8,max16,min8,min16}.fut and the
+    # unsigned results of max.fut / min.fut
+    for bits in (8, 16):
+        t, u = f"i{bits}", f"u{bits}"
+        for c in goldens[f"hist_add_{t}"]["cases"]:
+            assert oracle.rbi("add", t, c["dest"], c["is"], c["vs"]).tolist() == c["out"]
+        for op in ("and", "or", "xor"):
+            for c in goldens[f"hist_{op}{bits}"]["cases"]:
+                assert oracle.hist(op, t, c["n"], c["is"], c["vs"]).tolist() == c["out"], (op, bits, c)
+        for op in ("max", "min"):
+            for c in goldens[f"hist_{op}{bits}"]["cases"]:
+                vs = np.array(c["vs"], NARROW[t])
+                zeros = np.zeros(c["n"], NARROW[t])
+                assert oracle.rbi(op, t, zeros, c["is"], vs).tolist() == c["out"]
+                got = oracle.rbi(op, u, zeros.view(NARROW[u]), c["is"], vs.view(NARROW[u]))
+                assert got.view(NARROW[t]).tolist() == c["out_unsigned"], (op, bits, c)
+    for op in ("max", "min"):
+        for c in goldens[f"hist_{op}_u32"]["cases"]:
+            vs = np.array(c["vs"], np.int32).view(np.uint32)
+            got = oracle.rbi(op, "u32", np.zeros(c["n"], np.uint32), c["is"], vs)
+            assert got.view(np.int32).tolist() == c["out"]
+
+
+def test_hist_small_integer_types_against_numpy():
+    rng = np.random.default_rng(21)
+    ufuncs = {"add": np.add, "max": np.maximum, "min": np.minimum, "and": np.bitwise_and,
+              "or": np.bitwise_or, "xor": np.bitwise_xor}
+    for t, dt in NARROW.items():
+        ii = np.iinfo(dt)
+        vs = rng.integers(ii.min, ii.max, 5000, dtype=dt, endpoint=True)
+        is_ = rng.integers(-3, 40, 5000).astype(np.int32)
+        ok = (is_ >= 0) & (is_ < 37)
+        for op, uf in ufuncs.items():
+            dest = rng.integers(ii.min, ii.max, 37, dtype=dt, endpoint=True)
+            want = dest.copy()
+            uf.at(want, is_[ok], vs[ok])  # wraps in the element type
+            assert np.array_equal(oracle.rbi(op, t, dest, is_, vs), want), (t, op)
+            ne = oracle.hist(op, t, 3, np.zeros(0, np.int32), np.zeros(0, dt))
+            assert np.all(uf(ne, vs[:3]) == vs[:3]), (t, op)  # the neutral element is neutral
+
+
+def test_f16_rounding_and_histograms(goldens):
+    # f32 -> f16 is round-to-nearest-even: numpy's conversion is the check
+    rng = np.random.default_rng(3)
+    f = np.concatenate([
+        rng.integers(0, 2**32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32),
+        (rng.standard_normal(200000) * 10 ** rng.uniform(-9, 6, 200000)).astype(np.float32),
+        np.array([65504, 65519.99, 65520, 2**-24, 2**-25, 2**-25 * 1.0001, 2**-14, 0.0, -0.0,
+                  np.inf, -np.inf], np.float32)])
+    with np.errstate(all="ignore"):
+        want = f.astype(np.float16)
+    got = oracle.narrow_f16(f)
+    keep = ~np.isnan(f)
+    assert np.array_equal(got.view(np.uint16)[keep], want.view(np.uint16)[keep])
+    assert np.all(np.isnan(got[~keep]))
+    halves = np.arange(65536, dtype=np.uint16).view(np.float16)
+    back = oracle.narrow_f16(oracle.widen(halves.view(np.uint16), "f16"))
+    assert np.array_equal(back.view(np.uint16)[~np.isnan(halves)], halves.view(np.uint16)[~np.isnan(halves)])
+    # tests/hist/f16.fut and f64.fut
+    for c in goldens["hist_f16"]["cases"]:
+        for variant in ("lit", "f64acc"):
+            out = oracle.rbi("add", "f16", _f(c["dest"]).astype(np.float16), c["is"],
+                             _f(c["vs"]).astype(np.float16), variant)
+            np.testing.assert_allclose(out.astype(np.float32), _f(c["out"]), rtol=2e-3, equal_nan=True)
+    for c in goldens["hist_f64"]["cases"]:
+        out = oracle.rbi("add", "f64", _f(c["dest"]).astype(np.float64), c["is"], _f(c["vs"]).astype(np.float64))
+        np.testing.assert_allclose(out, _f(c["out"]).astype(np.float64), rtol=1e-6, equal_nan=True)
+    # small integers: every partial sum is an f16 value, so all three agree exactly
+    vs = rng.integers(0, 4, 3000).astype(np.float16)
+    is_ = rng.integers(-2, 9, 3000).astype(np.int32)
+    want = np.zeros(8, np.float64)
+    ok = (is_ >= 0) & (is_ < 8)
+    np.add.at(want, is_[ok], vs[ok].astype(np.float64))
+    for variant in ("lit", "f64acc"):
+        assert np.array_equal(oracle.hist("add", "f16", 8, is_, vs, variant).astype(np.float64), want)
+    # max / min ignore NaN operands like fmaxf / fminf
+    vs = np.array([1.5, np.nan, -2, 7, np.nan], np.float16)
+    assert oracle.hist("max", "f16", 2, [0, 0, 0, 1, 1], vs).tolist() == [1.5, 7.0]
+    assert oracle.hist("min", "f16", 2, [0, 0, 0, 1, 1], vs).tolist() == [-2.0, 7.0]
+
+
 def test_bitwise_reductions_and_scans_match_numpy():
     rng = np.random.default_rng(9)
     for t, dt in (("i32", np.int32), ("i64", np.int64)):
