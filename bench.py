@@ -124,8 +124,7 @@ def make_workload(name: str, ctx):
             vv = ctx.new("i32_1d", np.arange(n, dtype=np.int32))
 
             def step():
-                a, b = ctx.call("radix_sort_pairs_u64_i32", ["u64_1d", "i32_1d"], k, vv)
-                a.free(); b.free()
+                ctx.call("radix_sort_pairs_u64_i32", ["tup2_arr1d_u64_arr1d_i32"], k, vv).free()
             w.update(bytes=8 * 32 * n, keep=[k, vv])
         w.update(step=step, kernel="radix_sort", dtype=kt, bound="hbm",
                  describe=f"stable LSD radix sort, 8-bit digits, 2^{sz[2:]} {kt}")

@@ -123,6 +123,8 @@ def build_all() -> None:
     build_host()
     build_server()
     build_oracle()
+    from . import manifest  # include/segops.json, as `futhark hip --library` writes prog.json
+    manifest.write()
 
 
 if __name__ == "__main__":

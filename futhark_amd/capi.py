@@ -27,6 +27,9 @@ ARRAY_TYPES = {
     "i8_1d": (np.int8, 1), "i16_1d": (np.int16, 1), "u16_1d": (np.uint16, 1),
     "f16_1d": (np.uint16, 1),  # f16 crosses the API as its bits
 }
+# opaque tuple types: name -> element types of the two component arrays
+OPAQUE_PAIRS = {"tup2_arr1d_u32_arr1d_i32": ("u32", "i32"),
+                "tup2_arr1d_u64_arr1d_i32": ("u64", "i32")}
 OPS = ("add", "max", "min")
 BITOPS = ("and", "or", "xor")  # integer types only
 
@@ -120,8 +123,16 @@ class Segops:
             getattr(L, f"futhark_entry_{e}").argtypes = [vp, pp, vp, vp]
         L.futhark_entry_radix_sort_u32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u64.argtypes = [vp, pp, vp]
-        L.futhark_entry_radix_sort_pairs_u32_i32.argtypes = [vp, pp, pp, vp, vp]
-        L.futhark_entry_radix_sort_pairs_u64_i32.argtypes = [vp, pp, pp, vp, vp]
+        for name, (k, v) in OPAQUE_PAIRS.items():
+            getattr(L, f"futhark_entry_radix_sort_pairs_{k}_{v}").argtypes = [vp, pp, vp, vp]
+            getattr(L, f"futhark_free_opaque_{name}").argtypes = [vp, vp]
+            getattr(L, f"futhark_store_opaque_{name}").argtypes = [vp, vp, pp, C.POINTER(C.c_size_t)]
+            rs = getattr(L, f"futhark_restore_opaque_{name}")
+            rs.restype = vp
+            rs.argtypes = [vp, vp]
+            getattr(L, f"futhark_new_opaque_{name}").argtypes = [vp, pp, vp, vp]
+            for f in (0, 1):
+                getattr(L, f"futhark_project_opaque_{name}_{f}").argtypes = [vp, pp, vp]
         L.futhark_entry_transpose_f32.argtypes = [vp, pp, vp]
         L.futhark_entry_iota_i64.argtypes = [vp, pp, i64]
         L.futhark_entry_replicate_i32.argtypes = [vp, pp, i64, C.c_int32]
@@ -174,6 +185,40 @@ class Array:
     def free(self) -> None:
         if self.ptr and self.ctx.ptr:
             getattr(self.ctx.L, f"futhark_free_{self.kind}")(self.ctx.ptr, self.ptr)
+        self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Opaque:
+    """A futhark_opaque_NAME tuple of two arrays."""
+
+    def __init__(self, ctx: "Context", name: str, ptr: int):
+        self.ctx, self.name, self.ptr = ctx, name, ptr
+
+    def project(self, field: int) -> Array:
+        slot = C.c_void_p()
+        fn = getattr(self.ctx.L, f"futhark_project_opaque_{self.name}_{field}")
+        self.ctx.check(fn(self.ctx.ptr, C.byref(slot), self.ptr))
+        return Array(self.ctx, f"{OPAQUE_PAIRS[self.name][field]}_1d", slot.value)
+
+    def store(self) -> bytes:
+        n = C.c_size_t(0)
+        fn = getattr(self.ctx.L, f"futhark_store_opaque_{self.name}")
+        self.ctx.check(fn(self.ctx.ptr, self.ptr, None, C.byref(n)))
+        buf = (C.c_ubyte * n.value)()
+        p = C.c_void_p(C.addressof(buf))
+        self.ctx.check(fn(self.ctx.ptr, self.ptr, C.byref(p), C.byref(n)))
+        self.ctx.sync()
+        return bytes(buf)
+
+    def free(self) -> None:
+        if self.ptr and self.ctx.ptr:
+            getattr(self.ctx.L, f"futhark_free_opaque_{self.name}")(self.ctx.ptr, self.ptr)
         self.ptr = None
 
     def __del__(self):
@@ -242,6 +287,18 @@ class Context:
         self.sync()  # the copy is asynchronous; `a` may die after we return
         return Array(self, kind, p)
 
+    def new_opaque(self, name: str, f0: Array, f1: Array) -> Opaque:
+        slot = C.c_void_p()
+        self.check(getattr(self.L, f"futhark_new_opaque_{name}")(self.ptr, C.byref(slot), f0.ptr, f1.ptr))
+        return Opaque(self, name, slot.value)
+
+    def restore_opaque(self, name: str, data: bytes) -> Opaque:
+        p = getattr(self.L, f"futhark_restore_opaque_{name}")(self.ptr, data)
+        if not p:
+            raise FutharkError(1, self.get_error() or "futhark_restore_opaque failed")
+        self.sync()
+        return Opaque(self, name, p)
+
     def new_raw(self, kind: str, device_ptr: int, *dims: int) -> Array:
         p = getattr(self.L, f"futhark_new_raw_{kind}")(self.ptr, device_ptr, *dims)
         return Array(self, kind, p)
@@ -250,7 +307,7 @@ class Context:
     def call(self, entry: str, out_kinds, *args):
         """futhark_entry_<entry>(ctx, &out..., in...).
 
-        out_kinds: list of array kinds ("f32_1d") or scalar numpy dtypes.
+        out_kinds: list of array kinds ("f32_1d"), opaque type names or scalar numpy dtypes.
         Array inputs are passed as Array, scalars as Python numbers.
         Returns one value or a tuple; scalar results are read after a sync.
         """
@@ -274,6 +331,8 @@ class Context:
             if k is None:
                 need_sync = True
                 res.append(slot)
+            elif k in OPAQUE_PAIRS:
+                res.append(Opaque(self, k, slot.value))
             else:
                 res.append(Array(self, k, slot.value))
         if need_sync:

@@ -602,30 +602,153 @@ int futhark_entry_radix_sort_u64(struct futhark_context *ctx, struct futhark_u64
   LEAVE(ctx);
   return ret;
 }
-int futhark_entry_radix_sort_pairs_u32_i32(struct futhark_context *ctx,
-                                           struct futhark_u32_1d **out0,
-                                           struct futhark_i32_1d **out1,
-                                           const struct futhark_u32_1d *in0,
-                                           const struct futhark_i32_1d *in1) {
-  ENTER(ctx);
-  int ret = do_sort(ctx, 4, 4, (struct fut_array **)out0, (struct fut_array **)out1, &in0->a,
-                    &in1->a, "radix_sort_pairs_u32_i32");
-  LEAVE(ctx);
-  return ret;
-}
-int futhark_entry_radix_sort_pairs_u64_i32(struct futhark_context *ctx,
-                                           struct futhark_u64_1d **out0,
-                                           struct futhark_i32_1d **out1,
-                                           const struct futhark_u64_1d *in0,
-                                           const struct futhark_i32_1d *in1) {
-  ENTER(ctx);
-  int ret = do_sort(ctx, 8, 4, (struct fut_array **)out0, (struct fut_array **)out1, &in0->a,
-                    &in1->a, "radix_sort_pairs_u64_i32");
-  LEAVE(ctx);
-  return ret;
+/* ------------------------------------------------- tuples of two arrays
+ * An entry point has one result; a tuple result is an opaque record
+ * (docs/c-api.rst:318-432) named after its type by
+ * src/Futhark/CodeGen/Backends/SimpleRep.hs:144-186: ([]u32, []i32) is
+ * futhark_opaque_tup2_arr1d_u32_arr1d_i32.  Components are held as array
+ * values of their own (fields v0, v1); new and project hand out aliases with
+ * their own lifetime (GenericC/Types.hs:280-446); store writes the components
+ * one after the other in the binary data format and restore reads them back
+ * (GenericC/Types.hs:1063-1135). */
+static struct fut_array *array_alias(struct futhark_context *ctx, const struct fut_array *src) {
+  struct fut_array *a = (struct fut_array *)malloc(sizeof(struct fut_array));
+  if (a == NULL) return NULL;
+  memcpy(a, src, sizeof(*a));
+  pthread_mutex_lock(&ctx->lock);
+  if (a->mem.references != NULL) (*a->mem.references)++;
+  pthread_mutex_unlock(&ctx->lock);
+  return a;
 }
 
-/* ---------------------------------------------------------- data movement */
+#define VALUE_HEADER_BYTES 7 /* 'b', version, rank, four type characters */
+static unsigned char *put_header_1d(unsigned char *out, const char *tag, int64_t dim0) {
+  *out++ = 'b';
+  *out++ = 2;
+  *out++ = 1;
+  memcpy(out, tag, 4);
+  out += 4;
+  memcpy(out, &dim0, sizeof(int64_t));
+  return out + sizeof(int64_t);
+}
+static const unsigned char *get_header_1d(const unsigned char *src, const char *tag,
+                                          int64_t *dim0, int *err) {
+  *err |= (src[0] != 'b') | (src[1] != 2) | (src[2] != 1) | (memcmp(src + 3, tag, 4) != 0);
+  if (*err == 0) memcpy(dim0, src + VALUE_HEADER_BYTES, sizeof(int64_t));
+  return src + VALUE_HEADER_BYTES + sizeof(int64_t);
+}
+
+#define DEFINE_TUP2(NAME, T0, CT0, TAG0, T1, CT1, TAG1)                                         \
+  struct futhark_opaque_##NAME {                                                                \
+    struct futhark_##T0##_1d *v0;                                                               \
+    struct futhark_##T1##_1d *v1;                                                               \
+  };                                                                                            \
+  int futhark_free_opaque_##NAME(struct futhark_context *ctx,                                   \
+                                 struct futhark_opaque_##NAME *obj) {                           \
+    int ret = 0, tmp;                                                                           \
+    if (obj->v0 != NULL && (tmp = futhark_free_##T0##_1d(ctx, obj->v0)) != 0) ret = tmp;        \
+    if (obj->v1 != NULL && (tmp = futhark_free_##T1##_1d(ctx, obj->v1)) != 0) ret = tmp;        \
+    free(obj);                                                                                  \
+    return ret;                                                                                 \
+  }                                                                                             \
+  int futhark_store_opaque_##NAME(struct futhark_context *ctx,                                  \
+                                  const struct futhark_opaque_##NAME *obj, void **p,            \
+                                  size_t *n) {                                                  \
+    int ret = 0;                                                                                \
+    const int64_t n0 = obj->v0->a.shape[0], n1 = obj->v1->a.shape[0];                           \
+    const int64_t size_0 = VALUE_HEADER_BYTES + 8 + n0 * (int64_t)sizeof(CT0);                  \
+    const int64_t size_1 = VALUE_HEADER_BYTES + 8 + n1 * (int64_t)sizeof(CT1);                  \
+    *n = (size_t)(size_0 + size_1);                                                             \
+    if (p != NULL && *p == NULL) *p = malloc(*n);                                               \
+    if (p != NULL) {                                                                            \
+      unsigned char *out = (unsigned char *)*p;                                                 \
+      if (out == NULL) return FUTHARK_OUT_OF_MEMORY;                                            \
+      out = put_header_1d(out, TAG0, n0);                                                       \
+      ret |= futhark_values_##T0##_1d(ctx, obj->v0, (CT0 *)(void *)out);                        \
+      out += n0 * (int64_t)sizeof(CT0);                                                         \
+      out = put_header_1d(out, TAG1, n1);                                                       \
+      ret |= futhark_values_##T1##_1d(ctx, obj->v1, (CT1 *)(void *)out);                        \
+    }                                                                                           \
+    return ret;                                                                                 \
+  }                                                                                             \
+  struct futhark_opaque_##NAME *futhark_restore_opaque_##NAME(struct futhark_context *ctx,      \
+                                                              const void *p) {                  \
+    int err = 0;                                                                                \
+    const unsigned char *src = (const unsigned char *)p;                                        \
+    struct futhark_opaque_##NAME *obj = malloc(sizeof(*obj));                                   \
+    if (obj == NULL) return NULL;                                                               \
+    obj->v0 = NULL;                                                                             \
+    obj->v1 = NULL;                                                                             \
+    int64_t n0 = 0, n1 = 0;                                                                     \
+    const unsigned char *data_0 = get_header_1d(src, TAG0, &n0, &err);                          \
+    const unsigned char *data_1 = NULL;                                                         \
+    if (err == 0 && n0 < 0) err = 1;                                                            \
+    if (err == 0) data_1 = get_header_1d(data_0 + n0 * (int64_t)sizeof(CT0), TAG1, &n1, &err);  \
+    if (err == 0 && n1 < 0) err = 1;                                                            \
+    if (err == 0) {                                                                             \
+      /* the bytes need not be aligned for CT0 / CT1: the copy is byte-wise */                  \
+      obj->v0 = futhark_new_##T0##_1d(ctx, (const CT0 *)(const void *)data_0, n0);              \
+      if (obj->v0 == NULL) err = 1;                                                             \
+      obj->v1 = futhark_new_##T1##_1d(ctx, (const CT1 *)(const void *)data_1, n1);              \
+      if (obj->v1 == NULL) err = 1;                                                             \
+    }                                                                                           \
+    if (err != 0) {                                                                             \
+      futhark_free_opaque_##NAME(ctx, obj);                                                     \
+      obj = NULL;                                                                               \
+    }                                                                                           \
+    return obj;                                                                                 \
+  }                                                                                             \
+  int futhark_new_opaque_##NAME(struct futhark_context *ctx, struct futhark_opaque_##NAME **out, \
+                                const struct futhark_##T0##_1d *f_0,                            \
+                                const struct futhark_##T1##_1d *f_1) {                          \
+    struct futhark_opaque_##NAME *v = malloc(sizeof(*v));                                       \
+    if (v == NULL) return FUTHARK_OUT_OF_MEMORY;                                                \
+    v->v0 = (struct futhark_##T0##_1d *)array_alias(ctx, &f_0->a);                              \
+    v->v1 = (struct futhark_##T1##_1d *)array_alias(ctx, &f_1->a);                              \
+    if (v->v0 == NULL || v->v1 == NULL) {                                                       \
+      futhark_free_opaque_##NAME(ctx, v);                                                       \
+      return FUTHARK_OUT_OF_MEMORY;                                                             \
+    }                                                                                           \
+    *out = v;                                                                                   \
+    return FUTHARK_SUCCESS;                                                                     \
+  }                                                                                             \
+  int futhark_project_opaque_##NAME##_0(struct futhark_context *ctx,                            \
+                                        struct futhark_##T0##_1d **out,                         \
+                                        const struct futhark_opaque_##NAME *obj) {              \
+    struct fut_array *v = array_alias(ctx, &obj->v0->a);                                        \
+    if (v == NULL) return FUTHARK_OUT_OF_MEMORY;                                                \
+    *out = (struct futhark_##T0##_1d *)v;                                                       \
+    return 0;                                                                                   \
+  }                                                                                             \
+  int futhark_project_opaque_##NAME##_1(struct futhark_context *ctx,                            \
+                                        struct futhark_##T1##_1d **out,                         \
+                                        const struct futhark_opaque_##NAME *obj) {              \
+    struct fut_array *v = array_alias(ctx, &obj->v1->a);                                        \
+    if (v == NULL) return FUTHARK_OUT_OF_MEMORY;                                                \
+    *out = (struct futhark_##T1##_1d *)v;                                                       \
+    return 0;                                                                                   \
+  }                                                                                             \
+  int futhark_entry_radix_sort_pairs_##T0##_##T1(struct futhark_context *ctx,                   \
+                                                 struct futhark_opaque_##NAME **out0,           \
+                                                 const struct futhark_##T0##_1d *in0,           \
+                                                 const struct futhark_##T1##_1d *in1) {         \
+    struct futhark_opaque_##NAME *v = malloc(sizeof(*v));                                       \
+    if (v == NULL) return FUTHARK_OUT_OF_MEMORY;                                                \
+    ENTER(ctx);                                                                                 \
+    int ret = do_sort(ctx, (int)sizeof(CT0), (int)sizeof(CT1), (struct fut_array **)&v->v0,     \
+                      (struct fut_array **)&v->v1, &in0->a, &in1->a,                            \
+                      "radix_sort_pairs_" #T0 "_" #T1);                                         \
+    LEAVE(ctx);                                                                                 \
+    if (ret != 0) {                                                                             \
+      free(v); /* on error the out-parameter is not touched */                                  \
+      return ret;                                                                               \
+    }                                                                                           \
+    *out0 = v;                                                                                  \
+    return 0;                                                                                   \
+  }
+
+DEFINE_TUP2(tup2_arr1d_u32_arr1d_i32, u32, uint32_t, " u32", i32, int32_t, " i32")
+DEFINE_TUP2(tup2_arr1d_u64_arr1d_i32, u64, uint64_t, " u64", i32, int32_t, " i32")
 
 int futhark_entry_transpose_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
                                 const struct futhark_f32_2d *in0) {

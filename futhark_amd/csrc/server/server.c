@@ -224,18 +224,24 @@ static int e_radix_sort_u32(struct futhark_context *c, struct value *o, struct v
 static int e_radix_sort_u64(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_radix_sort_u64(c, (struct futhark_u64_1d **)&o->u.arr, ARRP(i[0]));
 }
-static int e_radix_sort_pairs_u32_i32(struct futhark_context *c, struct value *o,
-                                      struct value **i) {
-  return futhark_entry_radix_sort_pairs_u32_i32(
-      c, (struct futhark_u32_1d **)&o->u.fields[0]->value.u.arr,
-      (struct futhark_i32_1d **)&o->u.fields[1]->value.u.arr, ARRP(i[0]), ARRP(i[1]));
-}
-static int e_radix_sort_pairs_u64_i32(struct futhark_context *c, struct value *o,
-                                      struct value **i) {
-  return futhark_entry_radix_sort_pairs_u64_i32(
-      c, (struct futhark_u64_1d **)&o->u.fields[0]->value.u.arr,
-      (struct futhark_i32_1d **)&o->u.fields[1]->value.u.arr, ARRP(i[0]), ARRP(i[1]));
-}
+/* The tuple result arrives as one opaque value; the server keeps records as
+ * their fields, so it projects both and lets the tuple go. */
+#define SORT_PAIRS_ENTRY_FN(NAME, K, V)                                                         \
+  static int e_radix_sort_pairs_##K##_##V(struct futhark_context *c, struct value *o,           \
+                                          struct value **i) {                                   \
+    struct futhark_opaque_##NAME *t = NULL;                                                     \
+    int ret = futhark_entry_radix_sort_pairs_##K##_##V(c, &t, ARRP(i[0]), ARRP(i[1]));          \
+    if (ret != 0) return ret;                                                                   \
+    ret = futhark_project_opaque_##NAME##_0(                                                    \
+        c, (struct futhark_##K##_1d **)&o->u.fields[0]->value.u.arr, t);                        \
+    if (ret == 0)                                                                               \
+      ret = futhark_project_opaque_##NAME##_1(                                                  \
+          c, (struct futhark_##V##_1d **)&o->u.fields[1]->value.u.arr, t);                      \
+    int tmp = futhark_free_opaque_##NAME(c, t);                                                 \
+    return ret != 0 ? ret : tmp;                                                                \
+  }
+SORT_PAIRS_ENTRY_FN(tup2_arr1d_u32_arr1d_i32, u32, i32)
+SORT_PAIRS_ENTRY_FN(tup2_arr1d_u64_arr1d_i32, u64, i32)
 static int e_transpose_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_transpose_f32(c, (struct futhark_f32_2d **)&o->u.arr, ARRP(i[0]));
 }
@@ -250,7 +256,7 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
 #define HIST_PARAM "segops.hist_lds_bins_max"
 #define SEGRED_PARAM "segops.segred_small_threshold"
 #define SEGOP_ENTRY_ROWS(OP, T, CT)                                                             \
-  {"reduce_" #OP "_" #T, e_reduce_##OP##_##T, #T, 1, 1, {"[]" #T}, {0}, {NULL}},                \
+  {"reduce_" #OP "_" #T, e_reduce_##OP##_##T, #T, 0, 1, {"[]" #T}, {0}, {NULL}},                \
   {"scan_" #OP "_" #T, e_scan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {NULL}},               \
   {"exscan_" #OP "_" #T, e_exscan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {NULL}},           \
   {"segscan_" #OP "_" #T, e_segscan_##OP##_##T, "[]" #T, 1, 2, {"[]u8", "[]" #T}, {0}, {NULL}}, \

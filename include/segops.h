@@ -33,6 +33,7 @@
  *   entry bmm_bf16: [][][]u16 inputs, x -> f32.from_bits (u32.u16 x << 16)
  *   entry radix_sort_T (keys: []T) : []T       -- 8-bit LSD passes, stable
  *   entry radix_sort_pairs_K_V (keys: []K) (vals: []V) : ([]K, []V)
+ *                                  -- one opaque result, see "Opaque" below
  *   entry transpose_f32 (xss: [][]f32) : [][]f32 = transpose xss
  *
  * OP in {add, max, min}; NE = 0, T.lowest, T.highest; T in {i32, i64, f32, f64};
@@ -180,6 +181,40 @@ FUTHARK_DECLARE_ARRAY_3D(f32, float)
 FUTHARK_DECLARE_ARRAY_3D(f16, uint16_t) /* f16 crosses the API as its bits */
 FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
 
+/* ---------------------------------------------------------------- Opaque
+ * A tuple result is one opaque value (docs/c-api.rst:318-432); the type
+ * ([]K, []V) is named futhark_opaque_tup2_arr1d_K_arr1d_V
+ * (src/Futhark/CodeGen/Backends/SimpleRep.hs:144-186).
+ *   free     drops the value (its components have their own references)
+ *   store    serialises to *p (malloc'd if *p is NULL; p == NULL only sets *n);
+ *            the components follow each other in the binary data format
+ *   restore  the inverse; NULL on malformed input
+ *   new      a tuple aliasing the given arrays, with its own lifetime
+ *   project  component 0 / 1 as an array value the caller frees */
+#define FUTHARK_DECLARE_SORT_PAIRS(NAME, K, V)                                                 \
+  struct futhark_opaque_##NAME;                                                                \
+  int futhark_free_opaque_##NAME(struct futhark_context *ctx,                                  \
+                                 struct futhark_opaque_##NAME *obj);                           \
+  int futhark_store_opaque_##NAME(struct futhark_context *ctx,                                 \
+                                  const struct futhark_opaque_##NAME *obj, void **p,           \
+                                  size_t *n);                                                  \
+  struct futhark_opaque_##NAME *futhark_restore_opaque_##NAME(struct futhark_context *ctx,     \
+                                                              const void *p);                  \
+  int futhark_new_opaque_##NAME(struct futhark_context *ctx,                                   \
+                                struct futhark_opaque_##NAME **out,                            \
+                                const struct futhark_##K##_1d *f_0,                            \
+                                const struct futhark_##V##_1d *f_1);                           \
+  int futhark_project_opaque_##NAME##_0(struct futhark_context *ctx,                           \
+                                        struct futhark_##K##_1d **out,                         \
+                                        const struct futhark_opaque_##NAME *obj);              \
+  int futhark_project_opaque_##NAME##_1(struct futhark_context *ctx,                           \
+                                        struct futhark_##V##_1d **out,                         \
+                                        const struct futhark_opaque_##NAME *obj);              \
+  int futhark_entry_radix_sort_pairs_##K##_##V(struct futhark_context *ctx,                    \
+                                               struct futhark_opaque_##NAME **out0,            \
+                                               const struct futhark_##K##_1d *in0,             \
+                                               const struct futhark_##V##_1d *in1);
+
 /* ----------------------------------------------------------- Entry points
  * int futhark_entry_NAME(ctx, outputs..., inputs...): 0 on success; scalar
  * outputs are valid after futhark_context_sync; array outputs are new values
@@ -253,16 +288,8 @@ int futhark_entry_radix_sort_u32(struct futhark_context *ctx, struct futhark_u32
                                  const struct futhark_u32_1d *in0);
 int futhark_entry_radix_sort_u64(struct futhark_context *ctx, struct futhark_u64_1d **out0,
                                  const struct futhark_u64_1d *in0);
-int futhark_entry_radix_sort_pairs_u32_i32(struct futhark_context *ctx,
-                                           struct futhark_u32_1d **out0,
-                                           struct futhark_i32_1d **out1,
-                                           const struct futhark_u32_1d *in0,
-                                           const struct futhark_i32_1d *in1);
-int futhark_entry_radix_sort_pairs_u64_i32(struct futhark_context *ctx,
-                                           struct futhark_u64_1d **out0,
-                                           struct futhark_i32_1d **out1,
-                                           const struct futhark_u64_1d *in0,
-                                           const struct futhark_i32_1d *in1);
+FUTHARK_DECLARE_SORT_PAIRS(tup2_arr1d_u32_arr1d_i32, u32, i32)
+FUTHARK_DECLARE_SORT_PAIRS(tup2_arr1d_u64_arr1d_i32, u64, i32)
 
 int futhark_entry_transpose_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
                                 const struct futhark_f32_2d *in0);

@@ -162,8 +162,14 @@ static void section_two_results_and_report(struct futhark_context *ctx) {
   int32_t vals[6] = {0, 1, 2, 3, 4, 5};
   struct futhark_u32_1d *k = futhark_new_u32_1d(ctx, keys, 6), *ko;
   struct futhark_i32_1d *v = futhark_new_i32_1d(ctx, vals, 6), *vo;
+  struct futhark_opaque_tup2_arr1d_u32_arr1d_i32 *sorted;
   futhark_context_unpause_profiling(ctx);
-  CHECK(futhark_entry_radix_sort_pairs_u32_i32(ctx, &ko, &vo, k, v) == 0);
+  CHECK(futhark_entry_radix_sort_pairs_u32_i32(ctx, &sorted, k, v) == 0);
+  /* a tuple result is one opaque value; its fields are projected out
+   * (tests_lib/c/test_b.c) and outlive it */
+  CHECK(futhark_project_opaque_tup2_arr1d_u32_arr1d_i32_0(ctx, &ko, sorted) == 0);
+  CHECK(futhark_project_opaque_tup2_arr1d_u32_arr1d_i32_1(ctx, &vo, sorted) == 0);
+  CHECK(futhark_free_opaque_tup2_arr1d_u32_arr1d_i32(ctx, sorted) == 0);
   uint32_t kh[6];
   int32_t vh[6];
   CHECK(futhark_values_u32_1d(ctx, ko, kh) == 0 && futhark_values_i32_1d(ctx, vo, vh) == 0);

@@ -20,6 +20,48 @@ def test_keys_only(ctx, kt):
         assert np.array_equal(got, oracle.radix_sort(keys))
 
 
+def _sort_pairs(ctx, kt, keys, vals):
+    """The entry point returns one opaque tuple; its two components are projected out and the
+    tuple freed (the components live on)."""
+    k, v = ctx.new(f"{kt}_1d", keys), ctx.new("i32_1d", vals)
+    tup = ctx.call(f"radix_sort_pairs_{kt}_i32", [f"tup2_arr1d_{kt}_arr1d_i32"], k, v)
+    ko, vo = tup.project(0), tup.project(1)
+    for h in (tup, k, v):
+        h.free()
+    return ko, vo
+
+
+def test_opaque_tuple_new_project_store_restore(ctx):
+    """Call sequences of tests_lib/c/test_project.c (new, then project twice) and
+    test_restore.c (store with p == NULL for the size, then into a buffer, then restore)."""
+    keys = np.array([5, 1, 5, 0, 1, 9], np.uint32)
+    vals = np.arange(6, dtype=np.int32)
+    name = "tup2_arr1d_u32_arr1d_i32"
+    k, v = ctx.new("u32_1d", keys), ctx.new("i32_1d", vals)
+    tup = ctx.new_opaque(name, k, v)
+    k.free(); v.free()                          # the tuple holds its own references
+    for _ in range(2):
+        a = tup.project(0)
+        assert a.values().tolist() == keys.tolist()
+        a.free()
+    blob = tup.store()
+    # two values of the binary data format, one after the other
+    assert len(blob) == 2 * (7 + 8) + 6 * 4 + 6 * 4
+    assert blob[:7] == b"b\x02\x01 u32" and blob[15 + 24:15 + 24 + 7] == b"b\x02\x01 i32"
+    back = ctx.restore_opaque(name, blob)
+    assert back.project(0).values().tolist() == keys.tolist()
+    assert back.project(1).values().tolist() == vals.tolist()
+    out = ctx.call("radix_sort_pairs_u32_i32", [name], back.project(0), back.project(1))
+    assert out.project(0).values().tolist() == [0, 1, 1, 5, 5, 9]
+    assert out.project(1).values().tolist() == [3, 1, 4, 0, 2, 5]
+    with pytest.raises(Exception):
+        ctx.restore_opaque(name, b"b\x02\x01 i32" + blob[7:])   # wrong element type
+    with pytest.raises(Exception):
+        ctx.restore_opaque("tup2_arr1d_u64_arr1d_i32", blob)      # another tuple type
+    for h in (tup, back, out):
+        h.free()
+
+
 @pytest.mark.parametrize("kt", ["u32", "u64"])
 def test_pairs_are_stable(ctx, kt):
     for n in SIZES:
@@ -28,8 +70,7 @@ def test_pairs_are_stable(ctx, kt):
         keys = (raw % np.uint64(37)).astype(np.uint32 if kt == "u32" else np.uint64)
         keys = keys << (keys.dtype.type(13) if kt == "u32" else keys.dtype.type(45))
         vals = np.arange(n, dtype=np.int32)
-        ko, vo = ctx.call(f"radix_sort_pairs_{kt}_i32", [f"{kt}_1d", "i32_1d"],
-                          ctx.new(f"{kt}_1d", keys), ctx.new("i32_1d", vals))
+        ko, vo = _sort_pairs(ctx, kt, keys, vals)
         gk, gv = ko.values(), vo.values()
         perm = np.argsort(keys, kind="stable")
         assert np.array_equal(gk, keys[perm]) and np.array_equal(gv, vals[perm].astype(np.int32)), n
@@ -41,8 +82,7 @@ def test_reference_golden(ctx, goldens):
     c = goldens["radixsort"]["cases"][0]
     keys = np.array(c["keys"], np.float32).view(np.uint32)  # positive floats order as their bits
     vals = np.array(c["vals"], np.float32).view(np.int32)
-    ko, vo = ctx.call("radix_sort_pairs_u32_i32", ["u32_1d", "i32_1d"], ctx.new("u32_1d", keys),
-                      ctx.new("i32_1d", vals))
+    ko, vo = _sort_pairs(ctx, "u32", keys, vals)
     assert vo.values().view(np.float32).tolist() == np.array(c["out_vals"], np.float32).tolist()
 
 
@@ -59,8 +99,7 @@ def test_config5_full_size_pairs(ctx):
     n = 1 << 26
     keys = dg.uniform_u64(81, n)
     vals = np.arange(n, dtype=np.int32)
-    ko, vo = ctx.call("radix_sort_pairs_u64_i32", ["u64_1d", "i32_1d"], ctx.new("u64_1d", keys),
-                      ctx.new("i32_1d", vals))
+    ko, vo = _sort_pairs(ctx, "u64", keys, vals)
     gk, gv = ko.values(), vo.values()
     assert np.all(gk[1:] >= gk[:-1])
     assert np.array_equal(keys[gv], gk)                      # vo is the sorting permutation

@@ -45,7 +45,16 @@ def test_introspection(srv):
     types = srv.cmd("types")
     assert {"i32", "[]f32", "[][]f32", "[][][]f16", "([]u32, []i32)"} <= set(types)
     entries = srv.cmd("entry_points")
-    assert len(entries) == (4 * 3 + 2 * 3) * 8 + 11 and "segscan_add_f32" in entries
+    assert len(entries) == (4 * 3 + 2 * 3) * 8 + (6 * 6 + 3) * 2 + 11 and "segscan_add_f32" in entries
+    from futhark_amd import manifest
+    m = manifest.manifest()            # the server and the manifest describe the same API
+    assert set(entries) == set(m["entry_points"])
+    assert set(types) == set(m["types"]) | {"i32", "i64", "f32", "f64"}
+    for name in ("rbi_max_u16", "segred_add_f64", "reduce_min_i64", "radix_sort_pairs_u64_i32", "bmm_bf16"):
+        e = m["entry_points"][name]
+        assert srv.cmd("inputs", name) == [("*" if i["unique"] else "") + i["type"] for i in e["inputs"]]
+        assert srv.cmd("output", name) == [("*" if e["output"]["unique"] else "") + e["output"]["type"]]
+        assert [l.split()[0] for l in srv.cmd("tuning_params", name)] == e["tuning_params"]
     assert srv.cmd("inputs", "segscan_add_f32") == ["[]u8", "[]f32"]
     assert srv.cmd("output", "segscan_add_f32") == ["*[]f32"]
     assert srv.cmd("inputs", "rbi_add_i32") == ["*[]i32", "[]i32", "[]i32"]
