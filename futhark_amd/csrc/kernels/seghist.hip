@@ -233,10 +233,17 @@ template <class E> __device__ __forceinline__ void load_elems4(E (&dst)[4], cons
 // Grid layout: block b sits on XCD b % 8.  j = b / 8; range p = j % P;
 // chunk set s = (j / P) * 8 + b % 8 of S = gridDim.x / P sets.  The P blocks of
 // one chunk set read the same elements, each keeping the bins of its range.
-template <class T, class Op, class I>
+//
+// SEGMENTED: the input is [m][seg_len] and every row has its own H_seg bins
+// (`map (hist op ne H_seg) iss vss`, SegHist.hs:1057-1136 with segment
+// dimensions): element p belongs to row p / seg_len and its bin b, if inside
+// [0, H_seg), is bin row * H_seg + b of the m * H_seg = H bins of dest.  A
+// thread keeps (row, column) of its current vector and advances them by the
+// grid stride, so there is one division per thread, not per element.
+template <class T, class Op, class I, bool SEGMENTED>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
     const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t bin_base,
-    int64_t H, int range_bins, int P, int log2_copies) {
+    int64_t H, int range_bins, int P, int log2_copies, int64_t seg_len, int64_t H_seg) {
   using A = typename HistAcc<T>::A;
   using OpA = typename RebindOp<Op, A>::type;
   extern __shared__ __align__(16) unsigned char s_raw[];
@@ -266,18 +273,52 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
     if ((uint64_t)r < (uint64_t)nb)
       lds_update<A, OpA>(&sh[((int)r << log2_copies) + copy], (A)v);
   };
+  // Bin of dest for (position, raw bin): identity unless SEGMENTED.
+  auto seg_bin = [&](int64_t row, int64_t b) -> int64_t {
+    return (uint64_t)b < (uint64_t)H_seg ? row * H_seg + b : (int64_t)-1;
+  };
   if (nb > 0) {
-    for (int64_t i = s * HIST_BLOCK + threadIdx.x; i < nvec; i += stride) {
+    const int64_t i0 = s * HIST_BLOCK + threadIdx.x;
+    int64_t row = 0, col = 0, row_step = 0, col_step = 0;
+    if constexpr (SEGMENTED) {
+      row = (i0 * VEC) / seg_len;
+      col = (i0 * VEC) % seg_len;
+      row_step = (stride * VEC) / seg_len;
+      col_step = (stride * VEC) % seg_len;
+    }
+    for (int64_t i = i0; i < nvec; i += stride) {
       I bi[VEC];
       T bv[VEC];
       load_elems4(bi, is + i * VEC);
       load_elems4(bv, vs + i * VEC);
+      if constexpr (SEGMENTED) {
+        int64_t r = row, c = col;
 #pragma unroll
-      for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
+        for (int e = 0; e < VEC; e++) {
+          while (c >= seg_len) {  // at most once when seg_len >= VEC
+            c -= seg_len;
+            r++;
+          }
+          update(seg_bin(r, (int64_t)bi[e]), bv[e]);
+          c++;
+        }
+        row += row_step;
+        col += col_step;
+        if (col >= seg_len) {
+          col -= seg_len;
+          row++;
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
+      }
     }
     if (s == 0) {
       const int64_t t = nvec * VEC + threadIdx.x;
-      if (threadIdx.x < VEC && t < n) update((int64_t)is[t], vs[t]);
+      if (threadIdx.x < VEC && t < n) {
+        if constexpr (SEGMENTED) update(seg_bin(t / seg_len, (int64_t)is[t]), vs[t]);
+        else update((int64_t)is[t], vs[t]);
+      }
     }
   }
   __syncthreads();
@@ -380,9 +421,9 @@ static int hist_num_cus() {
 }
 
 // Launches the LDS kernel over bins [0,H) of `dest` (H <= max ranges * range size).
-template <class T, class Op, class I>
+template <class T, class Op, class I, bool SEGMENTED = false>
 static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
-                           int64_t H) {
+                           int64_t H, int64_t seg_len = 0, int64_t H_seg = 0) {
   using A = typename HistAcc<T>::A;
   const int max_range = HIST_LDS_BYTES / (int)sizeof(A);
   const int P = (int)ceil_div(H, max_range);
@@ -396,7 +437,7 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
   int grid = hist_num_cus() * per_cu;
   grid -= grid % (NUM_XCDS * P);
   if (grid < NUM_XCDS * P) grid = NUM_XCDS * P;
-  auto kernel = seghist_lds_kernel<T, Op, I>;
+  auto kernel = seghist_lds_kernel<T, Op, I, SEGMENTED>;
   static bool raised = false;
   if (!raised) {
     hipError_t e = hipFuncSetAttribute((const void *)kernel,
@@ -405,7 +446,7 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
     raised = true;
   }
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(HIST_BLOCK), lds, st, is, vs, n, dest, (int64_t)0,
-                     H, range_bins, P, log2_copies);
+                     H, range_bins, P, log2_copies, seg_len, H_seg);
   return launch_status();
 }
 
@@ -474,6 +515,53 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
   return launch_status();
 }
 
+// Row-major bins of a segmented histogram for the paths that take plain
+// indices: flat[p] = row(p) * H_seg + is[p], or -1 when is[p] is out of range.
+template <class I>
+__global__ __launch_bounds__(256) void seghist_flatten_kernel(const I *__restrict__ is, int64_t n,
+                                                              int64_t seg_len, int64_t H_seg,
+                                                              int64_t *__restrict__ flat) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t p = (int64_t)blockIdx.x * 256 + threadIdx.x; p < n; p += stride) {
+    const int64_t b = (int64_t)is[p];
+    flat[p] = (uint64_t)b < (uint64_t)H_seg ? (p / seg_len) * H_seg + b : (int64_t)-1;
+  }
+}
+
+template <class T, class Op>
+static int launch_hist_segmented(hipStream_t st, const void *is, int is64, const void *vs,
+                                 int64_t m, int64_t seg_len, void *dest, int64_t H_seg,
+                                 void *scratch, size_t scratch_bytes) {
+  const int64_t n = m * seg_len, H = m * H_seg;
+  if (H == 0 || n == 0) return 0;
+  if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
+  const int64_t lds_limit =
+      (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)sizeof(typename HistAcc<T>::A));
+  if (H <= lds_limit) {
+    if (is64)
+      return launch_lds_hist<T, Op, int64_t, true>(st, (const int64_t *)is, (const T *)vs, n,
+                                                   (T *)dest, H, seg_len, H_seg);
+    return launch_lds_hist<T, Op, int32_t, true>(st, (const int32_t *)is, (const T *)vs, n,
+                                                 (T *)dest, H, seg_len, H_seg);
+  }
+  // Too many bins for one launch of LDS ranges: flatten the indices, then the
+  // unsegmented paths.
+  const size_t flat_bytes = hist_align((size_t)n * sizeof(int64_t));
+  if (scratch_bytes < flat_bytes || !is_aligned(scratch, 256)) return FA_ESCRATCH;
+  int64_t *flat = (int64_t *)scratch;
+  const int grid = (int)std::min<int64_t>(ceil_div(n, (int64_t)256), (int64_t)hist_num_cus() * 16);
+  if (is64)
+    hipLaunchKernelGGL((seghist_flatten_kernel<int64_t>), dim3(grid), dim3(256), 0, st,
+                       (const int64_t *)is, n, seg_len, H_seg, flat);
+  else
+    hipLaunchKernelGGL((seghist_flatten_kernel<int32_t>), dim3(grid), dim3(256), 0, st,
+                       (const int32_t *)is, n, seg_len, H_seg, flat);
+  const int rc = launch_status();
+  if (rc != 0) return rc;
+  return launch_hist<T, Op>(st, flat, 1, vs, n, dest, H, (char *)scratch + flat_bytes,
+                            scratch_bytes - flat_bytes);
+}
+
 }  // namespace fa
 
 extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int64_t H) {
@@ -523,4 +611,31 @@ extern "C" int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op, const void *
   }
 #undef FA_HIST_NARROW_INT
   FA_DISPATCH_TYPE_OP(launch_hist, t, op, s, is, is64, vs, n, dest, H, scratch, scratch_bytes);
+}
+
+extern "C" size_t fa_seghist_segmented_scratch_bytes(fa_dtype t, int64_t m, int64_t seg_len,
+                                                     int64_t H_seg) {
+  if (m < 0 || seg_len < 0 || H_seg < 0) return 0;
+  const int64_t n = m * seg_len;
+  return hist_align((size_t)n * sizeof(int64_t)) + fa_seghist_scratch_bytes(t, 1, n, m * H_seg);
+}
+
+extern "C" int fa_seghist_segmented(fa_stream_t stream, fa_dtype t, fa_op op, const void *is,
+                                    int is64, const void *vs, int64_t m, int64_t seg_len,
+                                    void *dest, int64_t H_seg, void *scratch,
+                                    size_t scratch_bytes) {
+  if (m < 0 || seg_len < 0 || H_seg < 0) return FA_EINVAL;
+  if (m > 0 && ((H_seg > 0 && dest == nullptr) || (seg_len > 0 && (is == nullptr || vs == nullptr))))
+    return FA_EINVAL;
+  // m * seg_len and m * H_seg must be representable
+  if (m > 0 && (seg_len > INT64_MAX / m || H_seg > INT64_MAX / m)) return FA_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (t) {
+    case FA_I32: case FA_I64: case FA_F32: case FA_F64:
+      break;
+    default:
+      return FA_ENOTSUP;
+  }
+  FA_DISPATCH_TYPE_OP(launch_hist_segmented, t, op, s, is, is64, vs, m, seg_len, dest, H_seg,
+                      scratch, scratch_bytes);
 }

@@ -386,6 +386,47 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
   return 0;
 }
 
+/* `map2 (hist op ne k) iss vss`: one histogram of k bins per row. */
+static int do_seghist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                      struct fut_array **out, int64_t k, const struct fut_array *iss,
+                      const struct fut_array *vss, const char *entry) {
+  const int64_t m = iss->shape[0], len = iss->shape[1];
+  if (vss->shape[0] != m || vss->shape[1] != len) return bad_sizes(ctx, entry);
+  if (k < 0) {
+    rts_set_error(ctx, rts_msgprintf("Error: negative histogram size %lld.\n", (long long)k));
+    return FUTHARK_PROGRAM_ERROR;
+  }
+  const int64_t dims[2] = {m, k};
+  struct fut_array *res = out_array(ctx, m * k * (int64_t)es, 2, dims, "seghist.dest");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  int err = 0;
+  if (m * k > 0) {
+    int code = fa_replicate(ctx->stream, (int)es, res->mem.mem, m * k, neutral_bits(t, op));
+    err = rts_kernel_end(ctx, NULL, "replicate", code);
+  }
+  struct memblock_device scratch = {0};
+  if (err == 0)
+    err = rts_memblock_alloc(ctx, &scratch,
+                             (int64_t)fa_seghist_segmented_scratch_bytes(t, m, len, k),
+                             "seghist.scratch");
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "seghist_segmented",
+        rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld,\"bins\":%lld}", (long long)m,
+                      (long long)len, (long long)k));
+    int code = fa_seghist_segmented(ctx->stream, t, op, iss->mem.mem, 0, vss->mem.mem, m, len,
+                                    res->mem.mem, k, scratch.mem, (size_t)scratch.size);
+    err = rts_kernel_end(ctx, ev, "seghist_segmented", code);
+  }
+  rts_memblock_unref(ctx, &scratch, "seghist.scratch");
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
 #define ENTER(ctx) pthread_mutex_lock(&(ctx)->lock)
 #define LEAVE(ctx) pthread_mutex_unlock(&(ctx)->lock)
 
@@ -442,6 +483,16 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
     ENTER(ctx);                                                                               \
     int ret =                                                                                 \
         do_segreduce(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a);   \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_seghist_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_2d **out0, const int64_t in0,     \
+                                       const struct futhark_i32_2d *in1,                      \
+                                       const struct futhark_##T##_2d *in2) {                  \
+    ENTER(ctx);                                                                               \
+    int ret = do_seghist(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, in0,    \
+                         &in1->a, &in2->a, "seghist_" #OP "_" #T);                            \
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }                                                                                           \

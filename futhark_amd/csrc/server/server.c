@@ -186,6 +186,11 @@ struct entry {
     return futhark_entry_segreduce_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,        \
                                               ARRP(i[0]));                                     \
   }                                                                                            \
+  static int e_seghist_##OP##_##T(struct futhark_context *c, struct value *o,                  \
+                                  struct value **i) {                                          \
+    return futhark_entry_seghist_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,          \
+                                            i[0]->u.i64, ARRP(i[1]), ARRP(i[2]));              \
+  }                                                                                            \
   HIST_ENTRY_FNS(OP, T, CT)
 #define HIST_ENTRY_FNS(OP, T, CT)                                                              \
   static int e_hist_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) { \
@@ -264,6 +269,8 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
    {0}, {NULL}},                                                                                \
   {"segreduce_" #OP "_" #T, e_segreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0},            \
    {SEGRED_PARAM, NULL}},                                                                       \
+  {"seghist_" #OP "_" #T, e_seghist_##OP##_##T, "[][]" #T, 1, 3,                                \
+   {"i64", "[][]i32", "[][]" #T}, {0}, {HIST_PARAM, NULL}},                                     \
   HIST_ENTRY_ROWS(OP, T, CT)
 #define HIST_ENTRY_ROWS(OP, T, CT)                                                              \
   {"hist_" #OP "_" #T, e_hist_##OP##_##T, "[]" #T, 1, 3, {"i64", "[]i32", "[]" #T}, {0},        \

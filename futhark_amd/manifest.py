@@ -49,6 +49,8 @@ def entry_points() -> dict:
                 _entry(f"segscan_{op}_{t}", a, [("flags", "[]u8"), ("vs", a)]),
                 _entry(f"segred_{op}_{t}", a, [("offsets", "[]i64"), ("lens", "[]i64"), ("vs", a)]),
                 _entry(f"segreduce_{op}_{t}", a, [("xss", "[]" + a)], [SEGRED_PARAM]),
+                _entry(f"seghist_{op}_{t}", "[]" + a,
+                       [("k", "i64"), ("iss", "[][]i32"), ("vss", "[]" + a)], [HIST_PARAM]),
             ]
     for t in list(NUM_TYPES) + list(HIST_ONLY_TYPES):
         for op in ops_for(t):

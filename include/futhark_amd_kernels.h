@@ -143,6 +143,16 @@ int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op,
                const void *is, int is64, const void *vs, int64_t n,
                void *dest, int64_t H, void *scratch, size_t scratch_bytes);
 
+/* Segmented form, `map2 (hist op ne H_seg) iss vss` over [m][seg_len] inputs
+ * (SegHist.hs:1057-1136 with segment dimensions; tests/hist/segmented.fut):
+ * dest is [m][H_seg], row r receives the elements of row r whose index lies in
+ * [0, H_seg).  t is FA_I32, FA_I64, FA_F32 or FA_F64. */
+size_t fa_seghist_segmented_scratch_bytes(fa_dtype t, int64_t m, int64_t seg_len, int64_t H_seg);
+int fa_seghist_segmented(fa_stream_t stream, fa_dtype t, fa_op op,
+                         const void *is, int is64, const void *vs,
+                         int64_t m, int64_t seg_len, void *dest, int64_t H_seg,
+                         void *scratch, size_t scratch_bytes);
+
 /* -------------------------------------------------------------- radix sort
  * Stable LSD radix sort with 8-bit digits: per pass a digit histogram
  * (SegHist), an exclusive scan of the counts (SegScan) and a ranked scatter

@@ -23,6 +23,9 @@
  *   entry segreduce_OP_T (xss: [][]T) : []T    = map (reduce OP NE) xss
  *   entry hist_OP_T (k: i64) (is: []i32) (vs: []T) : [k]T =
  *     hist OP NE k (map i64.i32 is) vs           -- prelude/soacs.fut:132-146
+ *   entry seghist_OP_T (k: i64) (iss: [][]i32) (vss: [][]T) : [][]T =
+ *     map2 (\is vs -> hist OP NE k (map i64.i32 is) vs) iss vss
+ *                                   -- tests/hist/segmented.fut
  *   entry rbi_OP_T (dest: *[]T) (is: []i32) (vs: []T) : []T =
  *     reduce_by_index dest OP NE (map i64.i32 is) vs
  *   entry bmm_f32 (A: [][][]f32) (B: [][][]f32) : [][][]f32 =
@@ -243,6 +246,10 @@ FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
   int futhark_entry_segreduce_##OP##_##T(struct futhark_context *ctx,                         \
                                          struct futhark_##T##_1d **out0,                      \
                                          const struct futhark_##T##_2d *in0);                 \
+  int futhark_entry_seghist_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_2d **out0, const int64_t in0,     \
+                                       const struct futhark_i32_2d *in1,                      \
+                                       const struct futhark_##T##_2d *in2);                   \
   FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)
 
 #define FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)                                               \

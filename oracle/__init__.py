@@ -128,6 +128,16 @@ def hist(op: str, t: str, k: int, is_, vs, variant: str = "lit"):
     return rbi(op, t, np.full(k, NEUTRAL[(op, t)], dtype=dt), is_, vs, variant)
 
 
+def seghist(op: str, t: str, k: int, iss, vss, variant: str = "lit"):
+    """map2 (hist op ne k) iss vss (tests/hist/segmented.fut): one histogram per row."""
+    _, dt = _CT[t]
+    iss, vss = np.asarray(iss), np.asarray(vss)
+    out = np.empty((iss.shape[0], k), dtype=dt)
+    for r in range(iss.shape[0]):
+        out[r] = hist(op, t, k, iss[r], vss[r], variant)
+    return out
+
+
 def bmm_f32(A, B, variant: str = "f64acc"):
     A, B = _arr(A, np.float32), _arr(B, np.float32)
     if A.ndim == 2:

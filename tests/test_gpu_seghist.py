@@ -111,3 +111,64 @@ def test_config3_full_size_f32(ctx, H):
     out = ctx.call("hist_add_f32", ["f32_1d"], H, i, w)
     got, ref = out.values(), oracle.hist("add", "f32", H, is_, ws, "f64acc")
     assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(ref))
+
+
+# ------------------------------------------------------------ segmented histograms
+SEG_SHAPES = [  # (rows, row length, bins per row)
+    (3, 3, 10),          # tests/hist/segmented.fut
+    (1, 100003, 50),     # a single row is the unsegmented histogram
+    (1000, 1, 7),        # rows shorter than a vector
+    (777, 3, 5), (50, 1001, 64), (4096, 256, 16),
+    (7, 70001, 5000),    # several LDS ranges
+    (40, 5003, 30011),   # more bins than one launch of LDS ranges holds: flattened indices
+    (0, 5, 3), (4, 0, 3), (4, 6, 0),
+]
+
+
+@pytest.mark.parametrize("t,op", [("i32", "add"), ("i64", "max"), ("f32", "min"), ("i32", "xor"),
+                                  ("f64", "add")])
+def test_segmented_hist(ctx, t, op):
+    rng = np.random.default_rng(17)
+    for m, k, H in SEG_SHAPES:
+        iss = rng.integers(-2, max(H, 1) + 2, (m, k)).astype(np.int32)
+        if t[0] == "f":
+            vss = rng.integers(-50, 50, (m, k)).astype(NP[t])  # sums exact in any order
+        else:
+            vss = rng.integers(-1000, 1000, (m, k)).astype(NP[t])
+        i, v = ctx.new("i32_2d", iss), ctx.new(f"{t}_2d", vss)
+        out = ctx.call(f"seghist_{op}_{t}", [f"{t}_2d"], H, i, v)
+        assert out.shape == (m, H)
+        want = oracle.seghist(op, t, H, iss, vss)
+        assert np.array_equal(out.values(), want), (m, k, H)
+        for h in (out, i, v):
+            h.free()
+
+
+def test_segmented_hist_reference_golden_and_size_check(ctx, goldens):
+    c = goldens["hist_segmented"]["cases"][0]
+    xss = np.array(c["xss"], np.int32)
+    i, v = ctx.new("i32_2d", xss), ctx.new("i32_2d", np.ones_like(xss))
+    out = ctx.call("seghist_add_i32", ["i32_2d"], c["m"], i, v)
+    assert out.values().tolist() == c["out"]
+    out.free()
+    w = ctx.new("i32_2d", np.ones((3, 4), np.int32))
+    with pytest.raises(Exception, match="invalid sizes"):
+        ctx.call("seghist_add_i32", ["i32_2d"], 5, i, w)
+    for h in (i, v, w):
+        h.free()
+
+
+def test_segmented_hist_full_size_matches_row_sums(ctx):
+    # 2^27 elements in 2^14 rows; every row's histogram total equals the row's in-range sum
+    m, k, H = 1 << 14, 1 << 13, 64
+    iss = dg.hist_indices(90, m * k, H, "uniform", 1).reshape(m, k)
+    vss = dg.uniform_int(91, m * k, -1000, 1000).reshape(m, k)
+    i, v = ctx.new("i32_2d", iss), ctx.new("i32_2d", vss)
+    out = ctx.call("seghist_add_i32", ["i32_2d"], H, i, v)
+    got = out.values()
+    ok = (iss >= 0) & (iss < H)
+    assert np.array_equal(got.sum(axis=1, dtype=np.int64), np.where(ok, vss, 0).sum(axis=1, dtype=np.int64))
+    rows = [0, 1, m // 2, m - 1]
+    assert np.array_equal(got[rows], oracle.seghist("add", "i32", H, iss[rows], vss[rows]))
+    for h in (out, i, v):
+        h.free()
