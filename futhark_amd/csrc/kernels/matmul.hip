@@ -509,7 +509,68 @@ template <class Kern> static int raise_lds(Kern k, int bytes) {
 
 }  // namespace fa
 
-extern "C" int fa_matmul(fa_stream_t stream, fa_dtype in_t, const void *A, const void *B, float *C,
+// ---------------------------------------------------------- padded operands
+// Shapes the MFMA kernels do not take (M or N not a multiple of 256, K not a
+// multiple of the k-step) run on zero-padded copies of A and B in a workspace
+// when that is cheaper than the scalar kernel: dst[b][r][c] = src[b][r][c]
+// inside [rows][cols] and 0 outside, and the [M][N] corner of the padded
+// product is copied out.  Padding K with zeros adds zeros to every sum; padded
+// rows of A and columns of B only produce elements that are not copied.
+template <class T>
+__global__ __launch_bounds__(256) void mm_pad_kernel(const T *__restrict__ src, T *__restrict__ dst,
+                                                     int64_t rows, int64_t cols, int64_t rows_p,
+                                                     int64_t cols_p) {
+  const int64_t b = blockIdx.z;
+  const int64_t r = (int64_t)blockIdx.y;
+  const T *s = src + (b * rows + r) * cols;
+  T *d = dst + (b * rows_p + r) * cols_p;
+  const bool row_in = r < rows;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols_p; c += (int64_t)gridDim.x * 256)
+    d[c] = (row_in && c < cols) ? s[c] : T(0);
+}
+
+__global__ __launch_bounds__(256) void mm_unpad_kernel(const float *__restrict__ src,
+                                                       float *__restrict__ dst, int64_t rows,
+                                                       int64_t cols, int64_t rows_p, int64_t cols_p) {
+  const int64_t b = blockIdx.z;
+  const int64_t r = (int64_t)blockIdx.y;
+  const float *s = src + (b * rows_p + r) * cols_p;
+  float *d = dst + (b * rows + r) * cols;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += (int64_t)gridDim.x * 256)
+    d[c] = s[c];
+}
+
+struct MmPlan {
+  bool direct_tiled;  // the MFMA kernels take the shape as it is
+  bool padded;        // run them on padded copies
+  int64_t Mp, Np, Kp;
+  size_t a_bytes, b_bytes, c_bytes;  // 256-byte multiples
+};
+
+static size_t mm_align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+static MmPlan mm_plan(fa_dtype in_t, int64_t batch, int64_t M, int64_t N, int64_t K) {
+  MmPlan p = {};
+  const int bk = in_t == FA_F32 ? MM32_BK : MM16_BK;
+  const size_t es = in_t == FA_F32 ? 4 : 2;
+  p.direct_tiled = M % MM_BM == 0 && N % MM_BN == 0 && K % bk == 0 && K > 0;
+  if (p.direct_tiled || batch * M * N == 0 || K == 0) return p;
+  p.Mp = ceil_div(M, (int64_t)MM_BM) * MM_BM;
+  p.Np = ceil_div(N, (int64_t)MM_BN) * MM_BN;
+  p.Kp = ceil_div(K, (int64_t)bk) * bk;
+  // Worth it when there is enough work to pay for four more launches and the
+  // padding does not multiply the work too much: the scalar kernel runs at a
+  // few percent of the MFMA rate.
+  const double work = (double)batch * M * N * K, padded_work = (double)batch * p.Mp * p.Np * p.Kp;
+  p.padded = work >= (double)(1 << 24) && padded_work <= 8.0 * work && p.Mp <= 65535 &&
+             batch <= 65535;
+  p.a_bytes = mm_align((size_t)batch * p.Mp * p.Kp * es);
+  p.b_bytes = mm_align((size_t)batch * p.Kp * p.Np * es);
+  p.c_bytes = mm_align((size_t)batch * p.Mp * p.Np * 4);
+  return p;
+}
+
+static int matmul_direct(fa_stream_t stream, fa_dtype in_t, const void *A, const void *B, float *C,
                          int64_t batch, int64_t M, int64_t N, int64_t K) {
   if (batch < 0 || M < 0 || N < 0 || K < 0) return FA_EINVAL;
   if (in_t != FA_F32 && in_t != FA_F16 && in_t != FA_BF16) return FA_ENOTSUP;
@@ -556,4 +617,56 @@ extern "C" int fa_matmul(fa_stream_t stream, fa_dtype in_t, const void *A, const
     hipLaunchKernelGGL((matmul_generic_kernel<uint16_t, 2>), grid, dim3(256), 0, st,
                        (const uint16_t *)A, (const uint16_t *)B, C, M, N, K);
   return launch_status();
+}
+
+extern "C" size_t fa_matmul_workspace_bytes(fa_dtype in_t, int64_t batch, int64_t M, int64_t N,
+                                            int64_t K) {
+  if (batch < 0 || M < 0 || N < 0 || K < 0) return 0;
+  if (in_t != FA_F32 && in_t != FA_F16 && in_t != FA_BF16) return 0;
+  const MmPlan p = mm_plan(in_t, batch, M, N, K);
+  return p.padded ? p.a_bytes + p.b_bytes + p.c_bytes : 0;
+}
+
+template <class T>
+static int mm_pad(hipStream_t st, const void *src, void *dst, int64_t batch, int64_t rows,
+                  int64_t cols, int64_t rows_p, int64_t cols_p) {
+  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(cols_p, (int64_t)256), 64), (unsigned)rows_p,
+                  (unsigned)batch);
+  hipLaunchKernelGGL((mm_pad_kernel<T>), grid, dim3(256), 0, st, (const T *)src, (T *)dst, rows, cols,
+                     rows_p, cols_p);
+  return launch_status();
+}
+
+extern "C" int fa_matmul_ws(fa_stream_t stream, fa_dtype in_t, const void *A, const void *B,
+                            float *C, int64_t batch, int64_t M, int64_t N, int64_t K,
+                            void *workspace, size_t workspace_bytes) {
+  if (batch < 0 || M < 0 || N < 0 || K < 0) return FA_EINVAL;
+  if (in_t != FA_F32 && in_t != FA_F16 && in_t != FA_BF16) return FA_ENOTSUP;
+  const MmPlan p = mm_plan(in_t, batch, M, N, K);
+  if (!p.padded || workspace == nullptr || workspace_bytes < p.a_bytes + p.b_bytes + p.c_bytes ||
+      !is_aligned(workspace, 256))
+    return matmul_direct(stream, in_t, A, B, C, batch, M, N, K);
+  if (C == nullptr || A == nullptr || B == nullptr) return FA_EINVAL;
+  hipStream_t st = (hipStream_t)stream;
+  char *Ap = (char *)workspace, *Bp = Ap + p.a_bytes, *Cp = Bp + p.b_bytes;
+  int rc;
+  if (in_t == FA_F32) {
+    rc = mm_pad<float>(st, A, Ap, batch, M, K, p.Mp, p.Kp);
+    if (rc == 0) rc = mm_pad<float>(st, B, Bp, batch, K, N, p.Kp, p.Np);
+  } else {
+    rc = mm_pad<uint16_t>(st, A, Ap, batch, M, K, p.Mp, p.Kp);
+    if (rc == 0) rc = mm_pad<uint16_t>(st, B, Bp, batch, K, N, p.Kp, p.Np);
+  }
+  if (rc != 0) return rc;
+  rc = matmul_direct(stream, in_t, Ap, Bp, (float *)Cp, batch, p.Mp, p.Np, p.Kp);
+  if (rc != 0) return rc;
+  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(N, (int64_t)256), 64), (unsigned)M,
+                  (unsigned)batch);
+  hipLaunchKernelGGL(mm_unpad_kernel, grid, dim3(256), 0, st, (const float *)Cp, C, M, N, p.Mp, p.Np);
+  return launch_status();
+}
+
+extern "C" int fa_matmul(fa_stream_t stream, fa_dtype in_t, const void *A, const void *B, float *C,
+                         int64_t batch, int64_t M, int64_t N, int64_t K) {
+  return matmul_direct(stream, in_t, A, B, C, batch, M, N, K);
 }

@@ -554,14 +554,22 @@ static int do_bmm(struct futhark_context *ctx, fa_dtype in_t, struct fut_array *
   struct fut_array *res =
       out_array(ctx, b * M * N * 4, rank, rank == 3 ? dims3 : dims2, "bmm.out");
   if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
-  struct rts_event *ev = rts_kernel_begin(
-      ctx, "segmap_matmul",
-      rts_msgprintf("{\"batch\":%lld,\"M\":%lld,\"N\":%lld,\"K\":%lld,\"flop\":%lld}",
-                    (long long)b, (long long)M, (long long)N, (long long)K,
-                    (long long)(2 * b * M * N * K)));
-  int code = fa_matmul(ctx->stream, in_t, A->mem.mem, B->mem.mem, (float *)res->mem.mem, b, M,
-                       N, K);
-  int err = rts_kernel_end(ctx, ev, "segmap_matmul", code);
+  struct memblock_device ws = {0};
+  const size_t ws_bytes = fa_matmul_workspace_bytes(in_t, b, M, N, K);
+  int err = 0;
+  if (ws_bytes > 0) err = rts_memblock_alloc(ctx, &ws, (int64_t)ws_bytes, "bmm.workspace");
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "segmap_matmul",
+        rts_msgprintf("{\"batch\":%lld,\"M\":%lld,\"N\":%lld,\"K\":%lld,\"flop\":%lld,"
+                      "\"padded\":%s}",
+                      (long long)b, (long long)M, (long long)N, (long long)K,
+                      (long long)(2 * b * M * N * K), ws_bytes > 0 ? "true" : "false"));
+    int code = fa_matmul_ws(ctx->stream, in_t, A->mem.mem, B->mem.mem, (float *)res->mem.mem, b,
+                            M, N, K, ws.mem, ws_bytes);
+    err = rts_kernel_end(ctx, ev, "segmap_matmul", code);
+  }
+  rts_memblock_unref(ctx, &ws, "bmm.workspace");
   if (err != 0) {
     drop_array(ctx, res);
     return err;

@@ -176,6 +176,17 @@ int fa_radix_sort(fa_stream_t stream, int key_bytes, int val_bytes,
 int fa_matmul(fa_stream_t stream, fa_dtype in_t,
               const void *A, const void *B, float *C,
               int64_t batch, int64_t M, int64_t N, int64_t K);
+/* The same with a workspace of fa_matmul_workspace_bytes() bytes (256-byte
+ * aligned; may be NULL when that is 0).  Shapes the MFMA kernels do not take
+ * directly (M or N not a multiple of 256, K not a multiple of 64, or 16 for
+ * f32) then run on zero-padded copies of the operands instead of on the scalar
+ * kernel, when the padding costs less than that (mmBlkRegTiling guards every
+ * load and store instead, BlkRegTiling.hs:219-254). */
+size_t fa_matmul_workspace_bytes(fa_dtype in_t, int64_t batch, int64_t M, int64_t N, int64_t K);
+int fa_matmul_ws(fa_stream_t stream, fa_dtype in_t,
+                 const void *A, const void *B, float *C,
+                 int64_t batch, int64_t M, int64_t N, int64_t K,
+                 void *workspace, size_t workspace_bytes);
 
 /* ------------------------------------------------ builtin data movement
  * Batched 2-D transpose: dst[b][j][i] = src[b][i][j], src : [batch][rows][cols].

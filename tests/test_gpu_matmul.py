@@ -87,3 +87,26 @@ def test_config4_full_size(ctx, t, tol, b, m):
     rhs = np.matmul(Af.astype(np.float64), Bf.astype(np.float64).sum(axis=2)[..., None])[..., 0]
     scale = np.matmul(np.abs(Af).astype(np.float64), np.abs(Bf).astype(np.float64).sum(axis=2)[..., None])[..., 0]
     assert np.all(np.abs(lhs - rhs) <= tol * scale)
+
+
+@pytest.mark.parametrize("t,tol", [("f32", 1e-5), ("f16", 1e-2), ("bf16", 1e-2)])
+def test_ragged_shapes_through_padded_operands(ctx, t, tol):
+    """Shapes that are no multiples of the MFMA tile but large enough to run on
+    zero-padded copies; every output element is checked, and the report says
+    which way the product went."""
+    import json
+    from futhark_amd import Context
+    with Context(ctx.so, profiling=True) as c:
+        shapes = [(1, 300, 500, 200, True), (3, 257, 255, 129, True), (1, 1000, 1000, 1000, True),
+                  (4, 256, 256, 100, True), (1, 511, 256, 192, True), (1, 2011, 515, 777, True),
+                  (1, 255, 256, 64, False),     # too little work to pay for the copies
+                  (1, 2000, 3, 2000, False)]    # padding would multiply the work by 85
+        for b, M, N, K, _ in shapes:
+            Ain, Bin, Af, Bf, kind = _inputs(t, b, M, N, K, 66)
+            out = c.call(f"bmm_{t}", ["f32_3d"], c.new(kind, Ain), c.new(kind, Bin))
+            got = out.values()
+            assert got.shape == (b, M, N)
+            _check(got, Af, Bf, tol)
+            out.free()
+        ev = [e for e in json.loads(c.report())["events"] if e["name"] == "segmap_matmul"]
+        assert [e["details"]["padded"] for e in ev] == [p for *_, p in shapes], ev
