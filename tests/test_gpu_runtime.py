@@ -1,0 +1,132 @@
+"""The C runtime under the entry points, through the public API only: pooled
+device memory (rts/c/gpu.h:245-331, free_list.h), error reporting
+(docs/c-api.rst:37-58,153-166), contexts side by side, device selection,
+profiling report and logging."""
+import json
+import threading
+
+import numpy as np
+import pytest
+
+from futhark_amd import Context, FutharkError
+
+pytestmark = pytest.mark.gpu
+
+
+def test_out_of_memory_is_reported_and_does_not_stick(segops_lib):
+    with Context(segops_lib) as c:
+        small = c.call("iota_i64", ["i64_1d"], 1000)
+        small.free()                                      # a pooled block the retry loop may release
+        with pytest.raises(FutharkError) as e:
+            c.call("iota_i64", ["i64_1d"], 1 << 40)       # 8 TiB
+        assert e.value.code == 3                          # FUTHARK_OUT_OF_MEMORY
+        assert "Failed to allocate memory in space 'device'" in e.value.message
+        assert c.get_error() is None                      # reading the message cleared it
+        out = c.call("iota_i64", ["i64_1d"], 1000)        # the context is still usable
+        assert out.values()[-1] == 999
+        out.free()
+        with pytest.raises(FutharkError, match="Range 0..<-1 is invalid") as e:
+            c.call("iota_i64", ["i64_1d"], -1)
+        assert e.value.code == 2                          # FUTHARK_PROGRAM_ERROR
+
+
+def test_freed_blocks_are_reused_and_clear_caches_returns_them(segops_lib):
+    with Context(segops_lib) as c:
+        a = c.call("iota_i64", ["i64_1d"], 1 << 20)
+        p = a.device_ptr
+        a.free()
+        b = c.call("iota_i64", ["i64_1d"], 1 << 20)       # same size, same tag: the pooled block
+        assert b.device_ptr == p
+        assert b.values()[12345] == 12345
+        b.free()
+        c.clear_caches()
+        d = c.call("iota_i64", ["i64_1d"], 1 << 20)
+        assert d.values()[-1] == (1 << 20) - 1
+        d.free()
+
+
+def test_values_are_reference_counted_through_aliases(segops_lib):
+    with Context(segops_lib) as c:
+        k = c.new("u32_1d", np.array([3, 1, 2], np.uint32))
+        v = c.new("i32_1d", np.array([0, 1, 2], np.int32))
+        t = c.new_opaque("tup2_arr1d_u32_arr1d_i32", k, v)
+        alias = t.project(0)
+        assert alias.device_ptr == k.device_ptr           # an alias, not a copy
+        k.free(); t.free()                                # two of three references gone
+        junk = c.new("u32_1d", np.array([9, 9, 9], np.uint32))   # would reuse a freed block
+        assert junk.device_ptr != alias.device_ptr
+        assert alias.values().tolist() == [3, 1, 2]
+        for h in (alias, junk, v):
+            h.free()
+
+
+def test_two_contexts_and_two_threads(segops_lib):
+    xs = np.arange(100000, dtype=np.int32)
+    results = {}
+
+    def work(name, scale):
+        with Context(segops_lib) as c:
+            a = c.new("i32_1d", (xs.astype(np.int64) * scale).astype(np.int32))
+            for _ in range(20):
+                results[name] = int(c.call("reduce_add_i32", [np.int32], a))
+            a.free()
+
+    ts = [threading.Thread(target=work, args=(f"t{s}", s)) for s in (1, 2, 3)]
+    for t in ts:
+        t.start()
+    for t in ts:
+        t.join()
+    base = int(xs.astype(np.int64).sum())
+    wrap = lambda x: int(np.array(x, np.int64).astype(np.int32))   # i32 addition wraps
+    assert results == {f"t{s}": wrap(base * s) for s in (1, 2, 3)}
+
+
+def test_device_selection(segops_lib):
+    with Context(segops_lib, device="#0") as c:
+        assert c.call("reduce_add_i32", [np.int32], c.new("i32_1d", np.ones(10, np.int32))) == 10
+    with pytest.raises(FutharkError):
+        Context(segops_lib, device="#7")                  # one GPU on the box
+    with pytest.raises(FutharkError):
+        Context(segops_lib, device="no such device name")
+
+
+def test_profiling_report_and_pause(segops_lib):
+    with Context(segops_lib, profiling=True) as c:
+        a = c.new("f32_1d", np.ones(4096, np.float32))
+        c.call("scan_add_f32", ["f32_1d"], a).free()
+        c.L.futhark_context_pause_profiling(c.ptr)
+        c.call("reduce_add_f32", [np.float32], a)
+        c.L.futhark_context_unpause_profiling(c.ptr)
+        c.call("exscan_add_f32", ["f32_1d"], a).free()
+        rep = json.loads(c.report())
+        names = [e["name"] for e in rep["events"]]
+        assert names.count("segscan") == 2 and not any("segred" in n for n in names), names
+        assert all(e["duration"] > 0 and isinstance(e["details"], dict) for e in rep["events"])
+        assert rep["memory"]["device"] >= 2 * 4096 * 4      # peak: the input and one result
+        assert json.loads(c.report())["events"] == []     # a report empties the event list
+        a.free()
+    with Context(segops_lib) as c:                        # profiling off: nothing is recorded
+        a = c.new("f32_1d", np.ones(16, np.float32))
+        c.call("scan_add_f32", ["f32_1d"], a).free()
+        assert json.loads(c.report())["events"] == []
+        a.free()
+
+
+def test_debugging_log_goes_to_the_logging_file(segops_lib, tmp_path):
+    import ctypes as C
+    libc = C.CDLL(None)
+    libc.fopen.restype = C.c_void_p
+    libc.fopen.argtypes = [C.c_char_p, C.c_char_p]
+    libc.fclose.argtypes = [C.c_void_p]
+    path = tmp_path / "log.txt"
+    f = libc.fopen(str(path).encode(), b"w")
+    assert f
+    with Context(segops_lib, debugging=True) as c:
+        segops_lib.lib.futhark_context_set_logging_file.argtypes = [C.c_void_p, C.c_void_p]
+        segops_lib.lib.futhark_context_set_logging_file(c.ptr, f)
+        a = c.new("i32_1d", np.ones(100, np.int32))
+        c.call("scan_add_i32", ["i32_1d"], a).free()
+        a.free()
+    libc.fclose(f)
+    text = path.read_text()
+    assert "Allocating" in text and "segscan" in text
