@@ -4,6 +4,9 @@
   futhark_amd/lib/libsegops.so                C runtime + `segops` program API (gcc)
   futhark_amd/lib/libfuthark_amd_values.so    Futhark value reader/writer (gcc)
   futhark_amd/bin/segops-server               server executable of the program (gcc)
+  futhark_amd/bin/segops                      command-line executable of the program (gcc)
+  futhark_amd/bin/capi-harness                tests/c/capi_harness.c against include/segops.h
+  include/segops.json                         manifest of the program library
   oracle/liboracle.so                         CPU oracle and CPU baseline (gcc)
 
 Run as `python -m futhark_amd.build` or through `__graft_entry__.build()`.
@@ -101,6 +104,12 @@ def build_server() -> Path:
     _run(["gcc", *server_flags, "-c", str(CSRC / "server" / "server.c"), "-o", str(server_obj)])
     out = bindir / "segops-server"
     _run(["gcc", "-o", str(out), str(server_obj), str(values_obj), f"-L{LIB}", "-lsegops",
+          "-lfuthark_amd_kernels", f"-L{ROCM / 'lib'}", "-lamdhip64", "-lm",
+          "-Wl,-rpath,$ORIGIN/../lib", f"-Wl,-rpath,{ROCM / 'lib'}"])
+    # The command-line executable (`futhark hip prog.fut` without --server).
+    cli_obj = OBJ / "server_cli.o"
+    _run(["gcc", *server_flags, "-c", str(CSRC / "server" / "cli.c"), "-o", str(cli_obj)])
+    _run(["gcc", "-o", str(bindir / "segops"), str(cli_obj), str(values_obj), f"-L{LIB}", "-lsegops",
           "-lfuthark_amd_kernels", f"-L{ROCM / 'lib'}", "-lamdhip64", "-lm",
           "-Wl,-rpath,$ORIGIN/../lib", f"-Wl,-rpath,{ROCM / 'lib'}"])
     # A C program written against the public header only, the way a user of a

@@ -227,12 +227,261 @@ int fv_write_text(FILE *f, const struct fv_primtype *t, int rank, const int64_t 
   return ferror(f) ? 1 : 0;
 }
 
-int fv_end_of_input(FILE *f) {
+/* ------------------------------------------------------------ textual input
+ * The syntax rts/c/values.h:14-398 accepts.  Tokens are maximal runs of
+ * letters, digits and . - + _, or single other characters; `--` starts a
+ * comment that runs to the end of the line.  A value of rank r is r levels of
+ * [ ... , ... ] with rows of equal length, or empty([d0]...[dr-1]T) with some
+ * dimension 0.  Numbers may contain underscores and may carry their type as a
+ * suffix; integers also come in hexadecimal and octal (C's %i); u64 is decimal
+ * only; floats have T.nan, T.inf, -T.inf; bool is true / false. */
+struct text_parser {
+  FILE *f;
+  char tok[128];
+  int have; /* tok holds a token that was peeked at but not consumed */
+};
+
+static int is_constituent(int c) {
+  return isalnum(c) || c == '.' || c == '-' || c == '+' || c == '_';
+}
+
+/* An empty token means end of input. */
+static const char *peek_token(struct text_parser *p) {
+  if (p->have) return p->tok;
+  p->have = 1;
+  int c, n = 0;
+  for (;;) {
+    do {
+      c = getc(p->f);
+    } while (c != EOF && isspace(c));
+    if (c != '-') break;
+    const int d = getc(p->f);
+    if (d != '-') {
+      if (d != EOF) ungetc(d, p->f);
+      break;
+    }
+    while (c != '\n' && c != EOF) c = getc(p->f);
+  }
+  if (c == EOF) {
+    p->tok[0] = 0;
+    return p->tok;
+  }
+  p->tok[n++] = (char)c;
+  if (is_constituent(c)) {
+    while ((c = getc(p->f)) != EOF && is_constituent(c))
+      if (n < (int)sizeof(p->tok) - 1) p->tok[n++] = (char)c;
+    if (c != EOF) ungetc(c, p->f);
+  }
+  p->tok[n] = 0;
+  return p->tok;
+}
+
+static const char *next_token(struct text_parser *p) {
+  const char *t = peek_token(p);
+  p->have = 0;
+  return t;
+}
+
+static int accept_token(struct text_parser *p, const char *want) {
+  if (strcmp(peek_token(p), want) != 0) return 0;
+  p->have = 0;
+  return 1;
+}
+
+/* float -> binary16 the way the reference's reader narrows (float2halfbits,
+ * rts/c/half.h:220-228, tables after van der Zijp): the mantissa is cut, not
+ * rounded; too small goes to zero, too large to infinity. */
+static uint16_t float_to_half_bits_truncating(float v) {
+  uint32_t x;
+  memcpy(&x, &v, 4);
+  const uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  const int e = (int)((x >> 23) & 0xff);
+  const uint32_t man = x & 0x7fffffu;
+  if (e < 103) return sign;
+  if (e < 113) return (uint16_t)(sign | ((0x0400u >> (113 - e)) + (man >> (126 - e))));
+  if (e < 143) return (uint16_t)(sign | ((uint32_t)(e - 112) << 10) | (man >> 13));
+  if (e < 255) return (uint16_t)(sign | 0x7c00u);
+  return (uint16_t)(sign | 0x7c00u | (man >> 13));
+}
+
+/* The rest of a number token must be empty or the type's name. */
+static int suffix_ok(const char *rest, const char *name) {
+  return *rest == 0 || strcmp(rest, name) == 0;
+}
+
+static int parse_scalar(const char *token, const struct fv_primtype *t, unsigned char *dst) {
+  char buf[128];
+  size_t n = 0;
+  for (const char *r = token; *r && n < sizeof(buf) - 1; r++)
+    if (*r != '_') buf[n++] = *r;
+  buf[n] = 0;
+  const char *name = t->name;
+  if (strcmp(name, "bool") == 0) {
+    if (strcmp(token, "true") == 0) *dst = 1;
+    else if (strcmp(token, "false") == 0) *dst = 0;
+    else return 1;
+    return 0;
+  }
+  if (name[0] == 'f') {
+    char special[16];
+    double v;
+    int sign = 1;
+    const char *b = buf;
+    snprintf(special, sizeof special, "%s.nan", name);
+    if (strcmp(b, special) == 0) {
+      v = (double)NAN;
+    } else {
+      snprintf(special, sizeof special, "%s.inf", name);
+      if (b[0] == '-' && strcmp(b + 1, special) == 0) sign = -1, b++;
+      if (strcmp(b, special) == 0) {
+        v = sign * (double)INFINITY;
+      } else {
+        char *end;
+        if (t->size == 8) v = strtod(buf, &end);
+        else v = (double)strtof(buf, &end);
+        if (end == buf || !suffix_ok(end, name)) return 1;
+      }
+    }
+    if (t->size == 8) {
+      memcpy(dst, &v, 8);
+    } else if (t->size == 4) {
+      const float f = (float)v;
+      memcpy(dst, &f, 4);
+    } else {
+      const uint16_t h = float_to_half_bits_truncating((float)v);
+      memcpy(dst, &h, 2);
+    }
+    return 0;
+  }
+  /* integers: the digits the way scanf's %i reads them (sign, 0x, leading 0),
+   * u64 the way %u does; narrower types keep the low bits */
+  char *end;
+  if (strcmp(name, "u64") == 0) {
+    const char *d = buf;
+    if (*d == '+') d++;
+    if (!isdigit((unsigned char)*d)) return 1;
+    const uint64_t v = strtoull(d, &end, 10);
+    if (!suffix_ok(end, name)) return 1;
+    memcpy(dst, &v, 8);
+    return 0;
+  }
+  const char *d = buf;
+  if (*d == '-' || *d == '+') d++;
+  if (!isdigit((unsigned char)*d)) return 1;
+  const long long v = strtoll(buf, &end, 0);
+  if (end == buf || !suffix_ok(end, name)) return 1;
+  switch (t->size) {
+    case 1: { const int8_t x = (int8_t)v; memcpy(dst, &x, 1); } break;
+    case 2: { const int16_t x = (int16_t)v; memcpy(dst, &x, 2); } break;
+    case 4: { const int32_t x = (int32_t)v; memcpy(dst, &x, 4); } break;
+    default: { const int64_t x = (int64_t)v; memcpy(dst, &x, 8); } break;
+  }
+  return 0;
+}
+
+struct text_array {
+  const struct fv_primtype *t;
+  int rank;
+  int64_t *shape;
+  char known[FV_MAX_RANK];
+  unsigned char *elems;
+  size_t used, space; /* in elements */
+};
+
+static int parse_level(struct text_parser *p, struct text_array *a, int level) {
+  if (!accept_token(p, "[")) return 1;
+  int64_t count = 0;
+  while (strcmp(peek_token(p), "]") != 0) {
+    if (level == a->rank - 1) {
+      if (a->used == a->space) {
+        a->space *= 2;
+        unsigned char *grown = realloc(a->elems, a->space * (size_t)a->t->size);
+        if (grown == NULL) return 1;
+        a->elems = grown;
+      }
+      const char *tok = next_token(p);
+      if (*tok == 0 || parse_scalar(tok, a->t, a->elems + a->used * (size_t)a->t->size) != 0)
+        return 1;
+      a->used++;
+    } else if (parse_level(p, a, level + 1) != 0) {
+      return 1;
+    }
+    count++;
+    if (!accept_token(p, ",")) break; /* a comma may also precede the closing bracket */
+  }
+  if (!accept_token(p, "]")) return 1;
+  if (a->known[level]) return a->shape[level] != count;
+  a->known[level] = 1;
+  a->shape[level] = count;
+  return 0;
+}
+
+static int parse_empty(struct text_parser *p, const struct fv_primtype *t, int rank,
+                       int64_t *shape) {
+  if (!accept_token(p, "empty") || !accept_token(p, "(")) return 1;
+  int some_zero = 0;
+  for (int i = 0; i < rank; i++) {
+    if (!accept_token(p, "[")) return 1;
+    const char *tok = next_token(p);
+    char *end;
+    if (!isdigit((unsigned char)*tok)) return 1;
+    shape[i] = (int64_t)strtoull(tok, &end, 10);
+    if (*end != 0 || !accept_token(p, "]")) return 1;
+    some_zero |= shape[i] == 0;
+  }
+  if (!accept_token(p, t->name) || !accept_token(p, ")")) return 1;
+  return !some_zero;
+}
+
+int fv_read_text(FILE *f, const struct fv_primtype *t, int rank, int64_t *shape, void **data,
+                 char *err, size_t errlen) {
+  if (rank < 0 || rank > FV_MAX_RANK) return fail(err, errlen, "rank %d not supported", rank);
+  struct text_parser p = {f, {0}, 0};
+  if (*peek_token(&p) == 0) return fail(err, errlen, "end of input where a value was expected");
+  if (rank == 0) {
+    unsigned char *buf = malloc(8);
+    if (buf == NULL) return fail(err, errlen, "out of memory");
+    if (parse_scalar(next_token(&p), t, buf) != 0) {
+      free(buf);
+      return fail(err, errlen, "not a value of type %s: %s", t->name, p.tok);
+    }
+    *data = buf;
+    return 0;
+  }
+  if (strcmp(peek_token(&p), "empty") == 0) {
+    if (parse_empty(&p, t, rank, shape) != 0)
+      return fail(err, errlen, "malformed empty(...) for an array of %s of rank %d", t->name, rank);
+    *data = malloc(1);
+    return *data == NULL;
+  }
+  struct text_array a = {t, rank, shape, {0}, malloc(16 * (size_t)t->size), 0, 16};
+  if (a.elems == NULL) return fail(err, errlen, "out of memory");
+  if (parse_level(&p, &a, 0) != 0) {
+    free(a.elems);
+    return fail(err, errlen, "malformed array of %s of rank %d near '%s'", t->name, rank, p.tok);
+  }
+  /* dimensions inside an empty outer dimension were never seen */
+  for (int i = 0; i < rank; i++)
+    if (!a.known[i]) shape[i] = 0;
+  *data = a.elems;
+  return 0;
+}
+
+int fv_read_value(FILE *f, const struct fv_primtype *t, int rank, int64_t *shape, void **data,
+                  char *err, size_t errlen) {
   int c;
   do {
     c = getc(f);
   } while (c != EOF && isspace(c));
-  if (c == EOF) return 0;
-  ungetc(c, f);
-  return 1;
+  if (c != EOF) ungetc(c, f);
+  /* no textual value starts with the letter b (rts/c/values.h:590-610) */
+  if (c == 'b') return fv_read_binary(f, t, rank, shape, data, err, errlen);
+  return fv_read_text(f, t, rank, shape, data, err, errlen);
+}
+
+int fv_end_of_input(FILE *f) {
+  /* blanks and `--` comments may follow the last value (end_of_input,
+   * rts/c/values.h:713-722, reads a token) */
+  struct text_parser p = {f, {0}, 0};
+  return *peek_token(&p) != 0;
 }

@@ -3,6 +3,7 @@ data format (docs/binary-data-format.rst) and textual output, to and from numpy.
 
     write_binary(path_or_file, [array, ...])      one value after another
     read_binary(path, [("f32", 1), ("i64", 0)])   element type name and rank per value
+    read_text / read_values                       the textual syntax / whichever form each value has
 """
 from __future__ import annotations
 
@@ -36,6 +37,8 @@ class _Lib:
         self.v.fv_primtype.argtypes = [C.c_char_p]
         self.v.fv_read_binary.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(C.c_int64),
                                           C.POINTER(C.c_void_p), C.c_char_p, C.c_size_t]
+        self.v.fv_read_text.argtypes = self.v.fv_read_binary.argtypes
+        self.v.fv_read_value.argtypes = self.v.fv_read_binary.argtypes
         self.v.fv_write_binary.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.POINTER(C.c_int64),
                                            C.c_void_p]
         self.v.fv_write_text.argtypes = self.v.fv_write_binary.argtypes
@@ -91,6 +94,20 @@ def write_text(path, arrays) -> None:
 
 def read_binary(path, specs, expect_eof: bool = True):
     """specs: [(element type name, rank), ...]; returns numpy arrays (0-d for scalars)."""
+    return _read(path, specs, expect_eof, "fv_read_binary")
+
+
+def read_text(path, specs, expect_eof: bool = True):
+    """The same for values in the textual syntax."""
+    return _read(path, specs, expect_eof, "fv_read_text")
+
+
+def read_values(path, specs, expect_eof: bool = True):
+    """Each value in whichever of the two forms it is in."""
+    return _read(path, specs, expect_eof, "fv_read_value")
+
+
+def _read(path, specs, expect_eof, fn_name):
     L = _get()
     f = _open(path, b"rb")
     out = []
@@ -99,8 +116,8 @@ def read_binary(path, specs, expect_eof: bool = True):
             shape = (C.c_int64 * MAX_RANK)()
             data = C.c_void_p()
             err = C.create_string_buffer(256)
-            rc = L.v.fv_read_binary(f, L.v.fv_primtype(name.encode()), rank, shape, C.byref(data),
-                                    err, len(err))
+            rc = getattr(L.v, fn_name)(f, L.v.fv_primtype(name.encode()), rank, shape,
+                                       C.byref(data), err, len(err))
             if rc != 0:
                 raise ValueError_(err.value.decode())
             dims = tuple(shape[i] for i in range(rank))

@@ -1,7 +1,7 @@
 /* libfuthark_amd_values.so -- reading and writing Futhark values: the binary
  * data format (docs/binary-data-format.rst; the reference's reader/writer is
  * rts/c/values.h:498-812, pasted into every generated executable) and the
- * textual array syntax on output (rts/c/values.h:398-491,724-768).  Host memory
+ * textual syntax in both directions (rts/c/values.h:14-491,724-768).  Host memory
  * only.  The server executable and Python tools (futhark_amd/values.py) use it. */
 #ifndef FUTHARK_AMD_VALUES_H
 #define FUTHARK_AMD_VALUES_H
@@ -44,7 +44,20 @@ int fv_write_binary(FILE *f, const struct fv_primtype *t, int rank, const int64_
 int fv_write_text(FILE *f, const struct fv_primtype *t, int rank, const int64_t *shape,
                   const void *data);
 
-/* 0 if only whitespace remains before end of file. */
+/* Reads one value in the textual syntax (rts/c/values.h:14-398): nested
+ * brackets with rows of equal length, empty([0][3]i32), numbers with optional
+ * type suffix and underscores, hexadecimal integers, T.nan / T.inf / -T.inf,
+ * true / false, `--` comments.  Results as for fv_read_binary.  f16 literals are
+ * narrowed from float by cutting the mantissa, as the reference's reader does. */
+int fv_read_text(FILE *f, const struct fv_primtype *expect, int rank, int64_t *shape,
+                 void **data, char *err, size_t errlen);
+
+/* Reads one value in either form: binary if the next non-blank character is
+ * 'b', else textual (read_array / read_scalar, rts/c/values.h:705-712,814-829). */
+int fv_read_value(FILE *f, const struct fv_primtype *expect, int rank, int64_t *shape,
+                  void **data, char *err, size_t errlen);
+
+/* 0 if only blanks and `--` comments remain before end of file. */
 int fv_end_of_input(FILE *f);
 
 #ifdef __cplusplus

@@ -104,3 +104,97 @@ def test_text_form(tmp_path):
     assert text(np.array([0.1], np.float64)) == "[0.10000000000000001f64]"
     assert text(np.array([1.5, -2.0], np.float16)) == "[1.5f16, -2f16]"
     assert text(np.array(2 ** 64 - 1, np.uint64)) == "18446744073709551615u64"
+
+
+# ------------------------------------------------------------------ textual input
+def _read_text(tmp_path, text, specs, **kw):
+    p = tmp_path / "in.txt"
+    p.write_text(text)
+    return fv.read_text(p, specs, **kw)
+
+
+def test_text_reader_takes_the_inputs_of_the_reference_tests(tmp_path):
+    # input blocks as they stand in the reference's test programs
+    (a,) = _read_text(tmp_path, "[0i8, 0i8, 0i8, 0i8, 0i8]", [("i8", 1)])          # tests/hist/i8.fut:5
+    assert a.dtype == np.int8 and a.tolist() == [0] * 5
+    n, is_, img = _read_text(tmp_path, "5i64\n[1, 2, 1, 4, 5]\n[1i8, 1i8, 4i8, 4i8, 4i8]",
+                             [("i64", 0), ("i32", 1), ("i8", 1)])                    # tests/hist/and8.fut:24-27
+    assert n == 5 and is_.tolist() == [1, 2, 1, 4, 5] and img.tolist() == [1, 1, 4, 4, 4]
+    (h,) = _read_text(tmp_path, "[1f16, f16.nan, 3f16, 4f16, 5f16]", [("f16", 1)])    # tests/hist/f16.fut:32
+    assert np.isnan(h[1]) and h[[0, 2, 3, 4]].tolist() == [1, 3, 4, 5]
+    a, b = _read_text(tmp_path, "empty([0][1]i32) [[1]]", [("i32", 2), ("i32", 2)])   # tests/concat2.fut:10
+    assert a.shape == (0, 1) and b.tolist() == [[1]]
+    m, xss = _read_text(tmp_path, "10i64 [[1,2,3],[2,3,4],[3,4,5]]", [("i64", 0), ("i32", 2)])
+    assert m == 10 and xss.tolist() == [[1, 2, 3], [2, 3, 4], [3, 4, 5]]              # tests/hist/segmented.fut:2
+
+
+def test_text_reader_syntax(tmp_path):
+    out = _read_text(tmp_path, """-- a comment line
+        [[1, 2, 3], [4_000, 0x10, -6i32]]  -- trailing comment
+        4.5f64 [true, false] [] [[],[]] [1.5, 2,] 017 -0x1F 18446744073709551615u64 255u8 -1u8
+        [-f32.inf, f32.inf, f32.nan, 1e-3, -2.5e2f32] 1_0.5f64""",
+                     [("i32", 2), ("f64", 0), ("bool", 1), ("u8", 1), ("i64", 2), ("f32", 1),
+                      ("i32", 0), ("i16", 0), ("u64", 0), ("u8", 0), ("u8", 0), ("f32", 1), ("f64", 0)])
+    assert out[0].tolist() == [[1, 2, 3], [4000, 16, -6]]
+    assert out[1] == 4.5 and out[2].tolist() == [True, False]
+    assert out[3].shape == (0,) and out[4].shape == (2, 0) and out[5].tolist() == [1.5, 2.0]
+    assert out[6] == 15 and out[7] == -31 and out[8] == 2**64 - 1 and out[9] == 255 and out[10] == 255
+    f = out[11]
+    assert f[0] == -np.inf and f[1] == np.inf and np.isnan(f[2])
+    assert f[3] == np.float32(1e-3) and f[4] == -250 and out[12] == 10.5
+    for bad, spec in [("[[1, 2], [3]]", ("i32", 2)),           # rows of different length
+                      ("[1, 2", ("i32", 1)), ("[1 2]", ("i32", 1)), ("[1, x]", ("i32", 1)),
+                      ("[1i64]", ("i32", 1)), ("[[1]]", ("i32", 1)), ("[1]", ("i32", 2)),
+                      ("empty([1]i32)", ("i32", 1)), ("empty([0]i64)", ("i32", 1)),
+                      ("empty([0]i32)", ("i32", 2)), ("1.5", ("i32", 0)), ("yes", ("bool", 0)),
+                      ("0x10u64", ("u64", 0)), ("", ("i32", 0)), ("f64.nan", ("f32", 0))]:
+        with pytest.raises(fv.ValueError_):
+            _read_text(tmp_path, bad, [spec], expect_eof=False)
+    with pytest.raises(fv.ValueError_, match="end of input"):
+        _read_text(tmp_path, "1 2", [("i32", 0)])
+
+
+def test_f16_literals_are_cut_not_rounded(tmp_path):
+    """float2halfbits (rts/c/half.h:220-228) drops the low mantissa bits: 1.2 reads as
+    0x3ccc where rounding to nearest gives 0x3ccd; values that are f16 numbers read exactly."""
+    (h,) = _read_text(tmp_path, "[1.2f16, 0.1f16, 65504f16, 1e5f16, 1e-8f16, 6e-8, -0.5]", [("f16", 1)])
+    assert [hex(x) for x in h.view(np.uint16)] == ["0x3ccc", "0x2e66", "0x7bff", "0x7c00", "0x0",
+                                                   "0x1", "0xb800"]
+    rng = np.random.default_rng(4)
+    f = rng.standard_normal(2000).astype(np.float32) * np.float32(10.0) ** rng.integers(-6, 5, 2000)
+    (h,) = _read_text(tmp_path, "[" + ", ".join(f"{x:.9g}" for x in f) + "]", [("f16", 1)])
+    with np.errstate(over="ignore"):
+        rn = f.astype(np.float16)                     # round to nearest
+    toward_zero = np.where(np.abs(rn.astype(np.float32)) > np.abs(f),
+                           np.nextafter(rn, np.float16(0)), rn)
+    assert np.array_equal(h.view(np.uint16), toward_zero.view(np.uint16))
+
+
+@pytest.mark.parametrize("name", sorted(fv._DTYPES))
+def test_text_round_trip_of_every_type_and_rank(tmp_path, name):
+    rng = np.random.default_rng(8)
+    dt = np.dtype(fv._DTYPES[name])
+    for shape in [(), (7,), (3, 4), (2, 3, 2), (0,), (0, 3), (2, 0, 5)]:
+        n = int(np.prod(shape, dtype=np.int64))
+        if name == "bool":
+            a = rng.integers(0, 2, n).astype(np.bool_)
+        elif name[0] == "f":
+            a = (rng.standard_normal(n) * 1000).astype(dt)
+            if n > 2:
+                a[0], a[1], a[2] = np.nan, np.inf, -np.inf
+        else:
+            ii = np.iinfo(dt)
+            a = rng.integers(ii.min, ii.max, n, dtype=dt, endpoint=True)
+        a = a.reshape(shape)
+        p = tmp_path / "v.txt"
+        fv.write_text(p, [a])
+        (back,) = fv.read_text(p, [(name, len(shape))])
+        assert back.shape == a.shape and back.dtype == a.dtype
+        assert np.array_equal(back.view(np.uint8 if dt.itemsize == 1 else f"u{dt.itemsize}"),
+                              a.view(np.uint8 if dt.itemsize == 1 else f"u{dt.itemsize}")) or \
+            (name[0] == "f" and np.array_equal(back, a, equal_nan=True))
+        (either,) = fv.read_values(p, [(name, len(shape))])    # the detecting reader takes text ...
+        assert np.array_equal(either, back, equal_nan=name[0] == "f")
+        fv.write_binary(p, [a])
+        (either,) = fv.read_values(p, [(name, len(shape))])    # ... and binary
+        assert np.array_equal(either, a, equal_nan=name[0] == "f")
