@@ -150,6 +150,9 @@ constexpr size_t RS_LDS_FIXED = RS_WAVES * RS_RADIX * 4 + 2 * RS_RADIX * 4 + 64;
 // eight ballots; per-wave digit counters in LDS chain the 16 rounds; the tile
 // is then reordered in LDS so that the global stores of a wave are contiguous
 // runs per digit.  Order is preserved at every level (round, lane, wave, tile).
+// The stores stay ordinary ones: the runs are shorter than a cache line, and
+// non-temporal stores, which help every streaming kernel here, cost 35 % (L2
+// no longer merges the pieces of a line).
 template <class K, int VB, class DigitFn>
 __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
     const K *__restrict__ kin, K *__restrict__ kout, const void *__restrict__ vin_,
