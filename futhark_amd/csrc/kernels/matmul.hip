@@ -526,7 +526,7 @@ __global__ __launch_bounds__(256) void mm_pad_kernel(const T *__restrict__ src, 
   T *d = dst + (b * rows_p + r) * cols_p;
   const bool row_in = r < rows;
   for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols_p; c += (int64_t)gridDim.x * 256)
-    d[c] = (row_in && c < cols) ? s[c] : T(0);
+    __builtin_nontemporal_store((row_in && c < cols) ? s[c] : T(0), &d[c]);
 }
 
 __global__ __launch_bounds__(256) void mm_unpad_kernel(const float *__restrict__ src,
@@ -537,7 +537,7 @@ __global__ __launch_bounds__(256) void mm_unpad_kernel(const float *__restrict__
   const float *s = src + (b * rows_p + r) * cols_p;
   float *d = dst + (b * rows + r) * cols;
   for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += (int64_t)gridDim.x * 256)
-    d[c] = s[c];
+    __builtin_nontemporal_store(s[c], &d[c]);
 }
 
 struct MmPlan {
