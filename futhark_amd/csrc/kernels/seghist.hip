@@ -211,6 +211,13 @@ template <class T> __device__ __forceinline__ bool bits_equal(T a, T b) {
   else return bit_cast<uint64_t>(a) == bit_cast<uint64_t>(b);
 }
 
+// The inputs are read once: non-temporal loads (H = 256, 2^27 elements: 186 ->
+// 168 us; no change where several blocks share a chunk through L2).
+__device__ __forceinline__ uint4 hist_load_nt(const uint4 *p) {
+  using V4 = __attribute__((ext_vector_type(4))) uint32_t;
+  return bit_cast<uint4>(__builtin_nontemporal_load(reinterpret_cast<const V4 *>(p)));
+}
+
 // Four consecutive elements with the widest loads that fit (src is aligned to
 // 4 * sizeof(E) bytes).
 template <class E> __device__ __forceinline__ void load_elems4(E (&dst)[4], const E *src) {
@@ -224,7 +231,7 @@ template <class E> __device__ __forceinline__ void load_elems4(E (&dst)[4], cons
     constexpr int NV = (int)(4 * sizeof(E) / 16);
     uint4 raw[NV];
 #pragma unroll
-    for (int q = 0; q < NV; q++) raw[q] = reinterpret_cast<const uint4 *>(src)[q];
+    for (int q = 0; q < NV; q++) raw[q] = hist_load_nt(reinterpret_cast<const uint4 *>(src) + q);
     __builtin_memcpy(dst, raw, sizeof(raw));
   }
 }

@@ -98,14 +98,14 @@ __global__ __launch_bounds__(SEGRED_BLOCK) void segred_nonseg_kernel(
   for (; i + (SEGRED_UNROLL - 1) * stride < nvec; i += SEGRED_UNROLL * stride) {
     Vec16<T> v[SEGRED_UNROLL];
 #pragma unroll
-    for (int u = 0; u < SEGRED_UNROLL; u++) v[u] = load_vec16(xs + (i + u * stride) * VEC);
+    for (int u = 0; u < SEGRED_UNROLL; u++) v[u] = load_vec16_nt(xs + (i + u * stride) * VEC);
 #pragma unroll
     for (int u = 0; u < SEGRED_UNROLL; u++)
 #pragma unroll
       for (int e = 0; e < VEC; e++) acc[e] = Op::apply(acc[e], v[u].e[e]);
   }
   for (; i < nvec; i += stride) {
-    Vec16<T> v = load_vec16(xs + i * VEC);
+    Vec16<T> v = load_vec16_nt(xs + i * VEC);
 #pragma unroll
     for (int e = 0; e < VEC; e++) acc[e] = Op::apply(acc[e], v.e[e]);
   }
