@@ -40,6 +40,7 @@ def make_workload(name: str, ctx):
     if name.startswith("segscan_") or name.startswith("segred_"):
         kind, op, t, sz = name.split("_")
         n = 1 << int(sz[2:])
+        w["elements"] = n
         es = 4 if t == "f32" else 8
         offsets, lens, flags = dg.segments(32, n, 1024)
         xs = dg.uniform_f32(33, n) if t == "f32" else dg.uniform_int(34, n, -(1 << 20), 1 << 20, np.int64)
@@ -66,6 +67,7 @@ def make_workload(name: str, ctx):
     elif name.startswith("reduce_") or name.startswith("scan_"):
         kind, op, t, sz = name.split("_")
         n = 1 << int(sz[2:])
+        w["elements"] = n
         es = 4
         xs = dg.uniform_f32(17, n) if t == "f32" else dg.uniform_int(16, n, -1000, 1000)
         a = ctx.new(f"{t}_1d", xs)
@@ -89,6 +91,7 @@ def make_workload(name: str, ctx):
         # hist_add_i32_H65536_uniform_2p27
         _, op, t, hs, dist, sz = name.split("_")
         n, H = 1 << int(sz[2:]), int(hs[1:])
+        w["elements"] = n
         is_ = dg.hist_indices(48, n, H, dist)
         if t == "f16":
             vs, es = dg.to_f16_bits(dg.uniform_f32(50, n)), 2
@@ -113,6 +116,7 @@ def make_workload(name: str, ctx):
         # sort_u32_2p26 | sort_u64i32_2p26
         _, kt, sz = name.split("_")
         n = 1 << int(sz[2:])
+        w["elements"] = n
         if kt == "u32":
             k = ctx.new("u32_1d", dg.uniform_u32(80, n))
 
@@ -146,10 +150,26 @@ def make_workload(name: str, ctx):
             ctx.call(f"bmm_{t}", ["f32_3d"], a, bb).free()
         w.update(step=step, flops=2 * b * m * m * m, kernel="segmap_matmul", dtype=t, bound="mfma",
                  keep=[a, bb], describe=f"batched matmul b={b} M=N=K={m}, {t} in, f32 accumulate")
+    elif name.startswith("segreduce_"):
+        # segreduce_add_f32_65536x1024: regular segments, map (reduce op ne) xss
+        _, op, t, shape = name.split("_")
+        m, k = (int(x) for x in shape.split("x"))
+        w["elements"] = m * k
+        dt = {"f32": np.float32, "i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        xss = (dg.uniform_f32(36, m * k) if t[0] == "f" else dg.uniform_int(37, m * k, -1000, 1000)
+               ).astype(dt).reshape(m, k)
+        a = ctx.new(f"{t}_2d", xss)
+
+        def step():
+            ctx.call(f"segreduce_{op}_{t}", [f"{t}_1d"], a).free()
+        w.update(step=step, bytes=m * k * dt().itemsize + m * dt().itemsize, kernel="segred_regular",
+                 dtype=t, bound="hbm", keep=[a],
+                 describe=f"regular segmented reduce ({op}) of [{m}][{k}]{t}")
     elif name.startswith("transpose_"):
         # transpose_f32_8192x8192
         _, t, shape = name.split("_")
         rows, cols = (int(x) for x in shape.split("x"))
+        w["elements"] = rows * cols
         x = ctx.new("f32_2d", dg.uniform_f32(90, rows * cols).reshape(rows, cols))
 
         def step():
@@ -324,7 +344,9 @@ def main() -> None:
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
         "config": {"workload": w["describe"], "name": args.workload,
-                   "algorithmic_bytes_per_step" if w["bound"] == "hbm" else "flop_per_step": work},
+                   "algorithmic_bytes_per_step" if w["bound"] == "hbm" else "flop_per_step": work,
+                   **({"elements_per_s": round(w["elements"] / (ms_per_step * 1e-3), 1)}
+                      if "elements" in w else {})},
         "roofline": {"bound": w["bound"], "achieved": round(achieved, 3), "peak": peak,
                      "unit": unit, "frac": round(achieved / peak, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
