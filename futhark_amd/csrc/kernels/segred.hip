@@ -5,9 +5,11 @@
 // thread t folds elements t, t+T, t+2T, ... (SegRed.hs:802-832), per-block
 // partials, and a stage two run by one block of the same launch
 // (SegRed.hs:923-1047 picks the block that arrives last with an atomic counter;
-// here the block that starts last waits for the others).  The schedule is new:
-// 128-bit loads, four loads in flight per thread, a wave64 DPP reduction and a
-// single LDS exchange per block.
+// here the block that starts last waits for the others); short rows are folded
+// by groups of lanes (SegRed.hs:396-505), long rows by whole blocks, a few very
+// long rows by several blocks each (SegRed.hs:507-636).  The schedule is new:
+// 128-bit non-temporal loads, four loads in flight per thread, wave64 DPP
+// reductions and a single LDS exchange per block.
 #include "common.hip.h"
 
 namespace fa {
@@ -172,13 +174,68 @@ __global__ __launch_bounds__(256) void segred_small_kernel(const T *__restrict__
   if (seg < m && sub == 0) out[seg] = acc;
 }
 
-// k large: one block per segment (grid-stride over segments).
+// The same with 128-bit loads, for rows that are whole vectors (k a multiple of
+// VEC, 16-byte aligned base): lane `sub` of a group folds vectors sub, sub + G,
+// ... of its row, four loads in flight.  G = 1 is a row per lane.
+template <class T, class Op, int G>
+__global__ __launch_bounds__(256) void segred_small_vec_kernel(const T *__restrict__ xss, int64_t m,
+                                                               int64_t k, T *__restrict__ out) {
+  constexpr int VEC = Vec16<T>::N;
+  const int64_t gthread = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t seg = gthread / G;
+  const int sub = (int)(gthread % G);
+  T acc[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; e++) acc[e] = Op::identity();
+  if (seg < m) {
+    const T *row = xss + seg * k;
+    const int64_t kv = k / VEC;
+    int64_t j = sub;
+    for (; j + 3 * G < kv; j += 4 * G) {
+      Vec16<T> v[4];
+#pragma unroll
+      for (int u = 0; u < 4; u++) v[u] = load_vec16_nt(row + (j + u * G) * VEC);
+#pragma unroll
+      for (int u = 0; u < 4; u++)
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = Op::apply(acc[e], v[u].e[e]);
+    }
+    for (; j < kv; j += G) {
+      const Vec16<T> v = load_vec16_nt(row + j * VEC);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) acc[e] = Op::apply(acc[e], v.e[e]);
+    }
+  }
+  T a = acc[0];
+#pragma unroll
+  for (int e = 1; e < VEC; e++) a = Op::apply(a, acc[e]);
+#pragma unroll
+  for (int d = G / 2; d >= 1; d /= 2) {
+    T other;
+    if constexpr (sizeof(T) == 4) {
+      other = bit_cast<T>(__shfl_down(bit_cast<int>(a), d, WAVE));
+    } else {
+      other = bit_cast<T>((unsigned long long)__shfl_down(
+          (unsigned long long)bit_cast<uint64_t>(a), d, WAVE));
+    }
+    a = Op::apply(a, other);
+  }
+  if (seg < m && sub == 0) out[seg] = a;
+}
+
+// k large: one block per segment (grid-stride over segments).  With `pieces`
+// > 1 every row is cut into that many pieces of `piece_len` elements (the last
+// one shorter) and out[seg * pieces + p] receives the fold of piece p: the
+// first of two stages for a few very long rows.
 template <class T, class Op>
 __global__ __launch_bounds__(1024) void segred_large_kernel(const T *__restrict__ xss, int64_t m,
-                                                            int64_t k, T *__restrict__ out) {
+                                                            int64_t row_len, T *__restrict__ out,
+                                                            int64_t pieces, int64_t piece_len) {
   __shared__ T lds[1024 / WAVE];
-  for (int64_t seg = blockIdx.x; seg < m; seg += gridDim.x) {
-    const T *row = xss + seg * k;
+  for (int64_t seg = blockIdx.x; seg < m * pieces; seg += gridDim.x) {
+    const int64_t first = (seg % pieces) * piece_len;
+    const int64_t k = row_len - first < piece_len ? row_len - first : piece_len;
+    const T *row = xss + (seg / pieces) * row_len + first;
     T acc0 = Op::identity(), acc1 = Op::identity(), acc2 = Op::identity(),
       acc3 = Op::identity();
     int64_t j = threadIdx.x;
@@ -212,30 +269,66 @@ static int launch_nonseg(hipStream_t s, const void *xs, int64_t n, void *out, vo
   return launch_status();
 }
 
+// Rows longer than this are folded by whole blocks.
+constexpr int64_t SEGRED_LARGE_K = 8192;
+
+// How many pieces a row is cut into so that a few long rows still fill the
+// chip (the reference's large-segments case spreads a segment over several
+// blocks too, SegRed.hs:507-636).
+static int64_t segred_pieces(int64_t m, int64_t k) {
+  const int64_t blocks_wanted = (int64_t)segred_grid_limit() * 4;
+  if (k <= SEGRED_LARGE_K || m >= blocks_wanted) return 1;
+  const int64_t by_fill = ceil_div(blocks_wanted, m);
+  const int64_t by_size = ceil_div(k, 2 * SEGRED_LARGE_K);  // pieces stay at least this long
+  const int64_t p = by_fill < by_size ? by_fill : by_size;
+  return p < 1 ? 1 : p;
+}
+
 template <class T, class Op>
-static int launch_regular(hipStream_t s, const void *xss, int64_t m, int64_t k, void *out) {
-  if (m == 0) return 0;
-  const T *in = (const T *)xss;
-  T *o = (T *)out;
-#define FA_SMALL(G)                                                                          \
+static int launch_small(hipStream_t s, const T *in, int64_t m, int64_t k, T *o) {
+  constexpr int VEC = Vec16<T>::N;
+  const bool vec = k % VEC == 0 && is_aligned(in, 16);
+  const int64_t units = vec ? k / VEC : k;  // what one lane takes per step
+#define FA_SMALL(KERNEL, G)                                                                  \
   do {                                                                                       \
     int64_t threads = m * (G);                                                               \
     int64_t grid = ceil_div(threads, 256);                                                   \
     if (grid > INT32_MAX) return FA_EINVAL;                                                  \
-    hipLaunchKernelGGL((segred_small_kernel<T, Op, G>), dim3((unsigned)grid), dim3(256), 0, \
-                       s, in, m, k, o);                                                      \
+    hipLaunchKernelGGL((KERNEL<T, Op, G>), dim3((unsigned)grid), dim3(256), 0, s, in, m, k, o); \
   } while (0)
-  if (k <= 2) FA_SMALL(1);
-  else if (k <= 8) FA_SMALL(4);
-  else if (k <= 64) FA_SMALL(16);
-  else if (k <= 8192) FA_SMALL(64);
-  else {
-    int64_t grid = m < 65536 ? m : 65536;
-    hipLaunchKernelGGL((segred_large_kernel<T, Op>), dim3((unsigned)grid), dim3(1024), 0, s, in,
-                       m, k, o);
-  }
+#define FA_SMALL_BY_UNITS(KERNEL)            \
+  do {                                       \
+    if (units <= 2) FA_SMALL(KERNEL, 1);     \
+    else if (units <= 8) FA_SMALL(KERNEL, 4);   \
+    else if (units <= 64) FA_SMALL(KERNEL, 16); \
+    else FA_SMALL(KERNEL, 64);               \
+  } while (0)
+  if (vec) FA_SMALL_BY_UNITS(segred_small_vec_kernel);
+  else FA_SMALL_BY_UNITS(segred_small_kernel);
+#undef FA_SMALL_BY_UNITS
 #undef FA_SMALL
   return launch_status();
+}
+
+template <class T, class Op>
+static int launch_regular(hipStream_t s, const void *xss, int64_t m, int64_t k, void *out,
+                          void *workspace, size_t workspace_bytes) {
+  if (m == 0) return 0;
+  const T *in = (const T *)xss;
+  T *o = (T *)out;
+  if (k <= SEGRED_LARGE_K) return launch_small<T, Op>(s, in, m, k, o);
+  int64_t pieces = segred_pieces(m, k);
+  if (pieces > 1 && (workspace == nullptr || workspace_bytes < (size_t)(m * pieces) * sizeof(T) ||
+                     !is_aligned(workspace, 16)))
+    pieces = 1;
+  const int64_t piece_len = pieces == 1 ? k : ceil_div(ceil_div(k, pieces), (int64_t)4096) * 4096;
+  const int64_t blocks = m * pieces;
+  const int64_t grid = blocks < 65536 ? blocks : 65536;
+  hipLaunchKernelGGL((segred_large_kernel<T, Op>), dim3((unsigned)grid), dim3(1024), 0, s, in, m, k,
+                     pieces == 1 ? o : (T *)workspace, pieces, piece_len);
+  const int rc = launch_status();
+  if (rc != 0 || pieces == 1) return rc;
+  return launch_small<T, Op>(s, (const T *)workspace, m, pieces, o);
 }
 
 }  // namespace fa
@@ -257,10 +350,23 @@ extern "C" int fa_segred_nonseg(fa_stream_t stream, fa_dtype t, fa_op op, const 
   FA_DISPATCH_TYPE_OP(launch_nonseg, t, op, s, xs, n, out, scratch, scratch_bytes, epoch);
 }
 
-extern "C" int fa_segred_regular(fa_stream_t stream, fa_dtype t, fa_op op, const void *xss,
-                                 int64_t m, int64_t k, void *out) {
+extern "C" size_t fa_segred_regular_workspace_bytes(fa_dtype t, int64_t m, int64_t k) {
+  if (m <= 0 || k <= 0) return 0;
+  const int64_t pieces = segred_pieces(m, k);
+  const size_t es = (t == FA_I64 || t == FA_U64 || t == FA_F64) ? 8 : 4;
+  return pieces > 1 ? (size_t)(m * pieces) * es : 0;
+}
+
+extern "C" int fa_segred_regular_ws(fa_stream_t stream, fa_dtype t, fa_op op, const void *xss,
+                                    int64_t m, int64_t k, void *out, void *workspace,
+                                    size_t workspace_bytes) {
   if (m < 0 || k < 0 || (m > 0 && out == nullptr) || (m * k > 0 && xss == nullptr))
     return FA_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  FA_DISPATCH_TYPE_OP(launch_regular, t, op, s, xss, m, k, out);
+  FA_DISPATCH_TYPE_OP(launch_regular, t, op, s, xss, m, k, out, workspace, workspace_bytes);
+}
+
+extern "C" int fa_segred_regular(fa_stream_t stream, fa_dtype t, fa_op op, const void *xss,
+                                 int64_t m, int64_t k, void *out) {
+  return fa_segred_regular_ws(stream, t, op, xss, m, k, out, nullptr, 0);
 }

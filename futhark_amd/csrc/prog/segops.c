@@ -304,11 +304,19 @@ static int do_segreduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_
   const int64_t m = in->shape[0], k = in->shape[1];
   struct fut_array *res = out_array(ctx, m * (int64_t)es, 1, &m, "segreduce.out");
   if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
-  struct rts_event *ev = rts_kernel_begin(
-      ctx, "segred_regular",
-      rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)k));
-  int code = fa_segred_regular(ctx->stream, t, op, in->mem.mem, m, k, res->mem.mem);
-  int err = rts_kernel_end(ctx, ev, "segred_regular", code);
+  struct memblock_device ws = {0};
+  const size_t ws_bytes = fa_segred_regular_workspace_bytes(t, m, k);
+  int err = 0;
+  if (ws_bytes > 0) err = rts_memblock_alloc(ctx, &ws, (int64_t)ws_bytes, "segreduce.workspace");
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "segred_regular",
+        rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)k));
+    int code = fa_segred_regular_ws(ctx->stream, t, op, in->mem.mem, m, k, res->mem.mem, ws.mem,
+                                    ws_bytes);
+    err = rts_kernel_end(ctx, ev, "segred_regular", code);
+  }
+  rts_memblock_unref(ctx, &ws, "segreduce.workspace");
   if (err != 0) {
     drop_array(ctx, res);
     return err;

@@ -86,6 +86,14 @@ int fa_segred_nonseg(fa_stream_t stream, fa_dtype t, fa_op op,
  * Replaces: segred_small / segred_large (SegRed.hs:396-636).  No scratch. */
 int fa_segred_regular(fa_stream_t stream, fa_dtype t, fa_op op,
                       const void *xss, int64_t m, int64_t k, void *out);
+/* The same with a workspace of fa_segred_regular_workspace_bytes() bytes
+ * (16-byte aligned; 0 bytes for most shapes): a few very long rows are then cut
+ * into pieces that fill the chip and folded in two stages, as the reference's
+ * large-segments case spreads a segment over several blocks (SegRed.hs:507-636). */
+size_t fa_segred_regular_workspace_bytes(fa_dtype t, int64_t m, int64_t k);
+int fa_segred_regular_ws(fa_stream_t stream, fa_dtype t, fa_op op,
+                         const void *xss, int64_t m, int64_t k, void *out,
+                         void *workspace, size_t workspace_bytes);
 
 /* ----------------------------------------------------------------- SegScan
  * Single-pass scan with decoupled look-back.

@@ -184,8 +184,12 @@ def test_segreduce_regular(ctx, goldens, t):
     c = goldens["segsum"]["cases"][0]
     out = ctx.call("segreduce_add_f32", ["f32_1d"], ctx.new("f32_2d", np.array(c["xss"], np.float32)))
     assert out.values().tolist() == c["out"]
+    # rows of whole 16-byte vectors and not, every group width, rows folded by whole blocks,
+    # a few very long rows (cut into pieces, two stages; 33000 leaves an empty last piece)
     for m, k in [(1, 1), (1000, 1), (1000, 2), (777, 7), (300, 33), (100, 64), (50, 1000),
-                 (7, 9001), (3, 70000), (0, 5), (5, 0)]:
+                 (7, 9001), (3, 70000), (0, 5), (5, 0), (4099, 4), (513, 8), (257, 12), (129, 36),
+                 (65, 256), (33, 260), (17, 1028), (9, 8192), (5, 8196), (2, 33000), (3, 1 << 20),
+                 (1, 3000001)]:
         xss = _data(t, m * k, 9).reshape(m, k)
         out = ctx.call(f"segreduce_add_{t}", [f"{t}_1d"], ctx.new(f"{t}_2d", xss))
         got = out.values()
