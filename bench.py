@@ -150,6 +150,20 @@ def make_workload(name: str, ctx):
             ctx.call(f"bmm_{t}", ["f32_3d"], a, bb).free()
         w.update(step=step, flops=2 * b * m * m * m, kernel="segmap_matmul", dtype=t, bound="mfma",
                  keep=[a, bb], describe=f"batched matmul b={b} M=N=K={m}, {t} in, f32 accumulate")
+    elif name.startswith("scanrows_"):
+        # scanrows_add_f32_65536x1024: map (scan op ne) xss
+        _, op, t, shape = name.split("_")
+        m, k = (int(x) for x in shape.split("x"))
+        w["elements"] = m * k
+        dt = {"f32": np.float32, "i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        xss = (dg.uniform_f32(38, m * k) if t[0] == "f" else dg.uniform_int(39, m * k, -1000, 1000)
+               ).astype(dt).reshape(m, k)
+        a = ctx.new(f"{t}_2d", xss)
+
+        def step():
+            ctx.call(f"scanrows_{op}_{t}", [f"{t}_2d"], a).free()
+        w.update(step=step, bytes=2 * m * k * dt().itemsize, kernel="segscan_rows", dtype=t,
+                 bound="hbm", keep=[a], describe=f"scan ({op}) of every row of [{m}][{k}]{t}")
     elif name.startswith("segreduce_"):
         # segreduce_add_f32_65536x1024: regular segments, map (reduce op ne) xss
         _, op, t, shape = name.split("_")

@@ -114,6 +114,7 @@ class Segops:
                 getattr(L, f"futhark_entry_segred_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
                 getattr(L, f"futhark_entry_segreduce_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_seghist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
+                getattr(L, f"futhark_entry_scanrows_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
                 getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
         for t in HIST_ONLY_TYPES:

@@ -102,11 +102,34 @@ __device__ __forceinline__ bool desc_read(const uint64_t *desc, int64_t tile, ui
   return true;
 }
 
-// out[n]; flags optional (SEG); EXCL selects the exclusive form.
-template <class T, class Op, bool SEG, bool EXCL>
+// Segment starts among the VEC elements that begin at position `pos` of a row
+// of `seg_len` elements: bit e is set when element e opens a row.
+template <int VEC>
+__device__ __forceinline__ uint32_t regular_start_mask(int64_t pos, int64_t seg_len) {
+  uint32_t m = 0u;
+#pragma unroll
+  for (int e = 0; e < VEC; e++) {
+    if (pos == 0) m |= 1u << e;
+    pos++;
+    if (pos == seg_len) pos = 0;
+  }
+  return m;
+}
+
+// Where segments come from: nowhere, a flag byte per element, or rows of equal
+// length (`map (scan op ne) xss`: SegScan with segment dimensions,
+// SegScan/SinglePass.hs:327-361 -- the reference tests whether two positions
+// lie in the same row; here the row starts are computed from the element
+// index, so there is no flag array to read).
+enum { SEG_NONE = 0, SEG_FLAGS = 1, SEG_ROWS = 2 };
+
+// out[n]; EXCL selects the exclusive form.
+template <class T, class Op, int SEGKIND, bool EXCL>
 __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
     const T *__restrict__ xs, const uint8_t *__restrict__ flags, int64_t n, T *__restrict__ out,
-    uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles) {
+    uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles, int64_t seg_len) {
+  constexpr bool SEG = SEGKIND != SEG_NONE;
+  constexpr bool FLAGS = SEGKIND == SEG_FLAGS;
   constexpr int VEC = Vec16<T>::N;
   constexpr int SCAN_ROWS = scan_rows<T>();
   constexpr int WCHUNK = SCAN_ROWS * WAVE * VEC;
@@ -119,7 +142,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   __shared__ T s_pv;
   __shared__ uint32_t s_pf;
   // Flag bytes of the tile, one contiguous chunk per wave (segmented scans).
-  __shared__ __align__(16) uint32_t s_flags[SEG ? TILE / 4 : 4];
+  __shared__ __align__(16) uint32_t s_flags[FLAGS ? TILE / 4 : 4];
 
   if (threadIdx.x == 0) {
     const uint32_t t = atomicAdd(ticket, 1u);
@@ -139,7 +162,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   //      fetched with 16 bytes per lane (a few wide loads instead of one narrow
   //      load per row) and handed to the lanes that own them through LDS.
   bool flags_staged = false;
-  if constexpr (SEG) {
+  if constexpr (FLAGS) {
     constexpr int FB = WCHUNK / WAVE;  // flag bytes per lane
     static_assert(FB == 8 || FB % 16 == 0, "flag bytes per lane: one 8-byte or whole 16-byte loads");
     flags_staged = wbase + WCHUNK <= n && ((uintptr_t)flags & 15u) == 0;
@@ -171,7 +194,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
       Vec16<T> v = FA_SCAN_LOAD(xs + idx);
 #pragma unroll
       for (int e = 0; e < VEC; e++) x[r][e] = v.e[e];
-      if constexpr (SEG) {
+      if constexpr (FLAGS) {
         if (!flags_staged) {
           if constexpr (VEC == 4) {
             const uint32_t w = FA_SCAN_FLAG_LOAD(reinterpret_cast<const uint32_t *>(flags + idx));
@@ -189,13 +212,13 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
       for (int e = 0; e < VEC; e++) {
         const bool in = idx + e < n;
         x[r][e] = in ? xs[idx + e] : Op::identity();
-        if constexpr (SEG) {
+        if constexpr (FLAGS) {
           if (in && flags[idx + e] != 0) fm[r] |= 1u << e;
         }
       }
     }
   }
-  if constexpr (SEG) {
+  if constexpr (FLAGS) {
     if (flags_staged) {
       // Same wave wrote the chunk: LDS operations of a wave complete in order.
       __builtin_amdgcn_wave_barrier();
@@ -207,6 +230,23 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
         else w = *reinterpret_cast<const uint16_t *>(wf + (r * WAVE + lane) * 2);
 #pragma unroll
         for (int e = 0; e < VEC; e++) fm[r] |= ((w >> (8 * e)) & 0xffu) ? (1u << e) : 0u;
+      }
+    }
+  }
+
+  // Rows of equal length: the start masks come from the position of this
+  // lane's first element inside its row, kept up from one 16-byte row of the
+  // wave to the next (one division per thread), while the loads are in flight.
+  if constexpr (SEGKIND == SEG_ROWS) {
+    int64_t row_pos = (wbase + (int64_t)lane * VEC) % seg_len;
+#pragma unroll
+    for (int r = 0; r < SCAN_ROWS; r++) {
+      fm[r] = regular_start_mask<VEC>(row_pos, seg_len);
+      if (seg_len > WAVE * VEC) {
+        row_pos += WAVE * VEC;
+        if (row_pos >= seg_len) row_pos -= seg_len;
+      } else {
+        row_pos = (int64_t)((uint32_t)(row_pos + WAVE * VEC) % (uint32_t)seg_len);
       }
     }
   }
@@ -387,8 +427,8 @@ template <class T> static int64_t scan_num_tiles(int64_t n) {
 }
 
 template <class T, class Op>
-static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int64_t n,
-                       int exclusive, void *out, void *scratch, size_t scratch_bytes,
+static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int64_t seg_len,
+                       int64_t n, int exclusive, void *out, void *scratch, size_t scratch_bytes,
                        uint32_t epoch) {
   if (n == 0) return 0;
   const int64_t tiles = scan_num_tiles<T>(n);
@@ -402,13 +442,16 @@ static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int6
   const dim3 grid((unsigned)tiles), block(SCAN_BLOCK);
 #define FA_LAUNCH(SEGV, EXV)                                                              \
   hipLaunchKernelGGL((segscan_kernel<T, Op, SEGV, EXV>), grid, block, 0, s, (const T *)xs, \
-                     flags, n, (T *)out, ticket, desc, epoch, tiles)
-  if (flags) {
-    if (exclusive) FA_LAUNCH(true, true);
-    else FA_LAUNCH(true, false);
+                     flags, n, (T *)out, ticket, desc, epoch, tiles, seg_len)
+  if (seg_len > 0) {
+    if (exclusive) FA_LAUNCH(SEG_ROWS, true);
+    else FA_LAUNCH(SEG_ROWS, false);
+  } else if (flags) {
+    if (exclusive) FA_LAUNCH(SEG_FLAGS, true);
+    else FA_LAUNCH(SEG_FLAGS, false);
   } else {
-    if (exclusive) FA_LAUNCH(false, true);
-    else FA_LAUNCH(false, false);
+    if (exclusive) FA_LAUNCH(SEG_NONE, true);
+    else FA_LAUNCH(SEG_NONE, false);
   }
 #undef FA_LAUNCH
   return launch_status();
@@ -432,6 +475,19 @@ extern "C" int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op, const void *
     return FA_EINVAL;
   if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
   hipStream_t s = (hipStream_t)stream;
-  FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xs, flags, n, exclusive, out, scratch,
+  FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xs, flags, (int64_t)0, n, exclusive, out, scratch,
                       scratch_bytes, epoch);
+}
+
+extern "C" int fa_segscan_rows(fa_stream_t stream, fa_dtype t, fa_op op, const void *xss,
+                               int64_t m, int64_t k, int exclusive, void *out, void *scratch,
+                               size_t scratch_bytes, uint32_t epoch) {
+  if (m < 0 || k < 0 || (m > 0 && k > INT64_MAX / m)) return FA_EINVAL;
+  const int64_t n = m * k;
+  if (n > 0 && (xss == nullptr || out == nullptr || scratch == nullptr)) return FA_EINVAL;
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
+  if (n == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xss, (const uint8_t *)nullptr, k, n, exclusive, out,
+                      scratch, scratch_bytes, epoch);
 }

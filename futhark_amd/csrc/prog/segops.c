@@ -325,6 +325,31 @@ static int do_segreduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_
   return 0;
 }
 
+/* `map (scan op ne) xss`: the scan kernel with row starts in place of flags. */
+static int do_scanrows(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                       struct fut_array **out, const struct fut_array *in) {
+  const int64_t m = in->shape[0], k = in->shape[1];
+  uint32_t epoch = 0;
+  const size_t sbytes = fa_segscan_scratch_bytes(t, m * k);
+  void *scratch = rts_scan_scratch(ctx, sbytes, &epoch);
+  if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
+  const int64_t dims[2] = {m, k};
+  struct fut_array *res = out_array(ctx, m * k * (int64_t)es, 2, dims, "scanrows.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  struct rts_event *ev = rts_kernel_begin(
+      ctx, "segscan_rows",
+      rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)k));
+  int code = fa_segscan_rows(ctx->stream, t, op, in->mem.mem, m, k, 0, res->mem.mem, scratch,
+                             ctx->scan_scratch_bytes, epoch);
+  int err = rts_kernel_end(ctx, ev, "segscan_rows", code);
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
 /* Bit pattern of the neutral element: 0 for add, or, xor; all ones for and;
  * T.lowest / T.highest for max / min (prelude/math.fut: the smallest / largest
  * integer of the type, -inf / +inf for floats). */
@@ -491,6 +516,15 @@ static int do_seghist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t 
     ENTER(ctx);                                                                               \
     int ret =                                                                                 \
         do_segreduce(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a);   \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_scanrows_##OP##_##T(struct futhark_context *ctx,                          \
+                                        struct futhark_##T##_2d **out0,                       \
+                                        const struct futhark_##T##_2d *in0) {                 \
+    ENTER(ctx);                                                                               \
+    int ret =                                                                                 \
+        do_scanrows(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a);    \
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }                                                                                           \

@@ -118,6 +118,14 @@ int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op,
                const void *xs, const uint8_t *flags, int64_t n, int exclusive,
                void *out, void *scratch, size_t scratch_bytes, uint32_t epoch);
 
+/* The same over rows of equal length, `map (scan op ne) xss` with xss : [m][k]
+ * (SegScan with segment dimensions, SegScan/SinglePass.hs:327-361): the scan
+ * restarts at every multiple of k.  No flag array exists or is read.  Scratch
+ * and epoch as for fa_segscan with n = m * k. */
+int fa_segscan_rows(fa_stream_t stream, fa_dtype t, fa_op op,
+                    const void *xss, int64_t m, int64_t k, int exclusive,
+                    void *out, void *scratch, size_t scratch_bytes, uint32_t epoch);
+
 /* Irregular segmented reduction (Pass/Flatten/Builtins.hs:582-602):
  *   out[i] = lens[i] == 0 ? ne : segscan(flags-from-offsets, vs)[offsets[i]+lens[i]-1]
  * computed without materialising the scan.  Segments must be in order and

@@ -128,6 +128,16 @@ def hist(op: str, t: str, k: int, is_, vs, variant: str = "lit"):
     return rbi(op, t, np.full(k, NEUTRAL[(op, t)], dtype=dt), is_, vs, variant)
 
 
+def scanrows(op: str, t: str, xss, variant: str = "lit"):
+    """map (scan op ne) xss: every row scanned on its own."""
+    _, dt = _CT[t]
+    xss = _arr(xss, dt)
+    out = np.empty_like(xss)
+    for r in range(xss.shape[0]):
+        out[r] = scan(op, t, xss[r], variant)
+    return out
+
+
 def seghist(op: str, t: str, k: int, iss, vss, variant: str = "lit"):
     """map2 (hist op ne k) iss vss (tests/hist/segmented.fut): one histogram per row."""
     _, dt = _CT[t]
