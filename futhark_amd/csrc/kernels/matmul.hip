@@ -562,7 +562,9 @@ static MmPlan mm_plan(fa_dtype in_t, int64_t batch, int64_t M, int64_t N, int64_
   // padding does not multiply the work too much: the scalar kernel runs at a
   // few percent of the MFMA rate.
   const double work = (double)batch * M * N * K, padded_work = (double)batch * p.Mp * p.Np * p.Kp;
-  p.padded = work >= (double)(1 << 24) && padded_work <= 8.0 * work && p.Mp <= 65535 &&
+  fa_tuning tune;
+  fa_get_tuning(&tune);
+  p.padded = work >= (double)tune.matmul_pad_min_work && padded_work <= 8.0 * work && p.Mp <= 65535 &&
              batch <= 65535;
   p.a_bytes = mm_align((size_t)batch * p.Mp * p.Kp * es);
   p.b_bytes = mm_align((size_t)batch * p.Kp * p.Np * es);

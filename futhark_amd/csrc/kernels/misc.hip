@@ -112,3 +112,27 @@ extern "C" const char *fa_strerror(int code) {
     default: return "unknown error";
   }
 }
+
+// ------------------------------------------------------------------ tuning
+static fa_tuning g_tuning = {0, 0, 0};
+
+extern "C" void fa_set_tuning(const fa_tuning *t) {
+  if (t == nullptr) {
+    g_tuning = fa_tuning{0, 0, 0};
+    return;
+  }
+  g_tuning = *t;
+  if (g_tuning.segred_small_threshold < 0) g_tuning.segred_small_threshold = 0;
+  if (g_tuning.hist_lds_bins_max < 0) g_tuning.hist_lds_bins_max = 0;
+  if (g_tuning.matmul_pad_min_work < 0) g_tuning.matmul_pad_min_work = 0;
+}
+
+extern "C" void fa_get_tuning(fa_tuning *out) {
+  if (out == nullptr) return;
+  out->segred_small_threshold = g_tuning.segred_small_threshold > 0 ? g_tuning.segred_small_threshold : 8192;
+  int64_t bins = g_tuning.hist_lds_bins_max > 0 ? g_tuning.hist_lds_bins_max : 32768;
+  if (bins > 32768) bins = 32768;
+  if (bins < 64) bins = 64;
+  out->hist_lds_bins_max = bins;
+  out->matmul_pad_min_work = g_tuning.matmul_pad_min_work > 0 ? g_tuning.matmul_pad_min_work : (int64_t)1 << 24;
+}

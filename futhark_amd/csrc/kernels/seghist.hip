@@ -416,6 +416,15 @@ __global__ __launch_bounds__(256) void seghist_global_kernel(const I *__restrict
   }
 }
 
+// Most bins one LDS range holds for an accumulation type of `acc_bytes`
+// (fa_tuning.hist_lds_bins_max counts 4-byte bins).
+static int hist_range_bins_max(size_t acc_bytes) {
+  fa_tuning t;
+  fa_get_tuning(&t);
+  const int64_t bytes = t.hist_lds_bins_max * 4;
+  return (int)((bytes < HIST_LDS_BYTES ? bytes : HIST_LDS_BYTES) / (int64_t)acc_bytes);
+}
+
 static int hist_num_cus() {
   static int cus = 0;
   if (cus == 0) {
@@ -432,7 +441,7 @@ template <class T, class Op, class I, bool SEGMENTED = false>
 static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
                            int64_t H, int64_t seg_len = 0, int64_t H_seg = 0) {
   using A = typename HistAcc<T>::A;
-  const int max_range = HIST_LDS_BYTES / (int)sizeof(A);
+  const int max_range = hist_range_bins_max(sizeof(A));
   const int P = (int)ceil_div(H, max_range);
   const int range_bins = (int)ceil_div(H, P);
   int log2_copies = 0;
@@ -499,7 +508,7 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
   if (H == 0 || n == 0) return 0;
   if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
   const int64_t lds_limit =
-      (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)sizeof(typename HistAcc<T>::A));
+      (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
   if (H <= lds_limit) {
     if (is64) return launch_lds_hist<T, Op, int64_t>(st, (const int64_t *)is, (const T *)vs, n, (T *)dest, H);
     return launch_lds_hist<T, Op, int32_t>(st, (const int32_t *)is, (const T *)vs, n, (T *)dest, H);
@@ -543,7 +552,7 @@ static int launch_hist_segmented(hipStream_t st, const void *is, int is64, const
   if (H == 0 || n == 0) return 0;
   if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
   const int64_t lds_limit =
-      (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)sizeof(typename HistAcc<T>::A));
+      (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
   if (H <= lds_limit) {
     if (is64)
       return launch_lds_hist<T, Op, int64_t, true>(st, (const int64_t *)is, (const T *)vs, n,
@@ -576,7 +585,7 @@ extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int6
   if (es == 0) return 0;
   const size_t as = es < 4 ? 4 : es;  // size of the accumulation type
   if (n < 0) n = 0;
-  const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * (HIST_LDS_BYTES / (int64_t)as);
+  const int64_t lds_limit = (int64_t)HIST_MAX_RANGES * hist_range_bins_max(as);
   const int64_t part_limit = (int64_t)255 << (as == 4 ? 15 : 14);
   if (H <= lds_limit || H > part_limit) return 256;
   return hist_align(rs_scratch_bytes(rs_num_tiles(n))) +

@@ -269,17 +269,22 @@ static int launch_nonseg(hipStream_t s, const void *xs, int64_t n, void *out, vo
   return launch_status();
 }
 
-// Rows longer than this are folded by whole blocks.
-constexpr int64_t SEGRED_LARGE_K = 8192;
+// Rows longer than this are folded by whole blocks (fa_tuning).
+static int64_t segred_large_k() {
+  fa_tuning t;
+  fa_get_tuning(&t);
+  return t.segred_small_threshold;
+}
 
 // How many pieces a row is cut into so that a few long rows still fill the
 // chip (the reference's large-segments case spreads a segment over several
 // blocks too, SegRed.hs:507-636).
 static int64_t segred_pieces(int64_t m, int64_t k) {
   const int64_t blocks_wanted = (int64_t)segred_grid_limit() * 4;
-  if (k <= SEGRED_LARGE_K || m >= blocks_wanted) return 1;
+  const int64_t large_k = segred_large_k();
+  if (k <= large_k || m >= blocks_wanted) return 1;
   const int64_t by_fill = ceil_div(blocks_wanted, m);
-  const int64_t by_size = ceil_div(k, 2 * SEGRED_LARGE_K);  // pieces stay at least this long
+  const int64_t by_size = ceil_div(k, (int64_t)16384);  // pieces stay at least this long
   const int64_t p = by_fill < by_size ? by_fill : by_size;
   return p < 1 ? 1 : p;
 }
@@ -316,7 +321,7 @@ static int launch_regular(hipStream_t s, const void *xss, int64_t m, int64_t k, 
   if (m == 0) return 0;
   const T *in = (const T *)xss;
   T *o = (T *)out;
-  if (k <= SEGRED_LARGE_K) return launch_small<T, Op>(s, in, m, k, o);
+  if (k <= segred_large_k()) return launch_small<T, Op>(s, in, m, k, o);
   int64_t pieces = segred_pieces(m, k);
   if (pieces > 1 && (workspace == nullptr || workspace_bytes < (size_t)(m * pieces) * sizeof(T) ||
                      !is_aligned(workspace, 16)))

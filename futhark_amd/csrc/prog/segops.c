@@ -20,12 +20,22 @@
 static const char *const tuning_names[] = {
     "segops.hist_lds_bins_max",
     "segops.segred_small_threshold",
+    "segops.matmul_pad_min_work",
 };
-static const char *const tuning_classes[] = {"shared_memory", "threshold"};
-static const int64_t tuning_defaults[] = {0, 0};
+static const char *const tuning_classes[] = {"shared_memory", "threshold", "threshold"};
+static const int64_t tuning_defaults[] = {0, 0, 0}; /* 0: the kernel library's default */
+
+/* The parameters choose code paths inside the kernel library (fa_tuning). */
+static void apply_tuning(struct futhark_context *ctx) {
+  fa_tuning t;
+  t.hist_lds_bins_max = rts_tuning_param(ctx, tuning_names[0], 0);
+  t.segred_small_threshold = rts_tuning_param(ctx, tuning_names[1], 0);
+  t.matmul_pad_min_work = rts_tuning_param(ctx, tuning_names[2], 0);
+  fa_set_tuning(&t);
+}
 
 const struct rts_program futhark_program = {
-    "segops", 2, tuning_names, tuning_classes, tuning_defaults,
+    "segops", 3, tuning_names, tuning_classes, tuning_defaults, apply_tuning,
 };
 
 /* ------------------------------------------------------------------ arrays */

@@ -569,6 +569,7 @@ struct futhark_context *futhark_context_new(struct futhark_context_config *cfg) 
     (void)futhark_context_clear_caches(ctx);
     (void)futhark_context_sync(ctx);
   }
+  if (ctx->error == NULL && futhark_program.apply_tuning != NULL) futhark_program.apply_tuning(ctx);
   return ctx;
 }
 

@@ -84,12 +84,15 @@ struct tuning_param {
 };
 
 /* What a program tells the runtime about itself. */
+struct futhark_context;
 struct rts_program {
   const char *name;
   int num_tuning_params;
   const char *const *tuning_param_names;
   const char *const *tuning_param_classes;
   const int64_t *tuning_param_defaults;
+  /* called once a context is up: hands the tuning values to whoever uses them */
+  void (*apply_tuning)(struct futhark_context *ctx);
 };
 extern const struct rts_program futhark_program; /* defined by the program */
 

@@ -254,6 +254,7 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
 
 #define HIST_PARAM "segops.hist_lds_bins_max"
 #define SEGRED_PARAM "segops.segred_small_threshold"
+#define MATMUL_PARAM "segops.matmul_pad_min_work"
 #define SEGOP_ENTRY_ROWS(OP, T, CT)                                                             \
   {"reduce_" #OP "_" #T, e_reduce_##OP##_##T, #T, 0, 1, {"[]" #T}, {0}, {NULL}},                \
   {"scan_" #OP "_" #T, e_scan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {NULL}},               \
@@ -282,10 +283,10 @@ static const struct entry entries[] = {
     FUTHARK_FOR_EACH_INT_TYPE(SEGOP_BITOP_ROWS_FOR_TYPE)
     FUTHARK_FOR_EACH_HIST_ONLY_INT_TYPE(HIST_ONLY_INT_ROWS)
     FUTHARK_FOR_EACH_OP(HIST_ENTRY_ROWS, f16, uint16_t)
-    {"bmm_f32", e_bmm_f32, "[][][]f32", 1, 2, {"[][][]f32", "[][][]f32"}, {0}, {NULL}},
-    {"bmm_f16", e_bmm_f16, "[][][]f32", 1, 2, {"[][][]f16", "[][][]f16"}, {0}, {NULL}},
-    {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {NULL}},
-    {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {NULL}},
+    {"bmm_f32", e_bmm_f32, "[][][]f32", 1, 2, {"[][][]f32", "[][][]f32"}, {0}, {MATMUL_PARAM, NULL}},
+    {"bmm_f16", e_bmm_f16, "[][][]f32", 1, 2, {"[][][]f16", "[][][]f16"}, {0}, {MATMUL_PARAM, NULL}},
+    {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {MATMUL_PARAM, NULL}},
+    {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {MATMUL_PARAM, NULL}},
     {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {NULL}},
     {"radix_sort_u64", e_radix_sort_u64, "[]u64", 1, 1, {"[]u64"}, {0}, {NULL}},
     {"radix_sort_pairs_u32_i32", e_radix_sort_pairs_u32_i32, "([]u32, []i32)", 1, 2,

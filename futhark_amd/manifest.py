@@ -20,6 +20,7 @@ BACKEND = "hip"
 VERSION = "segops for gfx950, C API of Futhark 0.28.0"
 HIST_PARAM = "segops.hist_lds_bins_max"
 SEGRED_PARAM = "segops.segred_small_threshold"
+MATMUL_PARAM = "segops.matmul_pad_min_work"
 
 
 def _array_type_name(kind: str) -> str:
@@ -61,10 +62,10 @@ def entry_points() -> dict:
                 _entry(f"rbi_{op}_{t}", a, [("dest", "*" + a), ("is", "[]i32"), ("vs", a)], [HIST_PARAM]),
             ]
     eps += [
-        _entry("bmm_f32", "[][][]f32", [("A", "[][][]f32"), ("B", "[][][]f32")]),
-        _entry("bmm_f16", "[][][]f32", [("A", "[][][]f16"), ("B", "[][][]f16")]),
-        _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")]),
-        _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")]),
+        _entry("bmm_f32", "[][][]f32", [("A", "[][][]f32"), ("B", "[][][]f32")], [MATMUL_PARAM]),
+        _entry("bmm_f16", "[][][]f32", [("A", "[][][]f16"), ("B", "[][][]f16")], [MATMUL_PARAM]),
+        _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")], [MATMUL_PARAM]),
+        _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")], [MATMUL_PARAM]),
         _entry("radix_sort_u32", "[]u32", [("keys", "[]u32")]),
         _entry("radix_sort_u64", "[]u64", [("keys", "[]u64")]),
     ]

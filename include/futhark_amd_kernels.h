@@ -70,6 +70,27 @@ const char *fa_strerror(int code);
 /* Library/ABI version: major*1000 + minor. */
 int fa_version(void);
 
+/* Thresholds behind the launchers' choice of code path, the counterpart of
+ * the threshold and shared_memory tuning parameters a compiled program exposes
+ * (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:118-120, rts/c/gpu.h:93-135).  They are
+ * process-wide; a field that is 0 means the built-in default.
+ *   segred_small_threshold  rows of a regular segmented reduce up to this many
+ *                           elements are folded by groups of lanes, longer
+ *                           ones by whole blocks (default 8192)
+ *   hist_lds_bins_max       most bins (of 4 bytes; half as many of 8) one LDS
+ *                           range of a histogram holds (default and upper
+ *                           limit 32768); four ranges fit one launch, more
+ *                           bins go through the partitioned path
+ *   matmul_pad_min_work     least M*N*K*batch for which shapes off the tile
+ *                           grid run on padded copies (default 2^24) */
+typedef struct fa_tuning {
+  int64_t segred_small_threshold;
+  int64_t hist_lds_bins_max;
+  int64_t matmul_pad_min_work;
+} fa_tuning;
+void fa_set_tuning(const fa_tuning *t); /* NULL: all defaults */
+void fa_get_tuning(fa_tuning *out);     /* the values in effect */
+
 /* ------------------------------------------------------------------ SegRed
  * Non-segmented reduction `reduce op ne xs`.
  * Replaces: segred_nonseg (SegRed.hs:327-394): stage one, per-block partials,

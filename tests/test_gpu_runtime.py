@@ -130,3 +130,40 @@ def test_debugging_log_goes_to_the_logging_file(segops_lib, tmp_path):
     libc.fclose(f)
     text = path.read_text()
     assert "Allocating" in text and "segscan" in text
+
+
+def test_tuning_parameters_select_other_code_paths_with_the_same_results(segops_lib):
+    """The three tuning parameters are thresholds inside the kernel library.  Values far from
+    the defaults push small inputs down the paths that large inputs take."""
+    import oracle
+    rng = np.random.default_rng(12)
+    tuning = {"segops.hist_lds_bins_max": 256, "segops.segred_small_threshold": 16,
+              "segops.matmul_pad_min_work": 1}
+    with Context(segops_lib, profiling=True, tuning=tuning) as c:
+        # 3000 bins > 4 ranges of 256: the partitioned histogram
+        is_ = rng.integers(-5, 3005, 200000).astype(np.int32)
+        vs = rng.integers(-1000, 1000, 200000).astype(np.int32)
+        out = c.call("hist_add_i32", ["i32_1d"], 3000, c.new("i32_1d", is_), c.new("i32_1d", vs))
+        assert np.array_equal(out.values(), oracle.hist("add", "i32", 3000, is_, vs))
+        # 700 bins: three LDS ranges in one launch
+        out = c.call("hist_max_i32", ["i32_1d"], 700, c.new("i32_1d", is_ % 700), c.new("i32_1d", vs))
+        assert np.array_equal(out.values(), oracle.hist("max", "i32", 700, is_ % 700, vs))
+        # rows of 100 > 16: whole blocks per row; rows of 40000 in pieces
+        for m, k in [(300, 100), (3, 40000)]:
+            xss = rng.integers(-1000, 1000, (m, k)).astype(np.int64)
+            out = c.call("segreduce_add_i64", ["i64_1d"], c.new("i64_2d", xss))
+            assert np.array_equal(out.values(), xss.sum(axis=1))
+        # a 200 x 200 x 30 product on padded operands (1.2 M multiply-adds: below the default)
+        A = rng.standard_normal((1, 200, 30)).astype(np.float32)
+        B = rng.standard_normal((1, 30, 200)).astype(np.float32)
+        out = c.call("bmm_f32", ["f32_3d"], c.new("f32_3d", A), c.new("f32_3d", B))
+        np.testing.assert_allclose(out.values(), A.astype(np.float64) @ B.astype(np.float64), rtol=1e-4, atol=1e-5)
+        ev = [e for e in json.loads(c.report())["events"] if e["name"] == "segmap_matmul"]
+        assert ev[0]["details"]["padded"] is True
+    with Context(segops_lib, profiling=True) as c:    # back to the defaults
+        out = c.call("bmm_f32", ["f32_3d"], c.new("f32_3d", A), c.new("f32_3d", B))
+        np.testing.assert_allclose(out.values(), A.astype(np.float64) @ B.astype(np.float64), rtol=1e-4, atol=1e-5)
+        ev = [e for e in json.loads(c.report())["events"] if e["name"] == "segmap_matmul"]
+        assert ev[0]["details"]["padded"] is False
+    with pytest.raises(KeyError):
+        Context(segops_lib, tuning={"segops.no_such_parameter": 1})

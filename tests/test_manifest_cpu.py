@@ -92,4 +92,5 @@ def test_every_function_the_manifest_names_is_exported_and_every_entry_is_listed
     entries = {s for s in exported if s.startswith("futhark_entry_")}
     assert entries == {e["cfun"] for e in m["entry_points"].values()}
     tuning = {p for e in m["entry_points"].values() for p in e["tuning_params"]}
-    assert tuning == {"segops.hist_lds_bins_max", "segops.segred_small_threshold"}
+    assert tuning == {"segops.hist_lds_bins_max", "segops.segred_small_threshold",
+                      "segops.matmul_pad_min_work"}
