@@ -273,3 +273,33 @@ def test_scan_of_rows(ctx, t, op):
             for h in (same, f, v):
                 h.free()
         out.free(); a.free()
+
+
+@pytest.mark.parametrize("t", ["i32", "i64"])
+def test_segscan_long_look_back_chains(ctx, t):
+    """Flag patterns chosen for the look-back: segment starts hundreds of tiles apart (chains that
+    cross several 64-tile windows before they meet a start), starts exactly on tile boundaries and
+    on their neighbours, and runs of tiles with and without starts in turn.  2^23 elements are
+    256 tiles of 4-byte and 512 tiles of 8-byte elements."""
+    n = 1 << 23
+    tile = 32768 if t == "i32" else 8192
+    xs = _data(t, n, 21)
+    a = ctx.new(f"{t}_1d", xs)
+    patterns = {
+        "four starts": [0, n // 3 + 5, n // 2, n - 7],
+        "on tile boundaries": [k * tile for k in range(0, n // tile, 37)],
+        "around tile boundaries": [k * tile + d for k in range(1, n // tile, 29) for d in (-1, 1)],
+        "dense then none": list(range(0, 5 * tile, 97)) + [200 * tile + 3],
+        "alternating tiles": [k * tile + tile // 2 for k in range(0, n // tile, 2)],
+        "last element only": [n - 1],
+    }
+    for name, starts in patterns.items():
+        flags = np.zeros(n, np.uint8)
+        flags[np.array(starts)] = 1
+        f = ctx.new("u8_1d", flags)
+        for op in ("add", "max"):
+            out = ctx.call(f"segscan_{op}_{t}", [f"{t}_1d"], f, a)
+            assert np.array_equal(out.values(), oracle.segscan(op, t, flags, xs)), (name, op)
+            out.free()
+        f.free()
+    a.free()
