@@ -172,3 +172,40 @@ def test_segmented_hist_full_size_matches_row_sums(ctx):
     assert np.array_equal(got[rows], oracle.seghist("add", "i32", H, iss[rows], vss[rows]))
     for h in (out, i, v):
         h.free()
+
+
+def test_i64_indices_through_the_kernel_library(ctx):
+    """fa_seghist takes i64 indices as well (Futhark's hist does; the entry points of this program
+    widen i32 ones): every path with is64 = 1 against the oracle, including indices that only fit
+    64 bits."""
+    import ctypes as C
+    from futhark_amd import lib_path
+    k = C.CDLL(str(lib_path("libfuthark_amd_kernels.so")))
+    k.fa_seghist.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_void_p,
+                             C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_size_t]
+    k.fa_seghist_scratch_bytes.restype = C.c_size_t
+    k.fa_seghist_scratch_bytes.argtypes = [C.c_int, C.c_int, C.c_int64, C.c_int64]
+    FA_I32, FA_F32, FA_ADD, FA_MAX = 0, 2, 0, 1
+    rng = np.random.default_rng(23)
+    n = 300001
+    for H in (200, 5000, 200000, 9000000):   # wave-private / LDS, LDS ranges, partitioned, global
+        is64 = rng.integers(-3, H + 3, n).astype(np.int64)
+        is64[::1000] = (1 << 40) + 5          # far out of range, and not an i32
+        is64[1::1000] = -(1 << 35)
+        is32 = np.where((is64 >= 0) & (is64 < H), is64, -1).astype(np.int32)
+        for t, code, op, opname, vals in (
+                ("i32", FA_I32, FA_ADD, "add", rng.integers(-1000, 1000, n).astype(np.int32)),
+                ("f32", FA_F32, FA_ADD, "add", rng.integers(-8, 8, n).astype(np.float32)),
+                ("f32", FA_F32, FA_MAX, "max", rng.standard_normal(n).astype(np.float32))):
+            d_is, d_vs = ctx.new("i64_1d", is64), ctx.new(f"{t}_1d", vals)
+            dest0 = oracle.hist(opname, t, H, np.zeros(0, np.int32), vals[:0])   # neutral elements
+            dest = ctx.new(f"{t}_1d", dest0)
+            sb = k.fa_seghist_scratch_bytes(code, 1, n, H)
+            scratch = ctx.new("u8_1d", np.zeros(max(sb, 256), np.uint8))
+            print(f"fa_seghist is64 {t} {opname} H={H}", flush=True)
+            rc = k.fa_seghist(ctx.stream, code, op, d_is.device_ptr, 1, d_vs.device_ptr, n,
+                              dest.device_ptr, H, scratch.device_ptr, sb)
+            assert rc == 0
+            assert np.array_equal(dest.values(), oracle.hist(opname, t, H, is32, vals)), (t, opname, H)
+            for h in (d_is, d_vs, dest, scratch):
+                h.free()
