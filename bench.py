@@ -179,6 +179,21 @@ def make_workload(name: str, ctx):
         w.update(step=step, bytes=m * k * dt().itemsize + m * dt().itemsize, kernel="segred_regular",
                  dtype=t, bound="hbm", keep=[a],
                  describe=f"regular segmented reduce ({op}) of [{m}][{k}]{t}")
+    elif name.startswith("vecreduce_"):
+        # vecreduce_add_f32_65536x1024: reduce (map2 op) (replicate k ne) xss, xss : [n][k]
+        _, op, t, shape = name.split("_")
+        n, k = (int(x) for x in shape.split("x"))
+        w["elements"] = n * k
+        dt = {"f32": np.float32, "i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        xss = (dg.uniform_f32(38, n * k) if t[0] == "f" else dg.uniform_int(39, n * k, -1000, 1000)
+               ).astype(dt).reshape(n, k)
+        a = ctx.new(f"{t}_2d", xss)
+
+        def step():
+            ctx.call(f"vecreduce_{op}_{t}", [f"{t}_1d"], a).free()
+        w.update(step=step, bytes=n * k * dt().itemsize + k * dt().itemsize, kernel="segred_columns",
+                 dtype=t, bound="hbm", keep=[a],
+                 describe=f"reduce with vectorised operator (map2 {op}) of [{n}][{k}]{t}")
     elif name.startswith("transpose_"):
         # transpose_f32_8192x8192
         _, t, shape = name.split("_")

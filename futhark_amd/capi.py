@@ -113,6 +113,7 @@ class Segops:
                 getattr(L, f"futhark_entry_segscan_{op}_{t}").argtypes = [vp, pp, vp, vp]
                 getattr(L, f"futhark_entry_segred_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
                 getattr(L, f"futhark_entry_segreduce_{op}_{t}").argtypes = [vp, pp, vp]
+                getattr(L, f"futhark_entry_vecreduce_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_seghist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
                 getattr(L, f"futhark_entry_scanrows_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]

@@ -309,6 +309,33 @@ static int do_segred(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
   return 0;
 }
 
+/* reduce (map2 OP) (replicate k NE) xss : [k]T for xss : [n][k]T */
+static int do_vecreduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                        struct fut_array **out, const struct fut_array *in) {
+  const int64_t n = in->shape[0], k = in->shape[1];
+  struct fut_array *res = out_array(ctx, k * (int64_t)es, 1, &k, "vecreduce.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  struct memblock_device ws = {0};
+  const size_t ws_bytes = fa_segred_columns_workspace_bytes(t, n, k);
+  int err = 0;
+  if (ws_bytes > 0) err = rts_memblock_alloc(ctx, &ws, (int64_t)ws_bytes, "vecreduce.workspace");
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "segred_columns",
+        rts_msgprintf("{\"rows\":%lld,\"vector_size\":%lld}", (long long)n, (long long)k));
+    int code = fa_segred_columns(ctx->stream, t, op, in->mem.mem, n, k, res->mem.mem, ws.mem,
+                                 ws_bytes);
+    err = rts_kernel_end(ctx, ev, "segred_columns", code);
+  }
+  rts_memblock_unref(ctx, &ws, "vecreduce.workspace");
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
 static int do_segreduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
                         struct fut_array **out, const struct fut_array *in) {
   const int64_t m = in->shape[0], k = in->shape[1];
@@ -526,6 +553,15 @@ static int do_seghist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t 
     ENTER(ctx);                                                                               \
     int ret =                                                                                 \
         do_segreduce(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a);   \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_vecreduce_##OP##_##T(struct futhark_context *ctx,                         \
+                                         struct futhark_##T##_1d **out0,                      \
+                                         const struct futhark_##T##_2d *in0) {                \
+    ENTER(ctx);                                                                               \
+    int ret =                                                                                 \
+        do_vecreduce(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a);   \
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }                                                                                           \

@@ -175,6 +175,11 @@ struct entry {
     return futhark_entry_segreduce_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,        \
                                               ARRP(i[0]));                                     \
   }                                                                                            \
+  static int e_vecreduce_##OP##_##T(struct futhark_context *c, struct value *o,                \
+                                    struct value **i) {                                        \
+    return futhark_entry_vecreduce_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,        \
+                                              ARRP(i[0]));                                     \
+  }                                                                                            \
   static int e_scanrows_##OP##_##T(struct futhark_context *c, struct value *o,                 \
                                    struct value **i) {                                         \
     return futhark_entry_scanrows_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,         \
@@ -264,6 +269,7 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
    {0}, {NULL}},                                                                                \
   {"segreduce_" #OP "_" #T, e_segreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0},            \
    {SEGRED_PARAM, NULL}},                                                                       \
+  {"vecreduce_" #OP "_" #T, e_vecreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},   \
   {"scanrows_" #OP "_" #T, e_scanrows_##OP##_##T, "[][]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},   \
   {"seghist_" #OP "_" #T, e_seghist_##OP##_##T, "[][]" #T, 1, 3,                                \
    {"i64", "[][]i32", "[][]" #T}, {0}, {HIST_PARAM, NULL}},                                     \

@@ -50,6 +50,7 @@ def entry_points() -> dict:
                 _entry(f"segscan_{op}_{t}", a, [("flags", "[]u8"), ("vs", a)]),
                 _entry(f"segred_{op}_{t}", a, [("offsets", "[]i64"), ("lens", "[]i64"), ("vs", a)]),
                 _entry(f"segreduce_{op}_{t}", a, [("xss", "[]" + a)], [SEGRED_PARAM]),
+                _entry(f"vecreduce_{op}_{t}", a, [("xss", "[]" + a)]),
                 _entry(f"scanrows_{op}_{t}", "[]" + a, [("xss", "[]" + a)]),
                 _entry(f"seghist_{op}_{t}", "[]" + a,
                        [("k", "i64"), ("iss", "[][]i32"), ("vss", "[]" + a)], [HIST_PARAM]),

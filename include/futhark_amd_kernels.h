@@ -116,6 +116,18 @@ int fa_segred_regular_ws(fa_stream_t stream, fa_dtype t, fa_op op,
                          const void *xss, int64_t m, int64_t k, void *out,
                          void *workspace, size_t workspace_bytes);
 
+/* Reduction with a vectorised operator, `reduce (map2 op) (replicate k ne) xss`
+ * with xss : [n][k] row-major: out[j] = fold over i of xss[i][j], k results
+ * (the reference interchanges the loops of such a SegRed so that each thread
+ * folds one element of the vector, SegRed.hs:274-290).  n = 0 gives k neutral
+ * elements.  workspace: fa_segred_columns_workspace_bytes() bytes, 16-byte
+ * aligned, contents irrelevant; without it one block per column strip folds
+ * all rows. */
+size_t fa_segred_columns_workspace_bytes(fa_dtype t, int64_t n, int64_t k);
+int fa_segred_columns(fa_stream_t stream, fa_dtype t, fa_op op,
+                      const void *xss, int64_t n, int64_t k, void *out,
+                      void *workspace, size_t workspace_bytes);
+
 /* ----------------------------------------------------------------- SegScan
  * Single-pass scan with decoupled look-back.
  * Replaces: segscan (SegScan/SinglePass.hs:327-879) plus the status-flag fill

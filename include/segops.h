@@ -21,6 +21,7 @@
  *     in map2 (\o l -> if l == 0 then NE else s[o+l-1]) offsets lens
  *                                   -- Builtins.hs:570-602
  *   entry segreduce_OP_T (xss: [][]T) : []T    = map (reduce OP NE) xss
+ *   entry vecreduce_OP_T (xss: [n][k]T) : [k]T = reduce (map2 OP) (replicate k NE) xss
  *   entry scanrows_OP_T (xss: [][]T) : [][]T   = map (scan OP NE) xss
  *   entry hist_OP_T (k: i64) (is: []i32) (vs: []T) : [k]T =
  *     hist OP NE k (map i64.i32 is) vs           -- prelude/soacs.fut:132-146
@@ -245,6 +246,9 @@ FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
                                       const struct futhark_i64_1d *in1,                       \
                                       const struct futhark_##T##_1d *in2);                    \
   int futhark_entry_segreduce_##OP##_##T(struct futhark_context *ctx,                         \
+                                         struct futhark_##T##_1d **out0,                      \
+                                         const struct futhark_##T##_2d *in0);                 \
+  int futhark_entry_vecreduce_##OP##_##T(struct futhark_context *ctx,                         \
                                          struct futhark_##T##_1d **out0,                      \
                                          const struct futhark_##T##_2d *in0);                 \
   int futhark_entry_scanrows_##OP##_##T(struct futhark_context *ctx,                          \

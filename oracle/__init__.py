@@ -95,6 +95,24 @@ def segreduce(op: str, t: str, xss):
     return out
 
 
+def vecreduce(op: str, t: str, xss, variant: str = "lit"):
+    """reduce (map2 op) (replicate k ne) xss for xss : [n][k] -> [k]."""
+    _, dt = _CT[t]
+    xss = _arr(xss, dt)
+    n, k = xss.shape
+    out = np.empty(k, dtype=dt)
+    if variant != "lit":  # one reduction per column
+        cols = np.ascontiguousarray(xss.T)
+        for j in range(k):
+            out[j] = reduce(op, t, cols[j], variant)
+        return out
+    fn = getattr(lib(), f"orc_vecreduce_{op}_{t}_lit")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p]
+    fn(_p(xss), n, k, _p(out))
+    return out
+
+
 def rbi(op: str, t: str, dest, is_, vs, variant: str = "lit"):
     """reduce_by_index on a copy of dest."""
     _, dt = _CT[t]

@@ -134,6 +134,12 @@ static inline double min_f64(double a, double b) { return fmin(a, b); }
   void orc_segreduce_##OP##_##S##_lit(const T *xss, int64_t m, int64_t k, T *out) {            \
     for (int64_t i = 0; i < m; i++) out[i] = orc_reduce_##OP##_##S##_lit(xss + i * k, k);      \
   }                                                                                            \
+  /* reduce (map2 OP) (replicate k NE) xss, rows folded in order */                            \
+  void orc_vecreduce_##OP##_##S##_lit(const T *xss, int64_t n, int64_t k, T *out) {            \
+    for (int64_t j = 0; j < k; j++) out[j] = NE_##OP##_##S;                                    \
+    for (int64_t i = 0; i < n; i++)                                                            \
+      for (int64_t j = 0; j < k; j++) out[j] = OP##_##S(out[j], xss[i * k + j]);               \
+  }                                                                                            \
   /* hist / reduce_by_index: FirstOrderTransform.hs:505-560 */                                 \
   void orc_rbi_##OP##_##S##_lit(T *dest, int64_t H, const int32_t *is, const T *vs,            \
                                 int64_t n) {                                                   \

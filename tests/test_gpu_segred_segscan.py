@@ -201,6 +201,31 @@ def test_segreduce_regular(ctx, goldens, t):
         assert np.array_equal(outm.values(), oracle.segreduce("max", t, xss))
 
 
+@pytest.mark.parametrize("t", ["i32", "i64", "f32", "f64"])
+def test_reduce_with_vectorised_operator(ctx, t):
+    """reduce (map2 op) (replicate k ne) xss (tests/soacs/reduce7.fut has the shape): vectors
+    shorter than a wave's span (several rows per span, whole 16-byte vectors and not), as long,
+    longer (several strips, a ragged last one), one row, no rows, many rows (two stages)."""
+    for n, k in [(1, 1), (7, 1), (1000, 2), (1000, 3), (999, 4), (513, 12), (100, 64), (300, 100),
+                 (100, 100), (77, 128), (50, 252), (33, 256), (200, 260), (64, 1000), (9, 4099),
+                 (100003, 8), (70001, 5), (20000, 96), (3000, 1024), (1, 5000), (0, 6), (6, 0),
+                 (2, 1 << 20), (1 << 20, 2), (50000, 257)]:
+        xss = _data(t, n * k, 21).reshape(n, k)
+        a = ctx.new(f"{t}_2d", xss)
+        for op in ("add", "max", "min"):
+            out = ctx.call(f"vecreduce_{op}_{t}", [f"{t}_1d"], a)
+            got = out.values()
+            assert got.shape == (k,)
+            if t == "f32" and op == "add":
+                _close(got, xss.astype(np.float64).sum(axis=0))
+            elif t == "f64" and op == "add":
+                _close(got, oracle.vecreduce(op, t, xss), 1e-12)
+            else:
+                assert np.array_equal(got, oracle.vecreduce(op, t, xss)), (n, k, op)
+            out.free()
+        a.free()
+
+
 def test_config1_full_size(ctx):
     n = 1 << 24
     xi = dg.uniform_int(16, n, -1000, 1000)

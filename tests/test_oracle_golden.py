@@ -285,3 +285,21 @@ def test_multicore_baseline_agrees_with_oracle():
                           oracle.rbi("add", "i32", np.zeros(256, np.int32), is_, xs))
     big = oracle.mc_rbi_add_i32(np.zeros(200000, np.int32), is_, xs, 4)  # atomic path
     assert np.array_equal(big, oracle.rbi("add", "i32", np.zeros(200000, np.int32), is_, xs))
+
+
+def test_vectorised_reduce_is_a_reduce_per_column():
+    """reduce (map2 op) ne xss folds every column on its own: the same as the regular segmented
+    reduce of the transposed array, and numpy's wrapping integer reductions along axis 0."""
+    rng = np.random.default_rng(5)
+    for n, k in [(0, 3), (1, 5), (17, 4), (100, 33)]:
+        xi = rng.integers(-2**31, 2**31, (n, k), dtype=np.int64).astype(np.int32)
+        for op, f in (("add", np.add), ("max", np.maximum), ("min", np.minimum)):
+            got = oracle.vecreduce(op, "i32", xi)
+            assert np.array_equal(got, oracle.segreduce(op, "i32", np.ascontiguousarray(xi.T)))
+            if n > 0:
+                assert np.array_equal(got, f.reduce(xi, axis=0, dtype=np.int32))
+        xf = rng.standard_normal((n, k)).astype(np.float32)
+        assert np.array_equal(oracle.vecreduce("add", "f32", xf),
+                              oracle.segreduce("add", "f32", np.ascontiguousarray(xf.T)))
+        np.testing.assert_allclose(oracle.vecreduce("add", "f32", xf, "f64acc"),
+                                   xf.astype(np.float64).sum(axis=0), rtol=1e-6, atol=1e-6)
