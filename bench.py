@@ -112,6 +112,45 @@ def make_workload(name: str, ctx):
                                        f"indices, 1% out of range")
         if t == "i32" and op == "add":
             w["cpu"] = lambda: oracle.mc_rbi_add_i32(np.zeros(H, np.int32), is_, vs)
+    elif name.startswith("rbivec_"):
+        # rbivec_add_i32_H256x16_2p23: 2^23 updates of 16-element vectors into [256][16] bins
+        _, op, t, hs, sz = name.split("_")
+        n = 1 << int(sz[2:])
+        H, m = (int(x) for x in hs[1:].split("x"))
+        w["elements"] = n * m
+        dt = {"f32": np.float32, "i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        is_ = dg.hist_indices(52, n, H, "uniform").astype(np.int64)
+        vss = (dg.uniform_f32(53, n * m) if t[0] == "f" else dg.uniform_int(54, n * m, -1000, 1000)
+               ).astype(dt).reshape(n, m)
+        d, i, v = ctx.new(f"{t}_2d", np.zeros((H, m), dt)), ctx.new("i64_1d", is_), ctx.new(f"{t}_2d", vss)
+
+        def step():
+            ctx.call(f"rbi_vec_{op}_{t}", [f"{t}_2d"], d, i, v).free()
+        es = dt().itemsize
+        w.update(step=step, bytes=n * 8 + n * m * es + 2 * H * m * es, kernel="seghist_shaped",
+                 dtype=t, bound="hbm", keep=[d, i, v],
+                 describe=f"reduce_by_index with operator map2 {op}: 2^{sz[2:]} vectors of {m} {t} "
+                          f"into [{H}][{m}] bins, uniform i64 indices, 1% out of range")
+    elif name.startswith("rbi2d_"):
+        # rbi2d_add_i32_256x256_2p27: reduce_by_index_2d into [256][256] bins
+        _, op, t, hs, sz = name.split("_")
+        n = 1 << int(sz[2:])
+        H0, H1 = (int(x) for x in hs.split("x"))
+        w["elements"] = n
+        dt = {"f32": np.float32, "i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        is_ = dg.hist_indices(55, n, H0, "uniform").astype(np.int64)
+        js = dg.hist_indices(56, n, H1, "uniform").astype(np.int64)
+        vs = (dg.uniform_f32(57, n) if t[0] == "f" else dg.uniform_int(58, n, -1000, 1000)).astype(dt)
+        d = ctx.new(f"{t}_2d", np.zeros((H0, H1), dt))
+        i, j, v = ctx.new("i64_1d", is_), ctx.new("i64_1d", js), ctx.new(f"{t}_1d", vs)
+
+        def step():
+            ctx.call(f"rbi_2d_{op}_{t}", [f"{t}_2d"], d, i, j, v).free()
+        es = dt().itemsize
+        w.update(step=step, bytes=n * (16 + es) + 2 * H0 * H1 * es, kernel="seghist_shaped", dtype=t,
+                 bound="hbm", keep=[d, i, j, v],
+                 describe=f"reduce_by_index_2d ({op}) of 2^{sz[2:]} {t} into [{H0}][{H1}] bins, "
+                          f"uniform i64 index pairs, 1% out of range per coordinate")
     elif name.startswith("sort_"):
         # sort_u32_2p26 | sort_u64i32_2p26
         _, kt, sz = name.split("_")

@@ -118,6 +118,8 @@ class Segops:
                 getattr(L, f"futhark_entry_scanrows_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
                 getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
+                getattr(L, f"futhark_entry_rbi_vec_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
+                getattr(L, f"futhark_entry_rbi_2d_{op}_{t}").argtypes = [vp, pp, vp, vp, vp, vp]
         for t in HIST_ONLY_TYPES:
             for op in ops_for(t):
                 getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]

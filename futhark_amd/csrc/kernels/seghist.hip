@@ -247,10 +247,23 @@ template <class E> __device__ __forceinline__ void load_elems4(E (&dst)[4], cons
 // [0, H_seg), is bin row * H_seg + b of the m * H_seg = H bins of dest.  A
 // thread keeps (row, column) of its current vector and advances them by the
 // grid stride, so there is one division per thread, not per element.
-template <class T, class Op, class I, bool SEGMENTED>
+//
+// VECTOR: the operator works on whole vectors of seg_len elements
+// (`reduce_by_index dest (map2 op) (replicate seg_len ne) is vss`, the HistOp
+// with an operator shape, SegHist.hs:1057-1136; tests/hist/array.fut): vs is
+// [n / seg_len][seg_len], is has one index per row, and element (r, c) goes
+// to bin is[r] * seg_len + c when is[r] lies in [0, H_seg).
+//
+// PAIRS: two index arrays, is and js, address [H_seg][seg_len] bins
+// (`reduce_by_index_2d`, prelude/soacs.fut:149-150): element p goes to bin
+// is[p] * seg_len + js[p] when is[p] lies in [0, H_seg) and js[p] in [0, seg_len).
+enum { HIST_PLAIN = 0, HIST_ROWS = 1, HIST_VECTOR = 2, HIST_PAIRS = 3 };
+
+template <class T, class Op, class I, int MODE>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
-    const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t bin_base,
-    int64_t H, int range_bins, int P, int log2_copies, int64_t seg_len, int64_t H_seg) {
+    const I *__restrict__ is, const I *__restrict__ js, const T *__restrict__ vs, int64_t n, T *dest,
+    int64_t bin_base, int64_t H, int range_bins, int P, int log2_copies, int64_t seg_len,
+    int64_t H_seg) {
   using A = typename HistAcc<T>::A;
   using OpA = typename RebindOp<Op, A>::type;
   extern __shared__ __align__(16) unsigned char s_raw[];
@@ -280,7 +293,13 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
     if ((uint64_t)r < (uint64_t)nb)
       lds_update<A, OpA>(&sh[((int)r << log2_copies) + copy], (A)v);
   };
-  // Bin of dest for (position, raw bin): identity unless SEGMENTED.
+  // (row, column) of every element is tracked
+  constexpr bool SEGMENTED = MODE == HIST_ROWS || MODE == HIST_VECTOR;
+  auto pair_bin = [&](int64_t i, int64_t j) -> int64_t {
+    return (uint64_t)i < (uint64_t)H_seg && (uint64_t)j < (uint64_t)seg_len ? i * seg_len + j
+                                                                           : (int64_t)-1;
+  };
+  // Bin of dest for (position, raw bin) in a histogram per row.
   auto seg_bin = [&](int64_t row, int64_t b) -> int64_t {
     return (uint64_t)b < (uint64_t)H_seg ? row * H_seg + b : (int64_t)-1;
   };
@@ -296,9 +315,32 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
     for (int64_t i = i0; i < nvec; i += stride) {
       I bi[VEC];
       T bv[VEC];
-      load_elems4(bi, is + i * VEC);
+      if constexpr (MODE != HIST_VECTOR) load_elems4(bi, is + i * VEC);
       load_elems4(bv, vs + i * VEC);
-      if constexpr (SEGMENTED) {
+      if constexpr (MODE == HIST_PAIRS) {
+        I bj[VEC];
+        load_elems4(bj, js + i * VEC);
+#pragma unroll
+        for (int e = 0; e < VEC; e++) update(pair_bin((int64_t)bi[e], (int64_t)bj[e]), bv[e]);
+      } else if constexpr (MODE == HIST_VECTOR) {
+        int64_t r = row, c = col;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+          while (c >= seg_len) {
+            c -= seg_len;
+            r++;
+          }
+          const int64_t b = (int64_t)is[r];
+          update((uint64_t)b < (uint64_t)H_seg ? b * seg_len + c : (int64_t)-1, bv[e]);
+          c++;
+        }
+        row += row_step;
+        col += col_step;
+        if (col >= seg_len) {
+          col -= seg_len;
+          row++;
+        }
+      } else if constexpr (SEGMENTED) {
         int64_t r = row, c = col;
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
@@ -323,8 +365,16 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
     if (s == 0) {
       const int64_t t = nvec * VEC + threadIdx.x;
       if (threadIdx.x < VEC && t < n) {
-        if constexpr (SEGMENTED) update(seg_bin(t / seg_len, (int64_t)is[t]), vs[t]);
-        else update((int64_t)is[t], vs[t]);
+        if constexpr (MODE == HIST_PAIRS) {
+          update(pair_bin((int64_t)is[t], (int64_t)js[t]), vs[t]);
+        } else if constexpr (MODE == HIST_VECTOR) {
+          const int64_t b = (int64_t)is[t / seg_len];
+          update((uint64_t)b < (uint64_t)H_seg ? b * seg_len + t % seg_len : (int64_t)-1, vs[t]);
+        } else if constexpr (SEGMENTED) {
+          update(seg_bin(t / seg_len, (int64_t)is[t]), vs[t]);
+        } else {
+          update((int64_t)is[t], vs[t]);
+        }
       }
     }
   }
@@ -519,9 +569,10 @@ static int hist_num_cus() {
 }
 
 // Launches the LDS kernel over bins [0,H) of `dest` (H <= max ranges * range size).
-template <class T, class Op, class I, bool SEGMENTED = false>
+template <class T, class Op, class I, int MODE = HIST_PLAIN>
 static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
-                           int64_t H, int64_t seg_len = 0, int64_t H_seg = 0) {
+                           int64_t H, int64_t seg_len = 0, int64_t H_seg = 0,
+                           const I *js = nullptr) {
   using A = typename HistAcc<T>::A;
   const int max_range = hist_range_bins_max(sizeof(A));
   const int P = (int)ceil_div(H, max_range);
@@ -535,7 +586,7 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
   int grid = hist_num_cus() * per_cu;
   grid -= grid % (NUM_XCDS * P);
   if (grid < NUM_XCDS * P) grid = NUM_XCDS * P;
-  auto kernel = seghist_lds_kernel<T, Op, I, SEGMENTED>;
+  auto kernel = seghist_lds_kernel<T, Op, I, MODE>;
   static bool raised = false;
   if (!raised) {
     hipError_t e = hipFuncSetAttribute((const void *)kernel,
@@ -543,8 +594,8 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
     if (e != hipSuccess) return (int)e;
     raised = true;
   }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(HIST_BLOCK), lds, st, is, vs, n, dest, (int64_t)0,
-                     H, range_bins, P, log2_copies, seg_len, H_seg);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(HIST_BLOCK), lds, st, is, js, vs, n, dest,
+                     (int64_t)0, H, range_bins, P, log2_copies, seg_len, H_seg);
   return launch_status();
 }
 
@@ -670,9 +721,9 @@ static int launch_hist_segmented(hipStream_t st, const void *is, int is64, const
       (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
   if (H <= lds_limit) {
     if (is64)
-      return launch_lds_hist<T, Op, int64_t, true>(st, (const int64_t *)is, (const T *)vs, n,
+      return launch_lds_hist<T, Op, int64_t, HIST_ROWS>(st, (const int64_t *)is, (const T *)vs, n,
                                                    (T *)dest, H, seg_len, H_seg);
-    return launch_lds_hist<T, Op, int32_t, true>(st, (const int32_t *)is, (const T *)vs, n,
+    return launch_lds_hist<T, Op, int32_t, HIST_ROWS>(st, (const int32_t *)is, (const T *)vs, n,
                                                  (T *)dest, H, seg_len, H_seg);
   }
   // Too many bins for one launch of LDS ranges: flatten the indices, then the
@@ -690,6 +741,67 @@ static int launch_hist_segmented(hipStream_t st, const void *is, int is64, const
   const int rc = launch_status();
   if (rc != 0) return rc;
   return launch_hist<T, Op>(st, flat, 1, vs, n, dest, H, (char *)scratch + flat_bytes,
+                            scratch_bytes - flat_bytes);
+}
+
+// Flat bins for a histogram over [H0][H1] bins of vectors of m elements:
+// element e of vss belongs to update u = e / m and goes to bin
+// ((is[u] * H1 + js[u]) * m + e % m), or nowhere (-1) when a coordinate is out
+// of range.  js == nullptr stands for H1 = 1 and no second coordinate.
+template <class I>
+__global__ __launch_bounds__(256) void seghist_shape_kernel(const I *__restrict__ is,
+                                                            const I *__restrict__ js, int64_t n,
+                                                            int64_t H0, int64_t H1, int64_t m,
+                                                            int64_t *__restrict__ flat) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < n; e += stride) {
+    const int64_t u = e / m;
+    const int64_t i = (int64_t)is[u], j = js != nullptr ? (int64_t)js[u] : 0;
+    const bool inside = (uint64_t)i < (uint64_t)H0 && (uint64_t)j < (uint64_t)H1;
+    flat[e] = inside ? (i * H1 + j) * m + e % m : (int64_t)-1;
+  }
+}
+
+template <class T, class Op>
+static int launch_hist_shaped(hipStream_t st, const void *is, const void *js, int is64,
+                              const void *vss, int64_t n_updates, void *dest, int64_t H0,
+                              int64_t H1, int64_t m, void *scratch, size_t scratch_bytes) {
+  const int64_t n = n_updates * m, H = H0 * H1 * m;
+  if (H == 0 || n == 0) return 0;
+  if (!is_aligned(is, 16) || !is_aligned(vss, 16) || !is_aligned(dest, sizeof(T)) ||
+      (js != nullptr && !is_aligned(js, 16)))
+    return FA_EALIGN;
+  const int64_t lds_limit =
+      (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
+  if (js == nullptr && m > 1 && H <= lds_limit) {  // one index per vector: no flat indices needed
+    if (is64)
+      return launch_lds_hist<T, Op, int64_t, HIST_VECTOR>(st, (const int64_t *)is, (const T *)vss,
+                                                          n, (T *)dest, H, m, H0);
+    return launch_lds_hist<T, Op, int32_t, HIST_VECTOR>(st, (const int32_t *)is, (const T *)vss, n,
+                                                        (T *)dest, H, m, H0);
+  }
+  if (js == nullptr && m == 1)
+    return launch_hist<T, Op>(st, is, is64, vss, n, dest, H, scratch, scratch_bytes);
+  if (js != nullptr && m == 1 && H <= lds_limit) {  // index pairs: the bin is computed on the fly
+    if (is64)
+      return launch_lds_hist<T, Op, int64_t, HIST_PAIRS>(st, (const int64_t *)is, (const T *)vss, n,
+                                                         (T *)dest, H, H1, H0, (const int64_t *)js);
+    return launch_lds_hist<T, Op, int32_t, HIST_PAIRS>(st, (const int32_t *)is, (const T *)vss, n,
+                                                       (T *)dest, H, H1, H0, (const int32_t *)js);
+  }
+  const size_t flat_bytes = hist_align((size_t)n * sizeof(int64_t));
+  if (scratch_bytes < flat_bytes || !is_aligned(scratch, 256)) return FA_ESCRATCH;
+  int64_t *flat = (int64_t *)scratch;
+  const int grid = (int)std::min<int64_t>(ceil_div(n, (int64_t)256), (int64_t)hist_num_cus() * 16);
+  if (is64)
+    hipLaunchKernelGGL((seghist_shape_kernel<int64_t>), dim3(grid), dim3(256), 0, st,
+                       (const int64_t *)is, (const int64_t *)js, n, H0, H1, m, flat);
+  else
+    hipLaunchKernelGGL((seghist_shape_kernel<int32_t>), dim3(grid), dim3(256), 0, st,
+                       (const int32_t *)is, (const int32_t *)js, n, H0, H1, m, flat);
+  const int rc = launch_status();
+  if (rc != 0) return rc;
+  return launch_hist<T, Op>(st, flat, 1, vss, n, dest, H, (char *)scratch + flat_bytes,
                             scratch_bytes - flat_bytes);
 }
 
@@ -768,5 +880,35 @@ extern "C" int fa_seghist_segmented(fa_stream_t stream, fa_dtype t, fa_op op, co
       return FA_ENOTSUP;
   }
   FA_DISPATCH_TYPE_OP(launch_hist_segmented, t, op, s, is, is64, vs, m, seg_len, dest, H_seg,
+                      scratch, scratch_bytes);
+}
+
+extern "C" size_t fa_seghist_shaped_scratch_bytes(fa_dtype t, int is64, int64_t n_updates,
+                                                  int64_t H0, int64_t H1, int64_t m) {
+  if (n_updates < 0 || H0 < 0 || H1 < 0 || m < 0) return 0;
+  const int64_t n = n_updates * m;
+  return hist_align((size_t)n * sizeof(int64_t)) + fa_seghist_scratch_bytes(t, 1, n, H0 * H1 * m) +
+         fa_seghist_scratch_bytes(t, is64, n, H0 * H1 * m);
+}
+
+extern "C" int fa_seghist_shaped(fa_stream_t stream, fa_dtype t, fa_op op, const void *is,
+                                 const void *js, int is64, const void *vss, int64_t n_updates,
+                                 void *dest, int64_t H0, int64_t H1, int64_t m, void *scratch,
+                                 size_t scratch_bytes) {
+  if (n_updates < 0 || H0 < 0 || H1 < 0 || m < 0) return FA_EINVAL;
+  if (js == nullptr && H1 != 1) return FA_EINVAL;
+  // H0 * H1 * m and n_updates * m must be representable
+  if (H1 > 0 && H0 > INT64_MAX / H1) return FA_EINVAL;
+  if (m > 0 && (H0 * H1 > INT64_MAX / m || n_updates > INT64_MAX / m)) return FA_EINVAL;
+  if (H0 * H1 * m > 0 && dest == nullptr) return FA_EINVAL;
+  if (n_updates * m > 0 && (is == nullptr || vss == nullptr)) return FA_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (t) {
+    case FA_I32: case FA_I64: case FA_F32: case FA_F64:
+      break;
+    default:
+      return FA_ENOTSUP;
+  }
+  FA_DISPATCH_TYPE_OP(launch_hist_shaped, t, op, s, is, js, is64, vss, n_updates, dest, H0, H1, m,
                       scratch, scratch_bytes);
 }

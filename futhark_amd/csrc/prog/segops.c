@@ -497,6 +497,48 @@ static int do_seghist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t 
   return 0;
 }
 
+/* Histograms with a shape.  js == NULL: `reduce_by_index dest (map2 op) (replicate m ne) is vss`
+ * with dest : [k][m], vss : [n][m].  Otherwise `reduce_by_index_2d dest op ne (zip is js) vs`
+ * with dest : [k][l], vss = vs : [n]. */
+static int do_rbi_shaped(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                         struct fut_array **out, const struct fut_array *dest_in,
+                         const struct fut_array *is, const struct fut_array *js,
+                         const struct fut_array *vss, const char *entry) {
+  const int64_t n = is->shape[0];
+  const int64_t H0 = dest_in->shape[0];
+  const int64_t H1 = js != NULL ? dest_in->shape[1] : 1;
+  const int64_t m = js != NULL ? 1 : dest_in->shape[1];
+  if (vss->shape[0] != n) return bad_sizes(ctx, entry);
+  if (js != NULL && js->shape[0] != n) return bad_sizes(ctx, entry);
+  if (js == NULL && vss->shape[1] != m) return bad_sizes(ctx, entry);
+  const int64_t cells = dest_in->shape[0] * dest_in->shape[1];
+  struct fut_array *res = out_array(ctx, cells * (int64_t)es, 2, dest_in->shape, "hist.dest");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  int err = rts_copy_d2d(ctx, res->mem.mem, dest_in->mem.mem, (size_t)cells * es);
+  struct memblock_device scratch = {0};
+  if (err == 0)
+    err = rts_memblock_alloc(ctx, &scratch,
+                             (int64_t)fa_seghist_shaped_scratch_bytes(t, 1, n, H0, H1, m),
+                             "hist.scratch");
+  if (err == 0) {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "seghist_shaped",
+        rts_msgprintf("{\"n\":%lld,\"bins\":[%lld,%lld],\"vector_size\":%lld}", (long long)n,
+                      (long long)H0, (long long)H1, (long long)m));
+    int code = fa_seghist_shaped(ctx->stream, t, op, is->mem.mem, js != NULL ? js->mem.mem : NULL,
+                                 1, vss->mem.mem, n, res->mem.mem, H0, H1, m, scratch.mem,
+                                 (size_t)scratch.size);
+    err = rts_kernel_end(ctx, ev, "seghist_shaped", code);
+  }
+  rts_memblock_unref(ctx, &scratch, "hist.scratch");
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
 #define ENTER(ctx) pthread_mutex_lock(&(ctx)->lock)
 #define LEAVE(ctx) pthread_mutex_unlock(&(ctx)->lock)
 
@@ -581,6 +623,29 @@ static int do_seghist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t 
     ENTER(ctx);                                                                               \
     int ret = do_seghist(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, in0,    \
                          &in1->a, &in2->a, "seghist_" #OP "_" #T);                            \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_rbi_vec_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_2d **out0,                        \
+                                       const struct futhark_##T##_2d *in0,                    \
+                                       const struct futhark_i64_1d *in1,                      \
+                                       const struct futhark_##T##_2d *in2) {                  \
+    ENTER(ctx);                                                                               \
+    int ret = do_rbi_shaped(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0,      \
+                            &in0->a, &in1->a, NULL, &in2->a, "rbi_vec_" #OP "_" #T);          \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
+  int futhark_entry_rbi_2d_##OP##_##T(struct futhark_context *ctx,                            \
+                                      struct futhark_##T##_2d **out0,                         \
+                                      const struct futhark_##T##_2d *in0,                     \
+                                      const struct futhark_i64_1d *in1,                       \
+                                      const struct futhark_i64_1d *in2,                       \
+                                      const struct futhark_##T##_1d *in3) {                   \
+    ENTER(ctx);                                                                               \
+    int ret = do_rbi_shaped(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0,      \
+                            &in0->a, &in1->a, &in2->a, &in3->a, "rbi_2d_" #OP "_" #T);        \
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }                                                                                           \

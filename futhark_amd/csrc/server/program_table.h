@@ -190,6 +190,16 @@ struct entry {
     return futhark_entry_seghist_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,          \
                                             i[0]->u.i64, ARRP(i[1]), ARRP(i[2]));              \
   }                                                                                            \
+  static int e_rbi_vec_##OP##_##T(struct futhark_context *c, struct value *o,                  \
+                                  struct value **i) {                                          \
+    return futhark_entry_rbi_vec_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,          \
+                                            ARRP(i[0]), ARRP(i[1]), ARRP(i[2]));               \
+  }                                                                                            \
+  static int e_rbi_2d_##OP##_##T(struct futhark_context *c, struct value *o,                   \
+                                 struct value **i) {                                           \
+    return futhark_entry_rbi_2d_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,           \
+                                           ARRP(i[0]), ARRP(i[1]), ARRP(i[2]), ARRP(i[3]));    \
+  }                                                                                            \
   HIST_ENTRY_FNS(OP, T, CT)
 #define HIST_ENTRY_FNS(OP, T, CT)                                                              \
   static int e_hist_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) { \
@@ -273,6 +283,10 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
   {"scanrows_" #OP "_" #T, e_scanrows_##OP##_##T, "[][]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},   \
   {"seghist_" #OP "_" #T, e_seghist_##OP##_##T, "[][]" #T, 1, 3,                                \
    {"i64", "[][]i32", "[][]" #T}, {0}, {HIST_PARAM, NULL}},                                     \
+  {"rbi_vec_" #OP "_" #T, e_rbi_vec_##OP##_##T, "[][]" #T, 1, 3,                                \
+   {"[][]" #T, "[]i64", "[][]" #T}, {1, 0, 0}, {HIST_PARAM, NULL}},                             \
+  {"rbi_2d_" #OP "_" #T, e_rbi_2d_##OP##_##T, "[][]" #T, 1, 4,                                  \
+   {"[][]" #T, "[]i64", "[]i64", "[]" #T}, {1, 0, 0, 0}, {HIST_PARAM, NULL}},                   \
   HIST_ENTRY_ROWS(OP, T, CT)
 #define HIST_ENTRY_ROWS(OP, T, CT)                                                              \
   {"hist_" #OP "_" #T, e_hist_##OP##_##T, "[]" #T, 1, 3, {"i64", "[]i32", "[]" #T}, {0},        \

@@ -54,6 +54,11 @@ def entry_points() -> dict:
                 _entry(f"scanrows_{op}_{t}", "[]" + a, [("xss", "[]" + a)]),
                 _entry(f"seghist_{op}_{t}", "[]" + a,
                        [("k", "i64"), ("iss", "[][]i32"), ("vss", "[]" + a)], [HIST_PARAM]),
+                _entry(f"rbi_vec_{op}_{t}", "[]" + a,
+                       [("dest", "*[]" + a), ("is", "[]i64"), ("vss", "[]" + a)], [HIST_PARAM]),
+                _entry(f"rbi_2d_{op}_{t}", "[]" + a,
+                       [("dest", "*[]" + a), ("is", "[]i64"), ("js", "[]i64"), ("vs", a)],
+                       [HIST_PARAM]),
             ]
     for t in list(NUM_TYPES) + list(HIST_ONLY_TYPES):
         for op in ops_for(t):

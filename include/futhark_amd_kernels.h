@@ -202,6 +202,21 @@ int fa_seghist_segmented(fa_stream_t stream, fa_dtype t, fa_op op,
                          int64_t m, int64_t seg_len, void *dest, int64_t H_seg,
                          void *scratch, size_t scratch_bytes);
 
+/* Histograms with a shape: bins laid out as [H0][H1] vectors of m elements.
+ * Update u carries the index (is[u], js[u]) and the vector vss[u][0..m); when
+ * both coordinates are in range, dest[is[u]][js[u]][c] = op(that, vss[u][c])
+ * for every c.  js == NULL (then H1 must be 1) is the one-dimensional
+ * `reduce_by_index dest (map2 op) (replicate m ne) is vss` (a HistOp with an
+ * operator shape, SegHist.hs:1057-1136; tests/hist/array.fut); m == 1 with js
+ * is `reduce_by_index_2d` (prelude/soacs.fut:149-150; tests/hist/hist2d.fut).
+ * is and js have the same width (is64).  t is FA_I32, FA_I64, FA_F32 or FA_F64. */
+size_t fa_seghist_shaped_scratch_bytes(fa_dtype t, int is64, int64_t n_updates,
+                                       int64_t H0, int64_t H1, int64_t m);
+int fa_seghist_shaped(fa_stream_t stream, fa_dtype t, fa_op op,
+                      const void *is, const void *js, int is64, const void *vss,
+                      int64_t n_updates, void *dest, int64_t H0, int64_t H1, int64_t m,
+                      void *scratch, size_t scratch_bytes);
+
 /* -------------------------------------------------------------- radix sort
  * Stable LSD radix sort with 8-bit digits: per pass a digit histogram
  * (SegHist), an exclusive scan of the counts (SegScan) and a ranked scatter

@@ -30,6 +30,10 @@
  *                                   -- tests/hist/segmented.fut
  *   entry rbi_OP_T (dest: *[]T) (is: []i32) (vs: []T) : []T =
  *     reduce_by_index dest OP NE (map i64.i32 is) vs
+ *   entry rbi_vec_OP_T [m] (dest: *[][m]T) (is: []i64) (vss: [][m]T) : [][m]T =
+ *     reduce_by_index dest (map2 OP) (replicate m NE) is vss
+ *   entry rbi_2d_OP_T (dest: *[][]T) (is: []i64) (js: []i64) (vs: []T) : [][]T =
+ *     reduce_by_index_2d dest OP NE (zip is js) vs
  *   entry bmm_f32 (A: [][][]f32) (B: [][][]f32) : [][][]f32 =
  *     map2 (\a b -> map (\ar -> map (\bc -> reduce (+) 0 (map2 (*) ar bc))
  *                                   (transpose b)) a) A B
@@ -258,6 +262,17 @@ FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
                                        struct futhark_##T##_2d **out0, const int64_t in0,     \
                                        const struct futhark_i32_2d *in1,                      \
                                        const struct futhark_##T##_2d *in2);                   \
+  int futhark_entry_rbi_vec_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_2d **out0,                        \
+                                       const struct futhark_##T##_2d *in0,                    \
+                                       const struct futhark_i64_1d *in1,                      \
+                                       const struct futhark_##T##_2d *in2);                   \
+  int futhark_entry_rbi_2d_##OP##_##T(struct futhark_context *ctx,                            \
+                                      struct futhark_##T##_2d **out0,                         \
+                                      const struct futhark_##T##_2d *in0,                     \
+                                      const struct futhark_i64_1d *in1,                       \
+                                      const struct futhark_i64_1d *in2,                       \
+                                      const struct futhark_##T##_1d *in3);                    \
   FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)
 
 #define FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)                                               \

@@ -141,6 +141,31 @@ for _t in ("i8", "u8", "i16", "u16", "u32", "u64"):
                     ("and", _t): _ii.max if _ii.min == 0 else -1, ("or", _t): 0, ("xor", _t): 0})
 
 
+def rbi_vec(op: str, t: str, dest, is_, vss):
+    """reduce_by_index dest (map2 op) (replicate m ne) is vss on a copy of dest ([H][m])."""
+    _, dt = _CT[t]
+    out = np.array(dest, dtype=dt, copy=True, order="C")
+    is_ = _arr(is_, np.int64)
+    vss = _arr(vss, dt).reshape(is_.size, out.shape[1])
+    fn = getattr(lib(), f"orc_rbi_vec_{op}_{t}_lit")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64]
+    fn(_p(out), out.shape[0], out.shape[1], _p(is_), _p(vss), is_.size)
+    return out
+
+
+def rbi_2d(op: str, t: str, dest, is_, js, vs):
+    """reduce_by_index_2d dest op ne (zip is js) vs on a copy of dest ([H0][H1])."""
+    _, dt = _CT[t]
+    out = np.array(dest, dtype=dt, copy=True, order="C")
+    is_, js, vs = _arr(is_, np.int64), _arr(js, np.int64), _arr(vs, dt)
+    fn = getattr(lib(), f"orc_rbi_2d_{op}_{t}_lit")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64]
+    fn(_p(out), out.shape[0], out.shape[1], _p(is_), _p(js), _p(vs), is_.size)
+    return out
+
+
 def hist(op: str, t: str, k: int, is_, vs, variant: str = "lit"):
     _, dt = _CT[t]
     return rbi(op, t, np.full(k, NEUTRAL[(op, t)], dtype=dt), is_, vs, variant)

@@ -134,6 +134,26 @@ static inline double min_f64(double a, double b) { return fmin(a, b); }
   void orc_segreduce_##OP##_##S##_lit(const T *xss, int64_t m, int64_t k, T *out) {            \
     for (int64_t i = 0; i < m; i++) out[i] = orc_reduce_##OP##_##S##_lit(xss + i * k, k);      \
   }                                                                                            \
+  /* reduce_by_index dest (map2 OP) (replicate m NE) is vss: dest [H][m], vss [n][m]; the     \
+   * same in-order read-modify-write, a whole vector per update */                             \
+  void orc_rbi_vec_##OP##_##S##_lit(T *dest, int64_t H, int64_t m, const int64_t *is,          \
+                                    const T *vss, int64_t n) {                                 \
+    for (int64_t i = 0; i < n; i++) {                                                          \
+      const int64_t b = is[i];                                                                 \
+      if (b < 0 || b >= H) continue;                                                           \
+      for (int64_t c = 0; c < m; c++) dest[b * m + c] = OP##_##S(dest[b * m + c], vss[i * m + c]); \
+    }                                                                                          \
+  }                                                                                            \
+  /* reduce_by_index_2d dest OP NE (zip is js) vs (prelude/soacs.fut:149-150): an update     \
+   * is dropped unless both coordinates are in range */                                        \
+  void orc_rbi_2d_##OP##_##S##_lit(T *dest, int64_t H0, int64_t H1, const int64_t *is,         \
+                                   const int64_t *js, const T *vs, int64_t n) {                \
+    for (int64_t i = 0; i < n; i++) {                                                          \
+      if (is[i] < 0 || is[i] >= H0 || js[i] < 0 || js[i] >= H1) continue;                      \
+      T *cell = dest + is[i] * H1 + js[i];                                                     \
+      *cell = OP##_##S(*cell, vs[i]);                                                          \
+    }                                                                                          \
+  }                                                                                            \
   /* reduce (map2 OP) (replicate k NE) xss, rows folded in order */                            \
   void orc_vecreduce_##OP##_##S##_lit(const T *xss, int64_t n, int64_t k, T *out) {            \
     for (int64_t j = 0; j < k; j++) out[j] = NE_##OP##_##S;                                    \

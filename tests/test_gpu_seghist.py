@@ -209,3 +209,85 @@ def test_i64_indices_through_the_kernel_library(ctx):
             assert np.array_equal(dest.values(), oracle.hist(opname, t, H, is32, vals)), (t, opname, H)
             for h in (d_is, d_vs, dest, scratch):
                 h.free()
+
+
+def test_hist_with_vector_operator_goldens_and_shapes(ctx, goldens):
+    """reduce_by_index dest (map2 op) (replicate m ne) is vss: tests/hist/{array,equiv}.fut, then
+    vectors shorter and longer than what a thread loads at once, indices out of range, bins that
+    fit one LDS range, several, and none (flattened indices and the partition path)."""
+    for name in ("hist_array", "hist_equiv"):
+        for c in goldens[name]["cases"]:
+            d = ctx.new("i32_2d", np.array(c["dest"], np.int32))
+            i = ctx.new("i64_1d", np.array(c["is"], np.int64))
+            v = ctx.new("i32_2d", np.array(c["vss"], np.int32))
+            out = ctx.call("rbi_vec_add_i32", ["i32_2d"], d, i, v)
+            assert out.values().tolist() == c["out"]
+            for h in (out, d, i, v):
+                h.free()
+    rng = np.random.default_rng(3)
+    for t, op, H, m, n in [("i32", "add", 5, 1, 1000), ("i32", "add", 100, 3, 5000),
+                           ("i64", "max", 33, 4, 4099), ("i32", "xor", 1000, 7, 30001),
+                           ("f64", "min", 50, 16, 777), ("i32", "add", 3000, 100, 20000),
+                           ("i32", "add", 1 << 15, 64, 50000), ("i64", "add", 2, 1000, 300),
+                           ("i32", "min", 0, 4, 10), ("i32", "add", 4, 6, 0)]:
+        dt = {"i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        is_ = rng.integers(-3, H + 3, n).astype(np.int64)
+        vss = (rng.standard_normal((n, m)) if t == "f64" else rng.integers(-1000, 1000, (n, m))).astype(dt)
+        dest = (rng.standard_normal((H, m)) if t == "f64" else rng.integers(-5, 5, (H, m))).astype(dt)
+        d, i, v = ctx.new(f"{t}_2d", dest), ctx.new("i64_1d", is_), ctx.new(f"{t}_2d", vss)
+        out = ctx.call(f"rbi_vec_{op}_{t}", [f"{t}_2d"], d, i, v)
+        assert out.shape == (H, m)
+        assert np.array_equal(out.values(), oracle.rbi_vec(op, t, dest, is_, vss)), (t, op, H, m, n)
+        for h in (out, d, i, v):
+            h.free()
+    # f32 sums: tolerance against the f64 accumulation
+    H, m, n = 64, 8, 100000
+    is_ = rng.integers(0, H, n).astype(np.int64)
+    vss = rng.random((n, m), dtype=np.float32)
+    d, i, v = ctx.new("f32_2d", np.zeros((H, m), np.float32)), ctx.new("i64_1d", is_), ctx.new("f32_2d", vss)
+    out = ctx.call("rbi_vec_add_f32", ["f32_2d"], d, i, v)
+    want = np.zeros((H, m))
+    np.add.at(want, is_, vss.astype(np.float64))
+    assert np.allclose(out.values(), want, rtol=1e-5, atol=0)
+    w = ctx.new("f32_2d", np.zeros((n, m + 1), np.float32))
+    with pytest.raises(Exception, match="invalid sizes"):
+        ctx.call("rbi_vec_add_f32", ["f32_2d"], d, i, w)
+    for h in (out, d, i, v, w):
+        h.free()
+
+
+def test_hist_with_2d_indices_goldens_and_shapes(ctx, goldens):
+    """reduce_by_index_2d: tests/hist/hist2d.fut (an update is dropped when either coordinate is
+    outside), then random cases of both sizes of bin space."""
+    for c in goldens["hist2d"]["cases"]:
+        d = ctx.new("i32_2d", np.array(c["dest"], np.int32))
+        i, j = ctx.new("i64_1d", np.array(c["is"], np.int64)), ctx.new("i64_1d", np.array(c["js"], np.int64))
+        v = ctx.new("i32_1d", np.array(c["vs"], np.int32))
+        out = ctx.call("rbi_2d_add_i32", ["i32_2d"], d, i, j, v)
+        assert out.values().tolist() == c["out"]
+        for h in (out, d, i, j, v):
+            h.free()
+    rng = np.random.default_rng(4)
+    for t, op, H0, H1, n in [("i32", "add", 10, 10, 5000), ("i64", "max", 300, 7, 100003),
+                             ("i32", "or", 1000, 1000, 200000), ("f64", "max", 3, 50000, 99999),
+                             ("i32", "add", 3000, 3000, 1 << 20), ("i32", "add", 0, 5, 100)]:
+        dt = {"i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        is_ = rng.integers(-2, H0 + 2, n).astype(np.int64)
+        js = rng.integers(-2, H1 + 2, n).astype(np.int64)
+        vs = (rng.standard_normal(n) if t == "f64" else rng.integers(-1000, 1000, n)).astype(dt)
+        dest = (rng.standard_normal((H0, H1)) if t == "f64" else rng.integers(-5, 5, (H0, H1))).astype(dt)
+        d, i, j, v = (ctx.new(f"{t}_2d", dest), ctx.new("i64_1d", is_), ctx.new("i64_1d", js),
+                      ctx.new(f"{t}_1d", vs))
+        out = ctx.call(f"rbi_2d_{op}_{t}", [f"{t}_2d"], d, i, j, v)
+        assert np.array_equal(out.values(), oracle.rbi_2d(op, t, dest, is_, js, vs)), (t, op, H0, H1, n)
+        for h in (out, d, i, j, v):
+            h.free()
+    # the sparse 2-D histogram of tests/hist/large2d.fut, 100 x 100 bins, k = 10^6: closed form modulo 2^32
+    n_, m_, k = 100, 100, 1000000
+    it = np.arange(k, dtype=np.int64)
+    d = ctx.new("i32_2d", np.zeros((m_, n_), np.int32))
+    i, j, v = ctx.new("i64_1d", it % n_), ctx.new("i64_1d", it % m_), ctx.new("i32_1d", it.astype(np.int32))
+    out = ctx.call("rbi_2d_add_i32", ["i32_2d"], d, i, j, v)
+    assert int(out.values().sum(dtype=np.int64)) % 2**32 == (k * (k - 1) // 2) % 2**32  # bins wrap
+    for h in (out, d, i, j, v):
+        h.free()

@@ -303,3 +303,38 @@ def test_vectorised_reduce_is_a_reduce_per_column():
                               oracle.segreduce("add", "f32", np.ascontiguousarray(xf.T)))
         np.testing.assert_allclose(oracle.vecreduce("add", "f32", xf, "f64acc"),
                                    xf.astype(np.float64).sum(axis=0), rtol=1e-6, atol=1e-6)
+
+
+def test_hist_with_vector_operator_and_2d_indices_goldens(goldens):
+    # tests/hist/{array,array_novec,equiv,hist2d}.fut; tests/hist/lor.fut with bool as a byte
+    for name in ("hist_array", "hist_equiv"):
+        for c in goldens[name]["cases"]:
+            assert oracle.rbi_vec("add", "i32", c["dest"], c["is"], c["vss"]).tolist() == c["out"]
+    for c in goldens["hist2d"]["cases"]:
+        assert oracle.rbi_2d("add", "i32", c["dest"], c["is"], c["js"], c["vs"]).tolist() == c["out"]
+    for c in goldens["hist_lor"]["cases"]:
+        assert oracle.hist("or", "u8", c["n"], c["is"], c["vs"]).tolist() == c["out"]
+
+
+def test_shaped_hist_against_numpy():
+    """The vector form is a plain histogram over bins b * m + c, the 2-D form one over
+    i * H1 + j with updates dropped when either coordinate is outside (numpy's unbuffered
+    ufunc.at does the in-order read-modify-write)."""
+    rng = np.random.default_rng(11)
+    H, m, n = 7, 5, 400
+    is_ = rng.integers(-2, H + 2, n)
+    vss = rng.integers(-2**31, 2**31, (n, m), dtype=np.int64).astype(np.int32)
+    dest = rng.integers(-100, 100, (H, m)).astype(np.int32)
+    ok = (is_ >= 0) & (is_ < H)
+    for op, f in (("add", np.add), ("max", np.maximum), ("min", np.minimum), ("xor", np.bitwise_xor)):
+        want = dest.copy()
+        f.at(want, is_[ok], vss[ok])
+        assert np.array_equal(oracle.rbi_vec(op, "i32", dest, is_, vss), want)
+    H0, H1 = 6, 9
+    is_, js = rng.integers(-1, H0 + 1, n), rng.integers(-1, H1 + 1, n)
+    vs = rng.standard_normal(n)
+    dest = rng.standard_normal((H0, H1))
+    ok = (is_ >= 0) & (is_ < H0) & (js >= 0) & (js < H1)
+    want = dest.copy()
+    np.add.at(want, (is_[ok], js[ok]), vs[ok])
+    assert np.array_equal(oracle.rbi_2d("add", "f64", dest, is_, js, vs), want)
