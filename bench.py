@@ -290,8 +290,8 @@ def run_via_server(name: str, steps: int, warmup: int):
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same
 # counters on a 256 MiB copy); the runs and their commands are in profiles/<kernel>_<workload>.txt.
 MEASURED_TRAFFIC_BYTES = {
-    "segscan_add_f32_2p26": 606.0e6,
-    "scan_add_f32_2p26": 539.3e6,
+    "segscan_add_f32_2p26": 605.3e6,
+    "scan_add_f32_2p26": 538.6e6,
     "reduce_add_f32_2p26": 268.5e6,
     "segred_add_f32_2p26": 283.3e6,
     "hist_add_i32_H256_uniform_2p27": 1074.2e6,
@@ -300,6 +300,10 @@ MEASURED_TRAFFIC_BYTES = {
     "sort_u32_2p26": 4088.4e6,
     "hist_max_f32_H256_uniform_2p27": 1074.5e6,
     "transpose_f32_8192x8192": 537.6e6,
+    "vecreduce_add_f32_65536x1024": 269.5e6,
+    "hist_add_f32_H256_uniform_2p27": 1074.2e6,
+    "rbivec_add_i32_H256x16_2p23": 612.4e6,
+    "rbi2d_add_i32_16x16_2p27": 2911.9e6,
 }
 
 
