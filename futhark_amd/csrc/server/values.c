@@ -481,7 +481,20 @@ int fv_read_value(FILE *f, const struct fv_primtype *t, int rank, int64_t *shape
 
 int fv_end_of_input(FILE *f) {
   /* blanks and `--` comments may follow the last value (end_of_input,
-   * rts/c/values.h:713-722, reads a token) */
-  struct text_parser p = {f, {0}, 0};
-  return *peek_token(&p) != 0;
+   * rts/c/values.h:713-722); whatever else is found stays in the stream */
+  for (;;) {
+    int c = getc(f);
+    if (c == EOF) return 0;
+    if (isspace(c)) continue;
+    if (c == '-') {
+      int c2 = getc(f);
+      if (c2 == '-') {
+        while (c2 != EOF && c2 != '\n') c2 = getc(f);
+        continue;
+      }
+      if (c2 != EOF) ungetc(c2, f);
+    }
+    ungetc(c, f);
+    return 1;
+  }
 }

@@ -57,7 +57,8 @@ int fv_read_text(FILE *f, const struct fv_primtype *expect, int rank, int64_t *s
 int fv_read_value(FILE *f, const struct fv_primtype *expect, int rank, int64_t *shape,
                   void **data, char *err, size_t errlen);
 
-/* 0 if only blanks and `--` comments remain before end of file. */
+/* 0 if only blanks and `--` comments remain before end of file; otherwise
+ * nonzero, and the next value can still be read. */
 int fv_end_of_input(FILE *f);
 
 #ifdef __cplusplus

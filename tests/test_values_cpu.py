@@ -198,3 +198,28 @@ def test_text_round_trip_of_every_type_and_rank(tmp_path, name):
         fv.write_binary(p, [a])
         (either,) = fv.read_values(p, [(name, len(shape))])    # ... and binary
         assert np.array_equal(either, a, equal_nan=name[0] == "f")
+
+
+def test_end_of_input_check_leaves_the_next_value_in_the_stream(tmp_path):
+    """Asking whether the input has ended must not eat what follows: blanks and comments are
+    skipped, a value (also one starting with a minus sign) is still there for the next read."""
+    import ctypes as C
+    L = fv._get()
+    p = tmp_path / "in.txt"
+    p.write_text("  -- a comment\n -7i32 -- another\n[1, 2] -- last\n")
+    f = fv._open(p, b"rb")
+    try:
+        got = []
+        for name, rank in (("i32", 0), ("i32", 1)):
+            assert L.v.fv_end_of_input(f) != 0
+            assert L.v.fv_end_of_input(f) != 0   # asking twice changes nothing
+            shape, data, err = (C.c_int64 * fv.MAX_RANK)(), C.c_void_p(), C.create_string_buffer(256)
+            rc = L.v.fv_read_value(f, L.v.fv_primtype(name.encode()), rank, shape, C.byref(data), err, len(err))
+            assert rc == 0, err.value
+            n = shape[0] if rank else 1
+            got.append(np.frombuffer(C.string_at(data, 4 * n), np.int32).tolist())
+            L.c.free(data)
+        assert got == [[-7], [1, 2]]
+        assert L.v.fv_end_of_input(f) == 0
+    finally:
+        L.c.fclose(f)
