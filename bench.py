@@ -54,6 +54,9 @@ def make_workload(name: str, ctx):
             w["kernel"] = "segscan"
             if t in ("f32", "i64"):
                 w["cpu"] = lambda out=np.empty_like(xs): oracle.mc_segscan(t, flags, xs, op, out=out)
+                # the sequential `futhark c` fold (the oracle proper) on the first 2^24 elements
+                w["cpu_seq"] = (lambda: oracle.segscan(op, t, flags[:1 << 24], xs[:1 << 24]),
+                                (1 << 24) * (2 * es + 1))
         else:
             o, l = ctx.new("i64_1d", offsets), ctx.new("i64_1d", lens)
 
@@ -367,6 +370,8 @@ def main() -> None:
     report = json.loads(ctx.report())
     durs = [e["duration"] for e in report["events"] if e["name"] == w["kernel"]]
     kernel_us = float(np.mean(durs)) if durs else float("nan")
+    kernel_us_min = float(np.min(durs)) if durs else float("nan")
+    kernel_us_ci95 = float(1.96 * np.std(durs, ddof=1) / np.sqrt(len(durs))) if len(durs) > 1 else 0.0
 
     if w["bound"] == "hbm":
         work, unit, peak = w["bytes"], "GB/s", HBM_PEAK_GBS
@@ -393,6 +398,14 @@ def main() -> None:
                "cores": oracle.mc_threads(), "kind": "port",
                "sample": f"{reps} passes of the full workload with the futhark-multicore-style "
                          f"restatement in oracle/multicore.c ({t_cpu:.1f} s)"}
+        if "cpu_seq" in w:
+            fn, nbytes = w["cpu_seq"]
+            fn()
+            t_s = time.perf_counter()
+            fn()
+            cpu["single_thread"] = {"value": round(nbytes / (time.perf_counter() - t_s) / 1e9, 3),
+                                    "unit": "GB/s", "sample": "one pass of oracle/oracle.c (the "
+                                    "sequential futhark c fold) over the first 2^24 elements"}
 
     server = None
     if args.via_server:
@@ -422,7 +435,9 @@ def main() -> None:
         "roofline": {"bound": w["bound"], "achieved": round(achieved, 3), "peak": peak,
                      "unit": unit, "frac": round(achieved / peak, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "kernel": w["kernel"], "kernel_us": round(kernel_us, 3)},
+                     "kernel": w["kernel"], "kernel_us": round(kernel_us, 3),
+                     "kernel_us_min": round(kernel_us_min, 3),
+                     "kernel_us_ci95": round(kernel_us_ci95, 3)},
         "cpu_baseline": cpu,
     }
     if server is not None:
