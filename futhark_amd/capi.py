@@ -126,6 +126,9 @@ class Segops:
                 getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
         for e in ("bmm_f32", "bmm_f16", "bmm_bf16", "matmul_f32"):
             getattr(L, f"futhark_entry_{e}").argtypes = [vp, pp, vp, vp]
+        L.futhark_entry_scan_compose_i32.argtypes = [vp, pp, vp]
+        L.futhark_entry_exscan_compose_i32.argtypes = [vp, pp, vp]
+        L.futhark_entry_segscan_compose_i32.argtypes = [vp, pp, vp, vp]
         L.futhark_entry_radix_sort_u32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u64.argtypes = [vp, pp, vp]
         for name, (k, v) in OPAQUE_PAIRS.items():

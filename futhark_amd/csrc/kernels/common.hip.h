@@ -102,6 +102,20 @@ template <class T> struct OpXor {
   static __host__ __device__ __forceinline__ T apply(T a, T b) { return a ^ b; }
 };
 
+// x -> a*x + b modulo 2^32.  compose(f, g) is "f, then g": associative, not
+// commutative, so a scan that swaps or reorders operands gives wrong results.
+struct AffineI32 {
+  int32_t a, b;
+};
+struct OpCompose {
+  static constexpr bool commutative = false;
+  static __host__ __device__ __forceinline__ AffineI32 identity() { return AffineI32{1, 0}; }
+  static __host__ __device__ __forceinline__ AffineI32 apply(AffineI32 f, AffineI32 g) {
+    return AffineI32{(int32_t)((uint32_t)f.a * (uint32_t)g.a),
+                     (int32_t)((uint32_t)g.a * (uint32_t)f.b + (uint32_t)g.b)};
+  }
+};
+
 // ------------------------------------------------------- bit reinterpretation
 
 template <class To, class From>

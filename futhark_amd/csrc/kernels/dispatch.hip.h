@@ -67,7 +67,7 @@ using namespace fa;
 static inline size_t dtype_size(fa_dtype t) {
   switch (t) {
     case FA_I32: case FA_U32: case FA_F32: return 4;
-    case FA_I64: case FA_U64: case FA_F64: return 8;
+    case FA_I64: case FA_U64: case FA_F64: case FA_I32X2: return 8;
     case FA_F16: case FA_BF16: case FA_I16: case FA_U16: return 2;
     case FA_I8: case FA_U8: return 1;
     default: return 0;

@@ -475,6 +475,10 @@ extern "C" int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op, const void *
     return FA_EINVAL;
   if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
   hipStream_t s = (hipStream_t)stream;
+  if (t == FA_I32X2)
+    return op == FA_COMPOSE ? launch_scan<AffineI32, OpCompose>(s, xs, flags, (int64_t)0, n, exclusive,
+                                                                out, scratch, scratch_bytes, epoch)
+                            : FA_ENOTSUP;
   FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xs, flags, (int64_t)0, n, exclusive, out, scratch,
                       scratch_bytes, epoch);
 }
@@ -488,6 +492,11 @@ extern "C" int fa_segscan_rows(fa_stream_t stream, fa_dtype t, fa_op op, const v
   if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
   if (n == 0) return 0;
   hipStream_t s = (hipStream_t)stream;
+  if (t == FA_I32X2)
+    return op == FA_COMPOSE
+               ? launch_scan<AffineI32, OpCompose>(s, xss, (const uint8_t *)nullptr, k, n, exclusive,
+                                                   out, scratch, scratch_bytes, epoch)
+               : FA_ENOTSUP;
   FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xss, (const uint8_t *)nullptr, k, n, exclusive, out,
                       scratch, scratch_bytes, epoch);
 }

@@ -256,11 +256,13 @@ static int do_scan(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
                    const struct fut_array *in, int exclusive, const char *entry) {
   const int64_t n = in->shape[0];
   if (flags != NULL && flags->shape[0] != n) return bad_sizes(ctx, entry);
+  const int pairs = t == FA_I32X2;  /* [n][2]i32, one (a, b) per row */
+  if (pairs && in->shape[1] != 2) return bad_sizes(ctx, entry);
   uint32_t epoch = 0;
   const size_t sbytes = fa_segscan_scratch_bytes(t, n);
   void *scratch = rts_scan_scratch(ctx, sbytes, &epoch);
   if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
-  struct fut_array *res = out_array(ctx, n * (int64_t)es, 1, &n, "scan.out");
+  struct fut_array *res = out_array(ctx, n * (int64_t)es, pairs ? 2 : 1, in->shape, "scan.out");
   if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
   struct rts_event *ev = rts_kernel_begin(
       ctx, "segscan", rts_msgprintf("{\"n\":%lld,\"segmented\":%d,\"exclusive\":%d}",
@@ -673,6 +675,33 @@ static int do_rbi_shaped(struct futhark_context *ctx, fa_dtype t, fa_op op, size
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }
+
+/* Scans of affine maps x -> a*x + b (mod 2^32) under composition: rows (a, b) of [n][2]i32. */
+int futhark_entry_scan_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                   const struct futhark_i32_2d *in0) {
+  ENTER(ctx);
+  int ret = do_scan(ctx, FA_I32X2, FA_COMPOSE, 8, (struct fut_array **)out0, NULL, &in0->a, 0,
+                    "scan_compose_i32");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_exscan_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                     const struct futhark_i32_2d *in0) {
+  ENTER(ctx);
+  int ret = do_scan(ctx, FA_I32X2, FA_COMPOSE, 8, (struct fut_array **)out0, NULL, &in0->a, 1,
+                    "exscan_compose_i32");
+  LEAVE(ctx);
+  return ret;
+}
+int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                      const struct futhark_u8_1d *in0,
+                                      const struct futhark_i32_2d *in1) {
+  ENTER(ctx);
+  int ret = do_scan(ctx, FA_I32X2, FA_COMPOSE, 8, (struct fut_array **)out0, &in0->a, &in1->a, 0,
+                    "segscan_compose_i32");
+  LEAVE(ctx);
+  return ret;
+}
 
 #define DEFINE_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(DEFINE_SEGOP_ENTRIES, T, CT)
 FUTHARK_FOR_EACH_NUM_TYPE(DEFINE_FOR_TYPE)

@@ -225,6 +225,16 @@ static int e_bmm_f32(struct futhark_context *c, struct value *o, struct value **
 static int e_bmm_f16(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_bmm_f16(c, (struct futhark_f32_3d **)&o->u.arr, ARRP(i[0]), ARRP(i[1]));
 }
+static int e_scan_compose_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_scan_compose_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_exscan_compose_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_exscan_compose_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_segscan_compose_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_segscan_compose_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]),
+                                           ARRP(i[1]));
+}
 static int e_bmm_bf16(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_bmm_bf16(c, (struct futhark_f32_3d **)&o->u.arr, ARRP(i[0]), ARRP(i[1]));
 }
@@ -305,6 +315,10 @@ static const struct entry entries[] = {
     FUTHARK_FOR_EACH_OP(HIST_ENTRY_ROWS, f16, uint16_t)
     {"bmm_f32", e_bmm_f32, "[][][]f32", 1, 2, {"[][][]f32", "[][][]f32"}, {0}, {MATMUL_PARAM, NULL}},
     {"bmm_f16", e_bmm_f16, "[][][]f32", 1, 2, {"[][][]f16", "[][][]f16"}, {0}, {MATMUL_PARAM, NULL}},
+    {"scan_compose_i32", e_scan_compose_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
+    {"exscan_compose_i32", e_exscan_compose_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
+    {"segscan_compose_i32", e_segscan_compose_i32, "[][]i32", 1, 2, {"[]u8", "[][]i32"}, {0},
+     {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {MATMUL_PARAM, NULL}},
     {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {MATMUL_PARAM, NULL}},
     {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {NULL}},

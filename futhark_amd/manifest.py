@@ -70,6 +70,9 @@ def entry_points() -> dict:
     eps += [
         _entry("bmm_f32", "[][][]f32", [("A", "[][][]f32"), ("B", "[][][]f32")], [MATMUL_PARAM]),
         _entry("bmm_f16", "[][][]f32", [("A", "[][][]f16"), ("B", "[][][]f16")], [MATMUL_PARAM]),
+        _entry("scan_compose_i32", "[][]i32", [("abs", "[][]i32")]),
+        _entry("exscan_compose_i32", "[][]i32", [("abs", "[][]i32")]),
+        _entry("segscan_compose_i32", "[][]i32", [("flags", "[]u8"), ("abs", "[][]i32")]),
         _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")], [MATMUL_PARAM]),
         _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")], [MATMUL_PARAM]),
         _entry("radix_sort_u32", "[]u32", [("keys", "[]u32")]),

@@ -48,6 +48,9 @@ typedef enum {
   FA_U8 = 9,
   FA_I16 = 10,
   FA_U16 = 11,
+  /* A pair of i32, (a, b), standing for the map x -> a*x + b modulo 2^32
+   * (8 bytes, a first): the element type of FA_COMPOSE, scans only. */
+  FA_I32X2 = 12,
   FA_DTYPE_COUNT
 } fa_dtype;
 
@@ -56,8 +59,16 @@ typedef enum {
  * Semantics are those of rts/c/scalar.h: two's-complement wrap-around add
  * (scalar.h:29-30), smax/smin (scalar.h:488-503), fmaxf/fminf, i.e. NaN-ignoring
  * (scalar.h:931-934). */
-/* FA_AND, FA_OR, FA_XOR: integer types only (neutral elements -1, 0, 0). */
-typedef enum { FA_ADD = 0, FA_MAX = 1, FA_MIN = 2, FA_AND = 3, FA_OR = 4, FA_XOR = 5, FA_OP_COUNT } fa_op;
+/* FA_AND, FA_OR, FA_XOR: integer types only (neutral elements -1, 0, 0).
+ * FA_COMPOSE: FA_I32X2 only, (a1, b1) then (a2, b2) = (a1*a2, a2*b1 + b2) with
+ * wrap-around arithmetic, neutral (1, 0): composition of affine maps, the
+ * operator of linear recurrences.  Associative and NOT commutative; it exists
+ * so that the order in which the scans combine their operands is observable
+ * (the reference's single-pass scan keeps operand order, so non-commutative
+ * operators are legal there: SegScan/SinglePass.hs:738-746). */
+typedef enum {
+  FA_ADD = 0, FA_MAX = 1, FA_MIN = 2, FA_AND = 3, FA_OR = 4, FA_XOR = 5, FA_COMPOSE = 6, FA_OP_COUNT
+} fa_op;
 
 #define FA_EINVAL (-1)   /* bad argument (null pointer, negative size, ...) */
 #define FA_ENOTSUP (-2)  /* dtype/op combination not built */

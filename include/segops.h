@@ -309,6 +309,18 @@ int futhark_entry_bmm_f32(struct futhark_context *ctx, struct futhark_f32_3d **o
                           const struct futhark_f32_3d *in0, const struct futhark_f32_3d *in1);
 int futhark_entry_bmm_f16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
                           const struct futhark_f16_3d *in0, const struct futhark_f16_3d *in1);
+/* Scans with a non-commutative operator: composition of affine maps modulo 2^32,
+ *   def compose (a1: i32, b1: i32) (a2: i32, b2: i32) = (a1 * a2, a2 * b1 + b2)
+ *   entry scan_compose_i32 (abs: [][2]i32) : [][2]i32 =
+ *     scan compose (1, 0) (map (\r -> (r[0], r[1])) abs) |> map (\(a, b) -> [a, b])
+ * exscan_compose_i32 and segscan_compose_i32 (flags: []u8) likewise. */
+int futhark_entry_scan_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                   const struct futhark_i32_2d *in0);
+int futhark_entry_exscan_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                     const struct futhark_i32_2d *in0);
+int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                      const struct futhark_u8_1d *in0,
+                                      const struct futhark_i32_2d *in1);
 int futhark_entry_bmm_bf16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
                            const struct futhark_u16_3d *in0, const struct futhark_u16_3d *in1);
 int futhark_entry_matmul_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,

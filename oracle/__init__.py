@@ -141,6 +141,18 @@ for _t in ("i8", "u8", "i16", "u16", "u32", "u64"):
                     ("and", _t): _ii.max if _ii.min == 0 else -1, ("or", _t): 0, ("xor", _t): 0})
 
 
+def scan_compose_i32(abs_, flags=None, exclusive: bool = False):
+    """scan / exscan / segmented scan of affine maps (a, b) : [n][2]i32 under composition."""
+    abs_ = _arr(abs_, np.int32).reshape(-1, 2)
+    out = np.empty_like(abs_)
+    f = None if flags is None else _arr(flags, np.uint8)
+    fn = lib().orc_scan_compose_i32_lit
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]
+    fn(None if f is None else _p(f), _p(abs_), abs_.shape[0], int(exclusive), _p(out))
+    return out
+
+
 def rbi_vec(op: str, t: str, dest, is_, vss):
     """reduce_by_index dest (map2 op) (replicate m ne) is vss on a copy of dest ([H][m])."""
     _, dt = _CT[t]

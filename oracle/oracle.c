@@ -178,6 +178,24 @@ DEFINE_LIT_BITOPS(i64, int64_t)
 DEFINE_LIT_ALL_OPS(f32, float)
 DEFINE_LIT_ALL_OPS(f64, double)
 
+/* Scans of affine maps x -> a*x + b modulo 2^32 under composition,
+ *   (a1, b1) then (a2, b2) = (a1*a2, a2*b1 + b2), neutral (1, 0):
+ * an associative operator that does not commute.  abs and out are [n][2].
+ * The same left-to-right loops as the scans above (FirstOrderTransform.hs:613-656;
+ * flag operator Pass/Flatten/Builtins.hs:374-393). */
+void orc_scan_compose_i32_lit(const uint8_t *flags, const int32_t *abs, int64_t n, int exclusive,
+                              int32_t *out) {
+  uint32_t a = 1, b = 0;
+  for (int64_t i = 0; i < n; i++) {
+    const uint32_t xa = (uint32_t)abs[2 * i], xb = (uint32_t)abs[2 * i + 1];
+    if (flags != NULL && flags[i] != 0) { a = 1; b = 0; }
+    if (exclusive) { out[2 * i] = (int32_t)a; out[2 * i + 1] = (int32_t)b; }
+    const uint32_t na = a * xa, nb = xa * b + xb;
+    a = na; b = nb;
+    if (!exclusive) { out[2 * i] = (int32_t)a; out[2 * i + 1] = (int32_t)b; }
+  }
+}
+
 /* hist / reduce_by_index alone for the other integer types */
 #define DEFINE_RBI(OP, S, T)                                                                   \
   void orc_rbi_##OP##_##S##_lit(T *dest, int64_t H, const int32_t *is, const T *vs,            \

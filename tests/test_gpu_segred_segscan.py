@@ -328,3 +328,34 @@ def test_segscan_long_look_back_chains(ctx, t):
             out.free()
         f.free()
     a.free()
+
+
+def test_scan_with_a_non_commutative_operator(ctx):
+    """Composition of affine maps modulo 2^32 (associative, not commutative): every place where
+    the kernel combines two partial results - inside a thread, across lanes, rows, waves and the
+    look-back over tiles - must keep the operands in order, or some element differs.  Sizes from
+    one element to many tiles, ragged ends, segment starts dense and hundreds of tiles apart."""
+    rng = np.random.default_rng(17)
+    tile = 1024 * 8 * 2
+    for n in [0, 1, 2, 63, 64, 65, 4097, tile - 1, tile, tile + 1, 5 * tile + 3, 700 * tile + 11]:
+        abs_ = rng.integers(-2**31, 2**31, (n, 2), dtype=np.int64).astype(np.int32)
+        a = ctx.new("i32_2d", abs_)
+        for excl in (False, True):
+            out = ctx.call(("exscan" if excl else "scan") + "_compose_i32", ["i32_2d"], a)
+            assert out.shape == (n, 2)
+            assert np.array_equal(out.values(), oracle.scan_compose_i32(abs_, None, excl)), (n, excl)
+            out.free()
+        for every in (3, 1000, 300 * tile):
+            flags = np.zeros(n, np.uint8)
+            flags[::every] = 1
+            if n > 10:
+                flags[rng.integers(0, n, 3)] = 1
+            f = ctx.new("u8_1d", flags)
+            out = ctx.call("segscan_compose_i32", ["i32_2d"], f, a)
+            assert np.array_equal(out.values(), oracle.scan_compose_i32(abs_, flags)), (n, every)
+            out.free(); f.free()
+        a.free()
+    bad = ctx.new("i32_2d", np.zeros((4, 3), np.int32))
+    with pytest.raises(Exception, match="invalid sizes"):
+        ctx.call("scan_compose_i32", ["i32_2d"], bad)
+    bad.free()

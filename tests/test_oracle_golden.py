@@ -338,3 +338,27 @@ def test_shaped_hist_against_numpy():
     want = dest.copy()
     np.add.at(want, (is_[ok], js[ok]), vs[ok])
     assert np.array_equal(oracle.rbi_2d("add", "f64", dest, is_, js, vs), want)
+
+
+def test_affine_composition_scan_is_the_iterated_map():
+    """Element i of the scan, applied to x, must give what applying the maps 0..i one after the
+    other gives (modulo 2^32); the segmented form restarts at flags; the operator does not commute."""
+    rng = np.random.default_rng(8)
+    n = 300
+    abs_ = rng.integers(-2**31, 2**31, (n, 2), dtype=np.int64).astype(np.int32)
+    flags = (rng.random(n) < 0.1).astype(np.uint8)
+    M = 1 << 32
+    for fl in (None, flags):
+        inc = oracle.scan_compose_i32(abs_, fl).astype(np.int64)
+        exc = oracle.scan_compose_i32(abs_, fl, exclusive=True).astype(np.int64)
+        for x0 in (0, 1, 12345):
+            x = x0
+            for i in range(n):
+                if fl is not None and fl[i]:
+                    x = x0
+                assert (exc[i, 0] * x0 + exc[i, 1]) % M == x % M if fl is None or not fl[i] else True
+                x = (int(abs_[i, 0]) * x + int(abs_[i, 1])) % M
+                assert (inc[i, 0] * x0 + inc[i, 1]) % M == x
+    two = np.array([[2, 3], [5, 7]], np.int32)
+    assert oracle.scan_compose_i32(two)[1].tolist() == [10, 22]          # 5 * (2x + 3) + 7
+    assert oracle.scan_compose_i32(two[::-1])[1].tolist() == [10, 17]    # 2 * (5x + 7) + 3
