@@ -359,3 +359,20 @@ def test_scan_with_a_non_commutative_operator(ctx):
     with pytest.raises(Exception, match="invalid sizes"):
         ctx.call("scan_compose_i32", ["i32_2d"], bad)
     bad.free()
+
+
+def test_more_than_2p31_elements(ctx):
+    """Positions beyond 2^31: every index in the kernels and the runtime is 64 bits wide.
+    reduce and scan (+) over 2^31 + 4099 i32 (8 GiB in, 8 GiB out), wrap-around sums."""
+    n = (1 << 31) + 4099
+    block = dg.uniform_int(61, 1 << 20, -1000, 1000, np.int32)
+    xs = np.resize(block, n)
+    xs[-4099:] = 7
+    a = ctx.new("i32_1d", xs)
+    want = np.cumsum(xs, dtype=np.int32)
+    assert int(ctx.call("reduce_add_i32", [np.int32], a)) == int(want[-1])
+    out = ctx.call("scan_add_i32", ["i32_1d"], a)
+    got = out.values()
+    assert got.shape == (n,)
+    assert np.array_equal(got, want)
+    out.free(); a.free()
