@@ -236,9 +236,19 @@ def test_config1_full_size(ctx):
     a.free(); out.free()
     xf = dg.uniform_f32(17, n)
     a = ctx.new("f32_1d", xf)
-    _close(ctx.call("reduce_add_f32", [np.float32], a), oracle.reduce("add", "f32", xf, "f64acc"))
+    ref = float(oracle.reduce("add", "f32", xf, "f64acc"))
+    got = float(ctx.call("reduce_add_f32", [np.float32], a))
+    _close(got, ref)
     out = ctx.call("scan_add_f32", ["f32_1d"], a)
     _close(out.values(), oracle.scan("add", "f32", xf, "f64acc"))
+    # The literal `futhark c` left fold in f32 is itself far from the exact sum at this size
+    # (about 1.3e-4 relative), which is why the f64-accumulated value is the yardstick.
+    lit = float(oracle.reduce("add", "f32", xf))
+    dev_gpu, dev_lit = abs(got - ref) / ref, abs(lit - ref) / ref
+    print(f"\nreduce (+) f32 2^24: GPU deviates {dev_gpu:.2e} from the f64-accumulated sum, "
+          f"the sequential f32 fold {dev_lit:.2e}")
+    assert dev_lit > 2e-5 and dev_gpu < dev_lit
+    a.free(); out.free()
 
 
 @pytest.mark.parametrize("t,op", [("f32", "add"), ("f32", "max"), ("i64", "add"), ("i64", "max")])
@@ -259,8 +269,15 @@ def test_config2_full_size(ctx, t, op):
     red = ctx.call(f"segred_{op}_{t}", [f"{t}_1d"], o, l, v).values()
     ends = offsets + lens - 1
     if (t, op) == ("f32", "add"):
-        _close(red, oracle.segred(op, t, offsets, lens, xs, "f64acc"))
+        ref = oracle.segred(op, t, offsets, lens, xs, "f64acc")
+        _close(red, ref)
         _close(red, got[ends], 2e-6)
+        # informational: per segment (mean 1024 elements) the literal f32 fold stays close too
+        lit = oracle.segred(op, t, offsets, lens, xs)
+        nz = ref != 0
+        print(f"\nsegmented (+) f32: max relative deviation from the f64-accumulated sums: GPU "
+              f"{np.abs(red[nz] - ref[nz]).max() and (np.abs(red[nz] - ref[nz]) / np.abs(ref[nz])).max():.2e}, "
+              f"sequential f32 fold {(np.abs(lit[nz] - ref[nz]) / np.abs(ref[nz])).max():.2e}")
     else:
         assert np.array_equal(red, got[ends])
         assert np.array_equal(red, oracle.segred(op, t, offsets, lens, xs))
