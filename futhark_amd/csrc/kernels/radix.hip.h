@@ -68,7 +68,7 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__
                                                            int64_t num_tiles) {
   constexpr int VEC = 16 / sizeof(K);
   constexpr int ROWS = RS_KPT / VEC;
-  __shared__ uint32_t h[RS_WAVES][RS_RADIX];
+  __shared__ __align__(16) uint32_t h[RS_WAVES][RS_RADIX];
   for (int i = threadIdx.x; i < RS_WAVES * RS_RADIX; i += RS_BLOCK) (&h[0][0])[i] = 0u;
   const int wave = threadIdx.x / WAVE;
   const int64_t tile0 = (int64_t)blockIdx.x * RS_HIST_TILES;
@@ -88,14 +88,21 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__
     for (int r = 0; r < ROWS; r++)
       v[r] = load_vec16(keys + base + ((int64_t)r * RS_BLOCK + threadIdx.x) * VEC);
   };
-  if (full(0)) fetch(0, cur);
+  // The tiles of a block are taken in an order rotated by the block's number:
+  // blocks run in step, and with every block at the same place of its own run
+  // of tiles the reads of one moment would lie 8 tiles apart from each other
+  // (a stride that visits few memory channels) instead of covering a stretch
+  // of memory evenly.
+  const int rot = blockIdx.x % RS_HIST_TILES;
+  auto tile_at = [&](int i) { return (i + rot) % RS_HIST_TILES; };
+  if (full(tile_at(0))) fetch(tile_at(0), cur);
   __syncthreads();
 #pragma unroll
-  for (int t = 0; t < RS_HIST_TILES; t++) {
+  for (int i = 0; i < RS_HIST_TILES; i++) {
+    const int t = tile_at(i);
+    if (i + 1 < RS_HIST_TILES && full(tile_at(i + 1))) fetch(tile_at(i + 1), nxt);
     if (t < tiles_here) {  // uniform
-      const bool is_full = full(t);
-      if (full(t + 1)) fetch(t + 1, nxt);
-      if (is_full) {
+      if (full(t)) {
 #pragma unroll
         for (int r = 0; r < ROWS; r++)
 #pragma unroll
@@ -116,23 +123,28 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__
           sum += h[w][threadIdx.x];
           h[w][threadIdx.x] = 0u;
         }
-        c[t] = sum;
+        c[i] = sum;
       }
       __syncthreads();
-#pragma unroll
-      for (int r = 0; r < ROWS; r++) cur[r] = nxt[r];
     }
+#pragma unroll
+    for (int r = 0; r < ROWS; r++) cur[r] = nxt[r];
   }
   if (threadIdx.x < RS_RADIX) {
+    // c[i] belongs to tile tile_at(i): put the counts in tile order through
+    // this thread's own eight words of LDS (the counters are no longer in use)
+    static_assert(RS_WAVES * RS_RADIX >= RS_RADIX * RS_HIST_TILES, "room for the counts");
+    uint32_t *mine = &h[0][0] + threadIdx.x * RS_HIST_TILES;
+#pragma unroll
+    for (int i = 0; i < RS_HIST_TILES; i++) mine[tile_at(i)] = c[i];
     uint32_t *dst = counts + (int64_t)threadIdx.x * num_tiles + tile0;
     if (tiles_here == RS_HIST_TILES && (num_tiles & 3) == 0) {
       static_assert(RS_HIST_TILES == 8, "two 16-byte stores per digit");
-      reinterpret_cast<uint4 *>(dst)[0] = make_uint4(c[0], c[1], c[2], c[3]);
-      reinterpret_cast<uint4 *>(dst)[1] = make_uint4(c[4], c[5], c[6], c[7]);
+      reinterpret_cast<uint4 *>(dst)[0] = reinterpret_cast<const uint4 *>(mine)[0];
+      reinterpret_cast<uint4 *>(dst)[1] = reinterpret_cast<const uint4 *>(mine)[1];
     } else {
-#pragma unroll
       for (int t = 0; t < RS_HIST_TILES; t++)
-        if (t < tiles_here) dst[t] = c[t];
+        if (t < tiles_here) dst[t] = mine[t];
     }
   }
 }
