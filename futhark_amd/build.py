@@ -35,7 +35,7 @@ HIPCC_FLAGS = [
     "-Wno-unused-result",
 ]
 CC_FLAGS = [
-    "-O2", "-std=c99", "-fPIC", "-Wall", "-Wextra", "-pthread",
+    "-O2", "-std=c99", "-fPIC", "-Wall", "-Wextra", "-Werror", "-pthread",
     f"-I{ROOT / 'include'}", f"-I{ROCM / 'include'}", "-D__HIP_PLATFORM_AMD__=1",
 ]
 
@@ -95,7 +95,7 @@ def build_server() -> Path:
     OBJ.mkdir(parents=True, exist_ok=True)
     bindir = PKG / "bin"
     bindir.mkdir(parents=True, exist_ok=True)
-    server_flags = ["-O2", "-std=c99", "-fPIC", "-Wall", "-Wextra", f"-I{ROOT / 'include'}",
+    server_flags = ["-O2", "-std=c99", "-fPIC", "-Wall", "-Wextra", "-Werror", f"-I{ROOT / 'include'}",
                     f"-I{CSRC / 'server'}"]
     values_obj = OBJ / "server_values.o"
     _run(["gcc", *server_flags, "-c", str(CSRC / "server" / "values.c"), "-o", str(values_obj)])
@@ -115,7 +115,7 @@ def build_server() -> Path:
     # A C program written against the public header only, the way a user of a
     # generated library writes one (run by tests/test_capi_harness.py).
     harness = bindir / "capi-harness"
-    _run(["gcc", "-O1", "-std=c99", "-Wall", "-Wextra", f"-I{ROOT / 'include'}",
+    _run(["gcc", "-O1", "-std=c99", "-Wall", "-Wextra", "-Werror", f"-I{ROOT / 'include'}",
           str(ROOT / "tests" / "c" / "capi_harness.c"), "-o", str(harness), f"-L{LIB}", "-lsegops",
           "-lfuthark_amd_kernels", f"-L{ROCM / 'lib'}", "-lamdhip64", "-lpthread",
           "-Wl,-rpath,$ORIGIN/../lib", f"-Wl,-rpath,{ROCM / 'lib'}"])

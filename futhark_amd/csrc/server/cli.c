@@ -232,7 +232,7 @@ int main(int argc, char **argv) {
 
   /* Initialisation is not profiled; of the runs, only the last one is. */
   futhark_context_pause_profiling(ctx);
-  struct parsed in[3] = {{0}};
+  struct parsed in[ENTRY_MAX_INPUTS] = {{0}};
   read_inputs(e, in);
 
   struct variable fields[2] = {{0}};
@@ -248,8 +248,9 @@ int main(int argc, char **argv) {
   for (int run = 0; run < total; run++) {
     const int timed = !perform_warmup || run > 0;
     const int last = run == total - 1;
-    struct value vals[3];
-    struct value *ins[3] = {&vals[0], &vals[1], &vals[2]};
+    struct value vals[ENTRY_MAX_INPUTS];
+    struct value *ins[ENTRY_MAX_INPUTS];
+    for (int i = 0; i < ENTRY_MAX_INPUTS; i++) ins[i] = &vals[i];
     pack_inputs(ctx, e, in, vals);
     if (futhark_context_sync(ctx) != 0) context_panic(ctx);
     if (last) futhark_context_unpause_profiling(ctx);

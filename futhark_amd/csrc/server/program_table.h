@@ -134,14 +134,16 @@ struct variable {
 
 typedef int (*entry_fn)(struct futhark_context *, struct value *out, struct value **ins);
 
+#define ENTRY_MAX_INPUTS 4 /* most inputs any entry point of the program takes */
+
 struct entry {
   const char *name;
   entry_fn f;
   const char *out_type;
   int out_unique;
   int num_ins;
-  const char *in_types[3];
-  int in_consumed[3];
+  const char *in_types[ENTRY_MAX_INPUTS];
+  int in_consumed[ENTRY_MAX_INPUTS];
   const char *tuning_params[3]; /* NULL terminated */
 };
 

@@ -144,7 +144,7 @@ static void cmd_call(struct server *s, char **args) {
     reply_failure("Unknown entry point: %s\n", name);
     return;
   }
-  struct value *ins[3] = {0};
+  struct value *ins[ENTRY_MAX_INPUTS] = {0};
   for (int i = 0; i < e->num_ins; i++) {
     const char *in_name = need_arg(args, 2 + i);
     struct variable *v = find_var(s, in_name);

@@ -36,6 +36,21 @@ def test_text_in_text_out():
     assert p.stdout.decode() == "[" + ", ".join(rows) + "]\n"      # tests/hist/segmented.fut:3-7
 
 
+def test_entries_with_shaped_operators_take_the_inputs_of_the_reference_tests():
+    # tests/hist/array.fut:3-4
+    p = run(["-e", "rbi_vec_add_i32"],
+            b"[[1,2,3],[4,5,6]] [0i64,0i64,2i64,1i64] [[0,1,2],[0,1,2],[0,1,2],[0,1,2]]")
+    assert p.stdout.decode() == "[[1i32, 4i32, 7i32], [4i32, 6i32, 8i32]]\n"
+    # tests/hist/hist2d.fut:2-3, four inputs
+    p = run(["-e", "rbi_2d_add_i32"],
+            b"[[1,2,3],[4,5,6],[7,8,9]] [1i64, 1i64] [1i64, -1i64] [42, 1337]")
+    assert p.stdout.decode() == "[[1i32, 2i32, 3i32], [4i32, 47i32, 6i32], [7i32, 8i32, 9i32]]\n"
+    p = run(["-e", "vecreduce_add_i32"], b"[[1,2,3],[4,5,6]]")
+    assert p.stdout.decode() == "[5i32, 7i32, 9i32]\n"
+    p = run(["-e", "scan_compose_i32"], b"[[2,3],[5,7],[1,1]]")   # 5(2x+3)+7 = 10x+22, then +1
+    assert p.stdout.decode() == "[[2i32, 3i32], [10i32, 22i32], [10i32, 23i32]]\n"
+
+
 def test_tuple_result_prints_one_field_per_line():
     p = run(["-e", "radix_sort_pairs_u32_i32"], b"[5u32, 1u32, 5u32, 0u32] [0, 1, 2, 3]")
     assert p.stdout.decode() == "[0u32, 1u32, 5u32, 5u32]\n[3i32, 1i32, 0i32, 2i32]\n"

@@ -50,8 +50,7 @@ def test_introspection(srv):
     m = manifest.manifest()            # the server and the manifest describe the same API
     assert set(entries) == set(m["entry_points"])
     assert set(types) == set(m["types"]) | {"i32", "i64", "f32", "f64"}
-    for name in ("rbi_max_u16", "segred_add_f64", "reduce_min_i64", "radix_sort_pairs_u64_i32", "bmm_bf16"):
-        e = m["entry_points"][name]
+    for name, e in m["entry_points"].items():   # every entry point, whatever its number of inputs
         assert srv.cmd("inputs", name) == [("*" if i["unique"] else "") + i["type"] for i in e["inputs"]]
         assert srv.cmd("output", name) == [("*" if e["output"]["unique"] else "") + e["output"]["type"]]
         assert [l.split()[0] for l in srv.cmd("tuning_params", name)] == e["tuning_params"]
@@ -152,6 +151,23 @@ def test_scalars_new_array_index(srv, tmp_path):
     with pytest.raises(ServerFailure, match=r"Value 0 mismatch: expected type i32, got i64"):
         srv.cmd("new_array", "x", "[]i32", 1, "k")
     srv.cmd("free", "k", "a", "b", "arr", "elem", "rep", "io", "tot")
+
+
+@pytest.mark.gpu
+def test_entry_with_four_inputs(srv, tmp_path, goldens):
+    """reduce_by_index_2d takes the most inputs of all entries (tests/hist/hist2d.fut:2-3)."""
+    c = goldens["hist2d"]["cases"][0]
+    f = tmp_path / "h.bin"
+    fv.write_binary(f, [np.array(c["dest"], np.int32), np.array(c["is"], np.int64),
+                        np.array(c["js"], np.int64), np.array(c["vs"], np.int32)])
+    srv.cmd("restore", f, "dest", "[][]i32", "is", "[]i64", "js", "[]i64", "vs", "[]i32")
+    srv.call("rbi_2d_add_i32", "h2", "dest", "is", "js", "vs")
+    out = tmp_path / "o.bin"
+    srv.cmd("store", out, "h2")
+    (h2,) = fv.read_binary(out, [("i32", 2)])
+    assert h2.tolist() == c["out"]
+    assert srv.cmd("inputs", "rbi_2d_add_i32") == ["*[][]i32", "[]i64", "[]i64", "[]i32"]
+    srv.cmd("free", "dest", "is", "js", "vs", "h2")
 
 
 @pytest.mark.gpu
