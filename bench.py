@@ -300,7 +300,8 @@ MEASURED_TRAFFIC_BYTES = {
     "hist_add_i32_H256_uniform_2p27": 1074.2e6,
     "hist_add_i32_H65536_uniform_2p27": 1107.6e6,
     "hist_add_i32_H4194304_uniform_2p27": 4229.0e6,
-    "sort_u32_2p26": 4088.4e6,
+    "sort_u32_2p26": 3827.6e6,
+    "scanrows_add_f32_65536x1024": 539.1e6,
     "hist_max_f32_H256_uniform_2p27": 1074.5e6,
     "transpose_f32_8192x8192": 537.6e6,
     "vecreduce_add_f32_65536x1024": 269.5e6,
