@@ -9,7 +9,7 @@
 //   1. segred_bounds_kernel finds, for every tile boundary, the first segment
 //      that starts at or after it and the first that ends after it (every
 //      segment marks the boundaries it owns; segments are in order);
-//   2. segred_tiles_kernel scans every 16 KiB tile on its own (start flags from
+//   2. segred_tiles_kernel scans every 32 KiB tile on its own (start flags from
 //      `offsets` as an LDS bitmap, DPP wave scans, scanned tile kept in LDS),
 //      writes the result of every segment that lies inside the tile, and leaves
 //      three words per tile: the value at the end of the segment that entered
@@ -19,7 +19,7 @@
 //   3. segred_fixup_kernel finishes the segments that cross tile boundaries:
 //      one wave per tile with a head walks left over the tails, 64 tiles per
 //      step, up to the tile in which the segment starts.
-// Tiles are small and independent, so eight blocks share a CU and their memory
+// Tiles are small and independent, so four blocks share a CU and their memory
 // latencies (bounds, offsets, lens: one round trip each) hide one another.
 #include "dispatch.hip.h"
 
@@ -27,7 +27,10 @@ namespace fa {
 
 constexpr int SRI_BLOCK = 256;
 constexpr int SRI_WAVES = SRI_BLOCK / WAVE;
-constexpr int SRI_ROWS = 4;  // 16-byte loads per thread
+// 16-byte loads per thread.  Measured on 2^26 elements, 4 against 8: f32
+// 52.7 -> 51.6 us, i64 121.6 -> 103.8 us (and 100.2 us with non-temporal loads,
+// which do nothing for f32); 2 is slower for both.
+constexpr int SRI_ROWS = 8;
 
 template <class T> constexpr int sri_tile_elems() { return SRI_BLOCK * SRI_ROWS * Vec16<T>::N; }
 
@@ -149,7 +152,7 @@ __global__ __launch_bounds__(SRI_BLOCK) void segred_tiles_kernel(
   for (int r = 0; r < SRI_ROWS; r++) {
     const int64_t idx = wbase + (int64_t)(r * WAVE + lane) * VEC;
     if (idx + VEC <= n) {
-      const Vec16<T> v = load_vec16(vs + idx);
+      const Vec16<T> v = sizeof(T) == 8 ? load_vec16_nt(vs + idx) : load_vec16(vs + idx);
 #pragma unroll
       for (int e = 0; e < VEC; e++) x[r][e] = v.e[e];
     } else {
