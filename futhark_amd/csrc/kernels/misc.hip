@@ -114,7 +114,10 @@ extern "C" const char *fa_strerror(int code) {
 }
 
 // ------------------------------------------------------------------ tuning
-static fa_tuning g_tuning = {0, 0, 0};
+// One set per calling thread: the launchers read it on the thread that calls
+// them, so callers that hold different values (contexts with different tuning
+// parameters) can run side by side without touching each other's.
+static thread_local fa_tuning g_tuning = {0, 0, 0};
 
 extern "C" void fa_set_tuning(const fa_tuning *t) {
   if (t == nullptr) {

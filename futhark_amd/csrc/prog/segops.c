@@ -541,7 +541,14 @@ static int do_rbi_shaped(struct futhark_context *ctx, fa_dtype t, fa_op op, size
   return 0;
 }
 
-#define ENTER(ctx) pthread_mutex_lock(&(ctx)->lock)
+/* Every entry point runs under the context's lock and with the context's tuning
+ * parameters in force for the calling thread (the kernel library keeps them per
+ * thread), so contexts with different parameters can be used side by side. */
+#define ENTER(ctx)                      \
+  do {                                  \
+    pthread_mutex_lock(&(ctx)->lock);   \
+    apply_tuning(ctx);                  \
+  } while (0)
 #define LEAVE(ctx) pthread_mutex_unlock(&(ctx)->lock)
 
 #define DEFINE_SEGOP_ENTRIES(OP, T, CT)                                                       \

@@ -84,7 +84,9 @@ int fa_version(void);
 /* Thresholds behind the launchers' choice of code path, the counterpart of
  * the threshold and shared_memory tuning parameters a compiled program exposes
  * (src/Futhark/CodeGen/ImpGen/GPU/Base.hs:118-120, rts/c/gpu.h:93-135).  They are
- * process-wide; a field that is 0 means the built-in default.
+ * kept per calling thread (a launcher reads the values of the thread that calls
+ * it; a new thread starts with the defaults); a field that is 0 means the
+ * built-in default.
  *   segred_small_threshold  rows of a regular segmented reduce up to this many
  *                           elements are folded by groups of lanes, longer
  *                           ones by whole blocks (default 8192)

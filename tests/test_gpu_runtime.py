@@ -165,5 +165,13 @@ def test_tuning_parameters_select_other_code_paths_with_the_same_results(segops_
         np.testing.assert_allclose(out.values(), A.astype(np.float64) @ B.astype(np.float64), rtol=1e-4, atol=1e-5)
         ev = [e for e in json.loads(c.report())["events"] if e["name"] == "segmap_matmul"]
         assert ev[0]["details"]["padded"] is False
+    # two contexts alive at once keep their own values, whichever was created or used last
+    with Context(segops_lib, profiling=True, tuning=tuning) as c1, Context(segops_lib, profiling=True) as c2:
+        for c in (c1, c2, c1, c2):
+            out = c.call("bmm_f32", ["f32_3d"], c.new("f32_3d", A), c.new("f32_3d", B))
+            np.testing.assert_allclose(out.values(), A.astype(np.float64) @ B.astype(np.float64), rtol=1e-4, atol=1e-5)
+        for c, padded in ((c1, True), (c2, False)):
+            ev = [e for e in json.loads(c.report())["events"] if e["name"] == "segmap_matmul"]
+            assert len(ev) == 2 and all(e["details"]["padded"] is padded for e in ev)
     with pytest.raises(KeyError):
         Context(segops_lib, tuning={"segops.no_such_parameter": 1})
