@@ -123,7 +123,7 @@ def build_server() -> Path:
 
 
 def build_oracle() -> Path:
-    _run(["make", "-C", str(ROOT / "oracle"), "-s"])
+    _run(["make", "-B", "-C", str(ROOT / "oracle"), "-s"])  # always compiles, like the rest
     return ROOT / "oracle" / "liboracle.so"
 
 
