@@ -223,6 +223,57 @@ __global__ __launch_bounds__(256) void segred_small_vec_kernel(const T *__restri
   if (seg < m && sub == 0) out[seg] = a;
 }
 
+// Rows so short that a lane holds at most two 16-byte vectors of one: a group
+// of G lanes takes R rows at a time (rows g, g + groups, g + 2 groups, ..., so
+// that the lanes of a wave still read consecutive memory) and requests all
+// their vectors before folding any, which keeps 2 R loads in flight per lane
+// instead of 2.
+template <class T, class Op, int G, int R>
+__global__ __launch_bounds__(256) void segred_short_vec_kernel(const T *__restrict__ xss, int64_t m,
+                                                               int64_t k, T *__restrict__ out,
+                                                               int64_t groups) {
+  constexpr int VEC = Vec16<T>::N;
+  const int64_t gthread = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t g = gthread / G;
+  const int sub = (int)(gthread % G);
+  const int64_t kv = k / VEC;  // at most 2 G
+  Vec16<T> v[R][2];
+  bool have[R][2];
+#pragma unroll
+  for (int u = 0; u < R; u++) {
+    const int64_t seg = g + u * groups;
+#pragma unroll
+    for (int q = 0; q < 2; q++) {
+      const int64_t j = sub + q * G;
+      have[u][q] = g < groups && seg < m && j < kv;
+      if (have[u][q]) v[u][q] = load_vec16_nt(xss + seg * k + j * VEC);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < R; u++) {
+    T a = Op::identity();
+#pragma unroll
+    for (int q = 0; q < 2; q++)
+      if (have[u][q]) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) a = Op::apply(a, v[u][q].e[e]);
+      }
+#pragma unroll
+    for (int d = G / 2; d >= 1; d /= 2) {
+      T other;
+      if constexpr (sizeof(T) == 4) {
+        other = bit_cast<T>(__shfl_down(bit_cast<int>(a), d, WAVE));
+      } else {
+        other = bit_cast<T>((unsigned long long)__shfl_down(
+            (unsigned long long)bit_cast<uint64_t>(a), d, WAVE));
+      }
+      a = Op::apply(a, other);
+    }
+    const int64_t seg = g + u * groups;
+    if (g < groups && seg < m && sub == 0) __builtin_nontemporal_store(a, &out[seg]);
+  }
+}
+
 // k large: one block per segment (grid-stride over segments).  With `pieces`
 // > 1 every row is cut into that many pieces of `piece_len` elements (the last
 // one shorter) and out[seg * pieces + p] receives the fold of piece p: the
@@ -308,8 +359,21 @@ static int launch_small(hipStream_t s, const T *in, int64_t m, int64_t k, T *o) 
     else if (units <= 64) FA_SMALL(KERNEL, 16); \
     else FA_SMALL(KERNEL, 64);               \
   } while (0)
-  if (vec) FA_SMALL_BY_UNITS(segred_small_vec_kernel);
+#define FA_SHORT(G)                                                                           \
+  do {                                                                                        \
+    constexpr int R = 4;                                                                      \
+    const int64_t groups = ceil_div(m, (int64_t)R);                                           \
+    const int64_t grid = ceil_div(groups * (G), (int64_t)256);                                \
+    if (grid > INT32_MAX) return FA_EINVAL;                                                   \
+    hipLaunchKernelGGL((segred_short_vec_kernel<T, Op, G, R>), dim3((unsigned)grid), dim3(256), 0, \
+                       s, in, m, k, o, groups);                                               \
+  } while (0)
+  if (vec && units <= 2) FA_SHORT(1);
+  else if (vec && units <= 8) FA_SHORT(4);
+  else if (vec && units <= 32) FA_SHORT(16);
+  else if (vec) FA_SMALL_BY_UNITS(segred_small_vec_kernel);
   else FA_SMALL_BY_UNITS(segred_small_kernel);
+#undef FA_SHORT
 #undef FA_SMALL_BY_UNITS
 #undef FA_SMALL
   return launch_status();
