@@ -24,7 +24,10 @@ namespace fa {
 // One block of 1024 threads per CU: measured faster than more, smaller blocks
 // (fewer partials for the finisher to collect), 64 bytes in flight per thread.
 constexpr int SEGRED_BLOCK = 1024;
-constexpr int SEGRED_UNROLL = 4;
+// 16-byte loads a thread of the non-segmented kernel keeps in flight.  Measured
+// at 2^26 f32: 1 -> 48.1 us, 2 -> 43.9 us, 3 -> 45.5 us, 4 -> 46.5 us, 8 and 16 -> 46 us
+// (2^24 elements: 15.7 us for 2 and more).
+constexpr int SEGRED_UNROLL = 2;
 constexpr int SEGRED_MAX_GRID = 1024;
 constexpr size_t SEGRED_HEADER_BYTES = 256;
 
