@@ -296,7 +296,8 @@ MEASURED_TRAFFIC_BYTES = {
     "segscan_add_f32_2p26": 605.3e6,
     "scan_add_f32_2p26": 538.6e6,
     "reduce_add_f32_2p26": 268.5e6,
-    "segred_add_f32_2p26": 283.3e6,
+    "segred_add_f32_2p26": 277.3e6,
+    "segreduce_add_f32_1048576x64": 273.7e6,
     "hist_add_i32_H256_uniform_2p27": 1074.2e6,
     "hist_add_i32_H65536_uniform_2p27": 1107.6e6,
     "hist_add_i32_H4194304_uniform_2p27": 4229.0e6,
