@@ -28,10 +28,18 @@ namespace fa {
 #define FA_SCAN_ROWS4 8 /* 4-byte elements: 32 per thread */
 #endif
 #ifndef FA_SCAN_ROWS8
-#define FA_SCAN_ROWS8 4 /* 8-byte elements: 8 per thread (more spills registers) */
+#define FA_SCAN_ROWS8 8 /* 8-byte elements: 16 per thread */
 #endif
 #ifndef FA_SCAN_WAVES
 #define FA_SCAN_WAVES 16
+#endif
+// 8-byte elements: 16 per thread need more than the 128 registers a thread of a
+// 1024-thread block may have (8 per thread in such a block: 296 us for a
+// segmented i64 scan of 2^26 elements; 16 per thread there spill: 326 us), so
+// these scans run in 512-thread blocks, two to a CU, with tiles of 64 KiB:
+// 237 us.
+#ifndef FA_SCAN_WAVES8
+#define FA_SCAN_WAVES8 8
 #endif
 // Cache policy, measured: plain data loads, non-temporal flag loads and
 // non-temporal stores give the best rate (a copy kernel gains 25 % from
@@ -46,8 +54,8 @@ namespace fa {
 #define FA_SCAN_STORE store_vec16_nt
 #endif
 template <class T> constexpr int scan_rows() { return sizeof(T) == 4 ? FA_SCAN_ROWS4 : FA_SCAN_ROWS8; }
-constexpr int SCAN_WAVES = FA_SCAN_WAVES;
-constexpr int SCAN_BLOCK = SCAN_WAVES * WAVE;
+template <class T> constexpr int scan_waves() { return sizeof(T) == 4 ? FA_SCAN_WAVES : FA_SCAN_WAVES8; }
+template <class T> constexpr int scan_block() { return scan_waves<T>() * WAVE; }
 
 // Descriptors per lane in a look-back window.  Measured on 2^26 f32: 1 -> 99 us,
 // 2 -> 103 us, 4 -> 109 us; the nearest published prefix is normally within 64
@@ -62,7 +70,7 @@ constexpr size_t SCAN_HEADER_BYTES = 256;  // ticket counter, padded
 constexpr size_t SCAN_DESC_BYTES = 16;     // per tile
 
 template <class T> constexpr int scan_tile_elems() {
-  return SCAN_BLOCK * scan_rows<T>() * Vec16<T>::N;
+  return scan_block<T>() * scan_rows<T>() * Vec16<T>::N;
 }
 
 __device__ __forceinline__ uint32_t desc_meta(uint32_t epoch, uint32_t flag, uint32_t status) {
@@ -125,7 +133,7 @@ enum { SEG_NONE = 0, SEG_FLAGS = 1, SEG_ROWS = 2 };
 
 // out[n]; EXCL selects the exclusive form.
 template <class T, class Op, int SEGKIND, bool EXCL>
-__global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
+__global__ __launch_bounds__(scan_block<T>()) void segscan_kernel(
     const T *__restrict__ xs, const uint8_t *__restrict__ flags, int64_t n, T *__restrict__ out,
     uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles, int64_t seg_len) {
   constexpr bool SEG = SEGKIND != SEG_NONE;
@@ -133,6 +141,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void segscan_kernel(
   constexpr int VEC = Vec16<T>::N;
   constexpr int SCAN_ROWS = scan_rows<T>();
   constexpr int WCHUNK = SCAN_ROWS * WAVE * VEC;
+  constexpr int SCAN_WAVES = scan_waves<T>();
   constexpr int TILE = SCAN_WAVES * WCHUNK;
   using Pair = SegPair<T>;
 
@@ -466,7 +475,7 @@ static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int6
   if (tiles > INT32_MAX) return FA_EINVAL;
   uint32_t *ticket = (uint32_t *)scratch;
   uint64_t *desc = (uint64_t *)((char *)scratch + SCAN_HEADER_BYTES);
-  const dim3 grid((unsigned)tiles), block(SCAN_BLOCK);
+  const dim3 grid((unsigned)tiles), block(scan_block<T>());
 #define FA_LAUNCH(SEGV, EXV)                                                              \
   hipLaunchKernelGGL((segscan_kernel<T, Op, SEGV, EXV>), grid, block, 0, s, (const T *)xs, \
                      flags, n, (T *)out, ticket, desc, epoch, tiles, seg_len)
