@@ -511,6 +511,26 @@ static void cmd_fields(char **args) {
 
 /* The library's public API has no way to take a second reference to an
  * array, so a projected field is a copy made through host memory. */
+/* dst (an array value of the same type, still empty) becomes a copy of src. */
+static int copy_array_value(struct server *s, const struct value *src, struct value *dst) {
+  const struct stype *ft = src->type;
+  const struct fv_primtype *p = fv_primtype(ft->prim);
+  const int64_t *shape = ft->arr_shape(s->ctx, src->u.arr);
+  size_t count = 1;
+  for (int i = 0; i < ft->rank; i++) count *= (size_t)shape[i];
+  void *host = malloc(count * (size_t)p->size + 1);
+  if (host == NULL) return 1;
+  int err = ft->arr_values(s->ctx, src->u.arr, host);
+  err |= futhark_context_sync(s->ctx);
+  if (err == 0) {
+    dst->u.arr = ft->arr_new(s->ctx, host, shape);
+    err = dst->u.arr == NULL;
+    err |= futhark_context_sync(s->ctx);
+  }
+  free(host);
+  return err;
+}
+
 static void cmd_project(struct server *s, char **args) {
   const char *to = need_arg(args, 0);
   struct variable *from = find_var(s, need_arg(args, 1));
@@ -536,25 +556,51 @@ static void cmd_project(struct server *s, char **args) {
     return;
   }
   struct value *src = &from->value.u.fields[fi]->value;
-  const struct stype *ft = src->type;
-  const struct fv_primtype *p = fv_primtype(ft->prim);
-  const int64_t *shape = ft->arr_shape(s->ctx, src->u.arr);
-  size_t count = 1;
-  for (int i = 0; i < ft->rank; i++) count *= (size_t)shape[i];
-  void *host = malloc(count * (size_t)p->size + 1);
-  if (host == NULL) {
-    reply_failure("Out of memory.\n");
+  struct variable *out = create_var(s, to, src->type);
+  int err = copy_array_value(s, src, &out->value);
+  report_context_error(s, err);
+  if (err != 0) drop_var(s, out, 1);
+}
+
+/* new v0 type v1 v2 ...: a record of the given type with copies of the fields
+ * (cmd_new, rts/c/server.h:1220-1271). */
+static void cmd_new(struct server *s, char **args) {
+  const char *to = need_arg(args, 0);
+  const struct stype *t = find_type(need_arg(args, 1));
+  if (t == NULL) {
+    reply_failure("Unknown type: %s\n", args[1]);
     return;
   }
-  int err = ft->arr_values(s->ctx, src->u.arr, host);
-  err |= futhark_context_sync(s->ctx);
-  struct variable *out = create_var(s, to, ft);
-  if (err == 0) {
-    out->value.u.arr = ft->arr_new(s->ctx, host, shape);
-    err = out->value.u.arr == NULL;
-    err |= futhark_context_sync(s->ctx);
+  if (find_var(s, to) != NULL) {
+    reply_failure("Variable already exists: %s\n", to);
+    return;
   }
-  free(host);
+  if (t->kind != K_RECORD) {
+    reply_failure("Not a record type\n");
+    return;
+  }
+  const int given = count_args(args) - 2;
+  if (given != t->num_fields) {
+    reply_failure("%d fields expected but %d values provided.\n", given, t->num_fields);
+    return;
+  }
+  struct variable *from[4] = {0};
+  for (int i = 0; i < given; i++) {
+    from[i] = find_var(s, args[2 + i]);
+    if (from[i] == NULL) {
+      reply_failure("Unknown variable: %s\n", args[2 + i]);
+      return;
+    }
+    if (strcmp(from[i]->value.type->name, t->field_types[i]) != 0) {
+      reply_failure("Field %s mismatch: expected type %s, got %s\n", t->field_names[i],
+                    t->field_types[i], from[i]->value.type->name);
+      return;
+    }
+  }
+  struct variable *out = create_var(s, to, t);
+  int err = 0;
+  for (int i = 0; i < given && err == 0; i++)
+    err = copy_array_value(s, &from[i]->value, &out->value.u.fields[i]->value);
   report_context_error(s, err);
   if (err != 0) drop_var(s, out, 1);
 }
@@ -652,10 +698,10 @@ static void process_line(struct server *s, char *line) {
     for (int i = 0; i < NUM_ENTRIES; i++) puts(entries[i].name);
   } else if (strcmp(cmd, "types") == 0) {
     for (int i = 0; i < NUM_TYPES; i++) puts(types[i].name);
-  } else if (strcmp(cmd, "set") == 0 || strcmp(cmd, "zip") == 0 || strcmp(cmd, "unzip") == 0 ||
-             strcmp(cmd, "new") == 0) {
-    /* In-place array update and record construction: no entry point of this
-     * program takes a record, and no array of records exists. */
+  } else if (strcmp(cmd, "new") == 0) {
+    cmd_new(s, args);
+  } else if (strcmp(cmd, "set") == 0 || strcmp(cmd, "zip") == 0 || strcmp(cmd, "unzip") == 0) {
+    /* In-place array update and arrays of records: this program has neither. */
     reply_failure("Command `%s` is not supported by this program.\n", cmd);
   } else if (strcmp(cmd, "variants") == 0 || strcmp(cmd, "variant") == 0 ||
              strcmp(cmd, "construct") == 0 || strcmp(cmd, "destruct") == 0) {

@@ -192,6 +192,20 @@ def test_pair_sort_record_and_hist(srv, tmp_path):
     assert np.array_equal(k1, keys[order]) and np.array_equal(v1, vals[order])
     assert np.array_equal(k2, k1) and np.array_equal(v2, v1)
     assert np.array_equal(hist, oracle.rbi("add", "i32", np.zeros(1000, np.int32), idx, vals))
+    # a record built from its fields (cmd_new, rts/c/server.h:1220-1271) holds copies of them
+    srv.cmd("new", "rec", "([]u32, []i32)", "keys", "vals")
+    srv.cmd("store", out, "rec")
+    rk, rv = fv.read_binary(out, [("u32", 1), ("i32", 1)])
+    assert np.array_equal(rk, keys) and np.array_equal(rv, vals)
+    with pytest.raises(ServerFailure, match="1 fields expected but 2 values provided."):
+        srv.cmd("new", "r2", "([]u32, []i32)", "keys")
+    with pytest.raises(ServerFailure, match=r"Field 1 mismatch: expected type \[\]i32, got \[\]u32"):
+        srv.cmd("new", "r2", "([]u32, []i32)", "keys", "keys")
+    with pytest.raises(ServerFailure, match="Not a record type"):
+        srv.cmd("new", "r2", "[]u32", "keys")
+    with pytest.raises(ServerFailure, match="Variable already exists: rec"):
+        srv.cmd("new", "rec", "([]u32, []i32)", "keys", "vals")
+    srv.cmd("free", "rec")
     with pytest.raises(ServerFailure, match="No such field"):
         srv.cmd("project", "x", "sorted", "2")
     with pytest.raises(ServerFailure, match="Not a sum type"):
