@@ -521,23 +521,26 @@ __global__ __launch_bounds__(256) void mm_pad_kernel(const T *__restrict__ src, 
                                                      int64_t rows, int64_t cols, int64_t rows_p,
                                                      int64_t cols_p) {
   const int64_t b = blockIdx.z;
-  const int64_t r = (int64_t)blockIdx.y;
-  const T *s = src + (b * rows + r) * cols;
-  T *d = dst + (b * rows_p + r) * cols_p;
-  const bool row_in = r < rows;
-  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols_p; c += (int64_t)gridDim.x * 256)
-    __builtin_nontemporal_store((row_in && c < cols) ? s[c] : T(0), &d[c]);
+  // grid.y is capped (65535 at most), so a block walks rows with that stride.
+  for (int64_t r = blockIdx.y; r < rows_p; r += gridDim.y) {
+    const T *s = src + (b * rows + r) * cols;
+    T *d = dst + (b * rows_p + r) * cols_p;
+    const bool row_in = r < rows;
+    for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols_p; c += (int64_t)gridDim.x * 256)
+      __builtin_nontemporal_store((row_in && c < cols) ? s[c] : T(0), &d[c]);
+  }
 }
 
 __global__ __launch_bounds__(256) void mm_unpad_kernel(const float *__restrict__ src,
                                                        float *__restrict__ dst, int64_t rows,
                                                        int64_t cols, int64_t rows_p, int64_t cols_p) {
   const int64_t b = blockIdx.z;
-  const int64_t r = (int64_t)blockIdx.y;
-  const float *s = src + (b * rows_p + r) * cols_p;
-  float *d = dst + (b * rows + r) * cols;
-  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += (int64_t)gridDim.x * 256)
-    __builtin_nontemporal_store(s[c], &d[c]);
+  for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+    const float *s = src + (b * rows_p + r) * cols_p;
+    float *d = dst + (b * rows + r) * cols;
+    for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < cols; c += (int64_t)gridDim.x * 256)
+      __builtin_nontemporal_store(s[c], &d[c]);
+  }
 }
 
 struct MmPlan {
@@ -564,8 +567,7 @@ static MmPlan mm_plan(fa_dtype in_t, int64_t batch, int64_t M, int64_t N, int64_
   const double work = (double)batch * M * N * K, padded_work = (double)batch * p.Mp * p.Np * p.Kp;
   fa_tuning tune;
   fa_get_tuning(&tune);
-  p.padded = work >= (double)tune.matmul_pad_min_work && padded_work <= 8.0 * work && p.Mp <= 65535 &&
-             batch <= 65535;
+  p.padded = work >= (double)tune.matmul_pad_min_work && padded_work <= 8.0 * work && batch <= 65535;
   p.a_bytes = mm_align((size_t)batch * p.Mp * p.Kp * es);
   p.b_bytes = mm_align((size_t)batch * p.Kp * p.Np * es);
   p.c_bytes = mm_align((size_t)batch * p.Mp * p.Np * 4);
@@ -587,21 +589,18 @@ static int matmul_direct(fa_stream_t stream, fa_dtype in_t, const void *A, const
     const dim3 grid((unsigned)(N / MM_BN), (unsigned)(M / MM_BM), (unsigned)batch);
     int rc = 0;
     if (in_t == FA_F32) {
-      static bool raised = false;
-      if (!raised) { rc = raise_lds(matmul32_kernel, 2 * MM32_STAGE_BYTES); raised = rc == 0; }
-      if (rc) return rc;
+      static const int raised = raise_lds(matmul32_kernel, 2 * MM32_STAGE_BYTES);
+      if ((rc = raised)) return rc;
       hipLaunchKernelGGL(matmul32_kernel, grid, dim3(MM_THREADS), 2 * MM32_STAGE_BYTES, st,
                          (const float *)A, (const float *)B, C, (int)M, (int)N, (int)K);
     } else if (in_t == FA_F16) {
-      static bool raised = false;
-      if (!raised) { rc = raise_lds(matmul16_kernel<false>, 2 * MM16_STAGE_BYTES); raised = rc == 0; }
-      if (rc) return rc;
+      static const int raised = raise_lds(matmul16_kernel<false>, 2 * MM16_STAGE_BYTES);
+      if ((rc = raised)) return rc;
       hipLaunchKernelGGL((matmul16_kernel<false>), grid, dim3(MM16_THREADS), 2 * MM16_STAGE_BYTES, st,
                          (const uint16_t *)A, (const uint16_t *)B, C, (int)M, (int)N, (int)K);
     } else {
-      static bool raised = false;
-      if (!raised) { rc = raise_lds(matmul16_kernel<true>, 2 * MM16_STAGE_BYTES); raised = rc == 0; }
-      if (rc) return rc;
+      static const int raised = raise_lds(matmul16_kernel<true>, 2 * MM16_STAGE_BYTES);
+      if ((rc = raised)) return rc;
       hipLaunchKernelGGL((matmul16_kernel<true>), grid, dim3(MM16_THREADS), 2 * MM16_STAGE_BYTES, st,
                          (const uint16_t *)A, (const uint16_t *)B, C, (int)M, (int)N, (int)K);
     }
@@ -632,8 +631,8 @@ extern "C" size_t fa_matmul_workspace_bytes(fa_dtype in_t, int64_t batch, int64_
 template <class T>
 static int mm_pad(hipStream_t st, const void *src, void *dst, int64_t batch, int64_t rows,
                   int64_t cols, int64_t rows_p, int64_t cols_p) {
-  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(cols_p, (int64_t)256), 64), (unsigned)rows_p,
-                  (unsigned)batch);
+  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(cols_p, (int64_t)256), 64),
+                  (unsigned)std::min<int64_t>(rows_p, 65535), (unsigned)batch);
   hipLaunchKernelGGL((mm_pad_kernel<T>), grid, dim3(256), 0, st, (const T *)src, (T *)dst, rows, cols,
                      rows_p, cols_p);
   return launch_status();
@@ -662,8 +661,8 @@ extern "C" int fa_matmul_ws(fa_stream_t stream, fa_dtype in_t, const void *A, co
   if (rc != 0) return rc;
   rc = matmul_direct(stream, in_t, Ap, Bp, (float *)Cp, batch, p.Mp, p.Np, p.Kp);
   if (rc != 0) return rc;
-  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(N, (int64_t)256), 64), (unsigned)M,
-                  (unsigned)batch);
+  const dim3 grid((unsigned)std::min<int64_t>(ceil_div(N, (int64_t)256), 64),
+                  (unsigned)std::min<int64_t>(M, 65535), (unsigned)batch);
   hipLaunchKernelGGL(mm_unpad_kernel, grid, dim3(256), 0, st, (const float *)Cp, C, M, N, p.Mp, p.Np);
   return launch_status();
 }

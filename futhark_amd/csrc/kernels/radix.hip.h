@@ -318,13 +318,10 @@ static int rs_pass(hipStream_t st, const K *kin, K *kout, const void *vin, void 
   const size_t lds =
       RS_LDS_FIXED + (size_t)RS_TILE * (sizeof(K) > sizeof(V) ? sizeof(K) : sizeof(V));
   auto scatter = rs_scatter_kernel<K, VB, DigitFn>;
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void *)scatter,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    raised = true;
-  }
+  // Initialised once, under the lock C++ gives function-local statics.
+  static const hipError_t raised = hipFuncSetAttribute(
+      (const void *)scatter, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  if (raised != hipSuccess) return (int)raised;
   hipLaunchKernelGGL((rs_hist_kernel<K, DigitFn>),
                      dim3((unsigned)ceil_div(sc.tiles, (int64_t)RS_HIST_TILES)), dim3(RS_BLOCK), 0, st,
                      kin, n, fn, pass, sc.counts, sc.tiles);

@@ -587,13 +587,10 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
   grid -= grid % (NUM_XCDS * P);
   if (grid < NUM_XCDS * P) grid = NUM_XCDS * P;
   auto kernel = seghist_lds_kernel<T, Op, I, MODE>;
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    raised = true;
-  }
+  // Initialised once, under the lock C++ gives function-local statics.
+  static const hipError_t raised = hipFuncSetAttribute(
+      (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
+  if (raised != hipSuccess) return (int)raised;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(HIST_BLOCK), lds, st, is, js, vs, n, dest,
                      (int64_t)0, H, range_bins, P, log2_copies, seg_len, H_seg);
   return launch_status();
@@ -609,13 +606,10 @@ static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, in
   int index_bits = 1;
   while (((int64_t)1 << index_bits) < H) index_bits++;
   auto kernel = seghist_wave_private_kernel<T, I>;
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    raised = true;
-  }
+  // Initialised once, under the lock C++ gives function-local statics.
+  static const hipError_t raised = hipFuncSetAttribute(
+      (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
+  if (raised != hipSuccess) return (int)raised;
   const size_t lds = (size_t)H * sizeof(T) * (HIST_BLOCK / WAVE);
   const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
   hipLaunchKernelGGL(kernel, dim3(hist_num_cus() * per_cu), dim3(HIST_BLOCK), lds, st, is, vs, n,
@@ -647,13 +641,10 @@ static int launch_part_hist(hipStream_t st, const U *is, const T *vs, int64_t n,
   rc = rs_pass<U, (int)sizeof(T)>(st, is, pis, vs, pvs, n, fn, 0, 1u, sc);
   if (rc != 0) return rc;
   auto kernel = seghist_part_kernel<T, Op, U>;
-  static bool raised = false;
-  if (!raised) {
-    hipError_t e = hipFuncSetAttribute((const void *)kernel,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
-    if (e != hipSuccess) return (int)e;
-    raised = true;
-  }
+  // Initialised once, under the lock C++ gives function-local statics.
+  static const hipError_t raised = hipFuncSetAttribute(
+      (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
+  if (raised != hipSuccess) return (int)raised;
   hipLaunchKernelGGL(kernel, dim3(hist_num_cus()), dim3(HIST_BLOCK), HIST_LDS_BYTES, st, pis, pvs,
                      sc.offsets, sc.tiles, dest, H, shift);
   return launch_status();

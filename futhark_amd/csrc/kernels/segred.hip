@@ -56,8 +56,15 @@ __device__ __forceinline__ T block_reduce(T v, T *lds /* BLOCK/64 slots */) {
   return r;
 }
 
+// The scratch buffer and its epochs are shared with the single-pass scan, whose
+// descriptor words end in (epoch << 3 | flag << 2 | status) with status 1 or
+// 2.  A partial ends in (epoch << 3 | 3): no word a scan has ever left behind
+// can be taken for the partial of a later reduction, whatever the two epochs.
+__device__ __forceinline__ uint32_t partial_meta(uint32_t epoch) { return (epoch << 3) | 3u; }
+
 template <class T>
 __device__ __forceinline__ void partial_publish(uint64_t *desc, int slot, uint32_t epoch, T v) {
+  epoch = partial_meta(epoch);
   if constexpr (sizeof(T) == 4) {
     st_relaxed_u64(desc + 2 * slot, ((uint64_t)bit_cast<uint32_t>(v) << 32) | epoch);
   } else {
@@ -69,6 +76,7 @@ __device__ __forceinline__ void partial_publish(uint64_t *desc, int slot, uint32
 
 template <class T>
 __device__ __forceinline__ T partial_wait(const uint64_t *desc, int slot, uint32_t epoch) {
+  epoch = partial_meta(epoch);
   uint64_t w0;
   while ((uint32_t)(w0 = ld_relaxed_u64(desc + 2 * slot)) != epoch) __builtin_amdgcn_s_sleep(1);
   if constexpr (sizeof(T) == 4) {

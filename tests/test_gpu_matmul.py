@@ -110,3 +110,19 @@ def test_ragged_shapes_through_padded_operands(ctx, t, tol):
             out.free()
         ev = [e for e in json.loads(c.report())["events"] if e["name"] == "segmap_matmul"]
         assert [e["details"]["padded"] for e in ev] == [p for *_, p in shapes], ev
+
+
+def test_padded_operands_with_more_than_65535_rows(ctx):
+    """K beyond the 65535 a launch grid's second dimension holds, and off the
+    k-step: the copy into padded operands must walk rows, not give a launch error."""
+    b, M, N, K = 1, 300, 260, 70001
+    Ain, Bin, Af, Bf, kind = _inputs("f16", b, M, N, K, 68)
+    out = ctx.call("bmm_f16", ["f32_3d"], ctx.new(kind, Ain), ctx.new(kind, Bin))
+    got = out.values()
+    assert got.shape == (b, M, N)
+    _check(got, Af, Bf, 1e-2)
+    # M beyond it as well (f32, tall and thin, large enough for the padded path)
+    b, M, N, K = 1, 70003, 250, 60
+    Ain, Bin, Af, Bf, kind = _inputs("f32", b, M, N, K, 69)
+    got = ctx.call("bmm_f32", ["f32_3d"], ctx.new(kind, Ain), ctx.new(kind, Bin)).values()
+    _check(got, Af, Bf, 1e-5)

@@ -393,3 +393,26 @@ def test_more_than_2p31_elements(ctx):
     assert got.shape == (n,)
     assert np.array_equal(got, want)
     out.free(); a.free()
+
+
+@pytest.mark.parametrize("t", ["i32", "i64"])
+def test_reduce_after_scans_on_one_scratch(segops_lib, t):
+    """Scans and reductions of a context share the look-back scratch and its
+    epoch counter.  A scan of many tiles at epoch 1 leaves final descriptor words
+    ending in 8*1+2; eight one-block calls advance the epoch to 10 = 8*1+2
+    without touching those slots.  The many-block reduction that follows must
+    not take the stale scan words for partials of its own."""
+    from futhark_amd import Context
+    n = 1 << 22
+    xs = _data(t, n, 41)
+    small = _data(t, 100, 42)
+    for pad in range(0, 10):  # the colliding epoch, and its neighbours
+        with Context(segops_lib) as c:
+            a, s = c.new(f"{t}_1d", xs), c.new(f"{t}_1d", small)
+            out = c.call(f"scan_add_{t}", [f"{t}_1d"], a)
+            assert np.array_equal(out.values()[-5:], oracle.scan("add", t, xs)[-5:])
+            out.free()
+            for _ in range(pad):
+                assert c.call(f"reduce_add_{t}", [NP[t]], s) == oracle.reduce("add", t, small)
+            for _ in range(3):
+                assert c.call(f"reduce_add_{t}", [NP[t]], a) == oracle.reduce("add", t, xs), pad
