@@ -16,6 +16,8 @@
 //   * descriptors carry a launch epoch, so no kernel clears them between calls;
 //   * the look-back window is a full 64-lane wave with several descriptors per
 //     lane.
+#include <mutex>
+
 #include "dispatch.hip.h"
 
 namespace fa {
@@ -135,7 +137,11 @@ enum { SEG_NONE = 0, SEG_FLAGS = 1, SEG_ROWS = 2 };
 template <class T, class Op, int SEGKIND, bool EXCL>
 __global__ __launch_bounds__(scan_block<T>()) void segscan_kernel(
     const T *__restrict__ xs, const uint8_t *__restrict__ flags, int64_t n, T *__restrict__ out,
-    uint32_t *ticket, uint64_t *desc, uint32_t epoch, int64_t num_tiles, int64_t seg_len) {
+    uint32_t *ticket, uint64_t *desc, uint32_t epoch, const uint32_t *epoch_dev, int64_t num_tiles,
+    int64_t seg_len) {
+  // The epoch of this launch: an argument, or (for callers whose launches may
+  // be replayed with the same arguments) a word a preceding kernel advanced.
+  if (epoch_dev != nullptr) epoch = *epoch_dev;
   constexpr bool SEG = SEGKIND != SEG_NONE;
   constexpr bool FLAGS = SEGKIND == SEG_FLAGS;
   constexpr int VEC = Vec16<T>::N;
@@ -465,7 +471,7 @@ template <class T> static int64_t scan_num_tiles(int64_t n) {
 template <class T, class Op>
 static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int64_t seg_len,
                        int64_t n, int exclusive, void *out, void *scratch, size_t scratch_bytes,
-                       uint32_t epoch) {
+                       uint32_t epoch, const uint32_t *epoch_dev = nullptr) {
   if (n == 0) return 0;
   const int64_t tiles = scan_num_tiles<T>(n);
   if (scratch_bytes < SCAN_HEADER_BYTES + (size_t)tiles * SCAN_DESC_BYTES) return FA_ESCRATCH;
@@ -478,7 +484,7 @@ static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int6
   const dim3 grid((unsigned)tiles), block(scan_block<T>());
 #define FA_LAUNCH(SEGV, EXV)                                                              \
   hipLaunchKernelGGL((segscan_kernel<T, Op, SEGV, EXV>), grid, block, 0, s, (const T *)xs, \
-                     flags, n, (T *)out, ticket, desc, epoch, tiles, seg_len)
+                     flags, n, (T *)out, ticket, desc, epoch, epoch_dev, tiles, seg_len)
   if (seg_len > 0) {
     if (exclusive) FA_LAUNCH(SEG_ROWS, true);
     else FA_LAUNCH(SEG_ROWS, false);
@@ -493,7 +499,96 @@ static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int6
   return launch_status();
 }
 
+// ---- scratch for the entry point that allocates nothing
+constexpr size_t SCAN_STATIC_BYTES = 256 * 1024;
+constexpr int SCAN_STATIC_EPOCH_WORD = 16;  // 32-bit word of the header that holds the epoch
+
 }  // namespace fa
+
+// Look-back scratch of fa_segscan_static: ticket counter, epoch word and tile
+// descriptors.  Every GPU the library runs on holds its own copy, zero at
+// load time, until the process ends.
+static __device__ __align__(256) unsigned char static_scratch[fa::SCAN_STATIC_BYTES];
+
+namespace fa {
+
+// Advances the epoch word; before it would wrap, clears the descriptors.  One block.
+__global__ __launch_bounds__(256) void scan_static_epoch_kernel(uint32_t *header, uint64_t *desc,
+                                                                int words) {
+  const uint32_t next = header[SCAN_STATIC_EPOCH_WORD] + 1u;
+  const bool wrap = next >= (1u << 28);
+  if (wrap)
+    for (int i = threadIdx.x; i < words; i += blockDim.x) desc[i] = 0ull;
+  __syncthreads();
+  if (threadIdx.x == 0) header[SCAN_STATIC_EPOCH_WORD] = wrap ? 1u : next;
+}
+
+// Device address of `static_scratch` on the current device (in host code the array's
+// name is only a handle for this query).
+static int scan_static_scratch(void **out) {
+  constexpr int MAX_DEVICES = 64;
+  static std::mutex mu;
+  static void *ptrs[MAX_DEVICES];
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAX_DEVICES) return FA_EINVAL;
+  std::lock_guard<std::mutex> guard(mu);
+  if (ptrs[dev] == nullptr) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(static_scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return FA_EINVAL;
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return 0;
+}
+
+template <class T, class Op>
+static int launch_scan_static(hipStream_t s, const void *xs, const uint8_t *flags, int64_t n,
+                              int exclusive, void *out, void *base) {
+  uint32_t *header = (uint32_t *)base;
+  uint64_t *desc = (uint64_t *)((char *)base + SCAN_HEADER_BYTES);
+  hipLaunchKernelGGL(scan_static_epoch_kernel, dim3(1), dim3(256), 0, s, header, desc,
+                     (int)((SCAN_STATIC_BYTES - SCAN_HEADER_BYTES) / 8));
+  const int rc = launch_status();
+  if (rc != 0) return rc;
+  return launch_scan<T, Op>(s, xs, flags, (int64_t)0, n, exclusive, out, base, SCAN_STATIC_BYTES, 1u,
+                            header + SCAN_STATIC_EPOCH_WORD);
+}
+
+}  // namespace fa
+
+extern "C" int64_t fa_segscan_static_max_n(fa_dtype t) {
+  const size_t es = dtype_size(t);
+  if (es != 4 && es != 8) return 0;
+  const int64_t tile = (es == 4) ? scan_tile_elems<int32_t>() : scan_tile_elems<int64_t>();
+  return (int64_t)((SCAN_STATIC_BYTES - SCAN_HEADER_BYTES) / SCAN_DESC_BYTES) * tile;
+}
+
+extern "C" int fa_segscan_static_init(void) {
+  void *base = nullptr;
+  return scan_static_scratch(&base);
+}
+
+extern "C" int fa_segscan_static(fa_stream_t stream, fa_dtype t, fa_op op, const void *xs,
+                                 const uint8_t *flags, int64_t n, int exclusive, void *out) {
+  if (n < 0 || (n > 0 && (xs == nullptr || out == nullptr))) return FA_EINVAL;
+  const size_t es = dtype_size(t);
+  if (es != 4 && es != 8) return FA_ENOTSUP;
+  if (n > fa_segscan_static_max_n(t)) return FA_ESCRATCH;  // beyond what the fixed scratch holds
+  if (n == 0) return 0;
+  void *base = nullptr;
+  const int rc = scan_static_scratch(&base);
+  if (rc != 0) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (t == FA_I32X2)
+    return op == FA_COMPOSE
+               ? launch_scan_static<AffineI32, OpCompose>(s, xs, flags, n, exclusive, out, base)
+               : FA_ENOTSUP;
+  FA_DISPATCH_TYPE_OP(launch_scan_static, t, op, s, xs, flags, n, exclusive, out, base);
+}
 
 extern "C" size_t fa_segscan_scratch_bytes(fa_dtype t, int64_t n) {
   const size_t es = dtype_size(t);

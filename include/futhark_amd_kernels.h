@@ -172,6 +172,22 @@ int fa_segscan_rows(fa_stream_t stream, fa_dtype t, fa_op op,
                     const void *xss, int64_t m, int64_t k, int exclusive,
                     void *out, void *scratch, size_t scratch_bytes, uint32_t epoch);
 
+/* fa_segscan for callers that cannot allocate or pass a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
+ * has no counterpart in the reference.  The look-back scratch is a fixed
+ * 256 KiB array inside the library (one copy per GPU, held until the process
+ * ends), its epoch lives in that array and is advanced on the device, so
+ * identical launches may be repeated.  No device memory is allocated or
+ * freed.  n beyond fa_segscan_static_max_n(t) returns FA_ESCRATCH.  All calls
+ * on one GPU share the array: calls that overlap in time on one GPU race.
+ * fa_segscan_static_init() resolves the array's address on the current device
+ * ahead of the first call (which otherwise does it). */
+int64_t fa_segscan_static_max_n(fa_dtype t);
+int fa_segscan_static_init(void);
+int fa_segscan_static(fa_stream_t stream, fa_dtype t, fa_op op,
+                      const void *xs, const uint8_t *flags, int64_t n, int exclusive,
+                      void *out);
+
 /* Irregular segmented reduction (Pass/Flatten/Builtins.hs:582-602):
  *   out[i] = lens[i] == 0 ? ne : segscan(flags-from-offsets, vs)[offsets[i]+lens[i]-1]
  * computed without materialising the scan.  Segments must be in order and
