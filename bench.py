@@ -291,25 +291,97 @@ def run_via_server(name: str, steps: int, warmup: int):
 
 
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (scaled by the same
-# counters on a 256 MiB copy); the runs and their commands are in profiles/<kernel>_<workload>.txt.
-MEASURED_TRAFFIC_BYTES = {
-    "segscan_add_f32_2p26": 605.3e6,
-    "scan_add_f32_2p26": 538.6e6,
-    "reduce_add_f32_2p26": 268.5e6,
-    "segred_add_f32_2p26": 277.3e6,
-    "segreduce_add_f32_1048576x64": 273.7e6,
-    "hist_add_i32_H256_uniform_2p27": 1074.2e6,
-    "hist_add_i32_H65536_uniform_2p27": 1107.6e6,
-    "hist_add_i32_H4194304_uniform_2p27": 4229.0e6,
-    "sort_u32_2p26": 3827.6e6,
-    "scanrows_add_f32_65536x1024": 539.1e6,
-    "hist_max_f32_H256_uniform_2p27": 1074.5e6,
-    "transpose_f32_8192x8192": 537.6e6,
-    "vecreduce_add_f32_65536x1024": 269.5e6,
-    "hist_add_f32_H256_uniform_2p27": 1074.2e6,
-    "rbivec_add_i32_H256x16_2p23": 612.4e6,
-    "rbi2d_add_i32_16x16_2p27": 2911.9e6,
-}
+# counters on a 256 MiB copy).  The figure is read from the summary of that run,
+# profiles/<kernel>_<workload>.txt, which ends its traffic section with a line
+# "TRAFFIC_BYTES_PER_STEP <workload> <bytes>"; a workload without such a summary reports null.
+def measured_traffic_bytes(workload: str):
+    for f in sorted((ROOT / "profiles").glob("*.txt")):
+        for line in f.read_text().splitlines():
+            p = line.split()
+            if len(p) == 3 and p[0] == "TRAFFIC_BYTES_PER_STEP" and p[1] == workload:
+                return float(p[2])
+    return None
+
+
+# What the default run measures besides the headline workload: every BASELINE configuration at
+# its full size (reduce / scan / segmented reduce at 2^26, histograms at 2^27 into 256, 65 536 and
+# 2^22 bins, both sorts at 2^26, the matmuls of config 4) and the MFMA rate this GPU sustains on
+# registers alone, which bounds what a matmul kernel can reach here.
+SUITE = [
+    "reduce_add_f32_2p26", "scan_add_f32_2p26", "scan_add_i32_2p24", "reduce_add_i32_2p24",
+    "segred_add_f32_2p26", "segscan_add_i64_2p26",
+    "hist_add_i32_H256_uniform_2p27", "hist_add_i32_H65536_uniform_2p27",
+    "hist_add_i32_H4194304_uniform_2p27", "hist_add_i32_H4194304_zipf_2p27",
+    "hist_add_f32_H256_uniform_2p27", "hist_add_f32_H256_zipf_2p27", "hist_max_f32_H65536_uniform_2p27",
+    "sort_u32_2p26", "sort_u64i32_2p26",
+    "bmm_f16_1x4096", "bmm_bf16_1x4096", "bmm_f32_1x4096", "bmm_f16_64x512", "bmm_f32_64x512",
+]
+
+
+def measure(ctx, w, steps: int, warmup: int, prewarm_seconds: float):
+    """Times one workload.  Two loops of the same K steps: the first with profiling paused gives
+    the wall time per step (`ms_per_step`, what `value` is computed from); the second records a HIP
+    event pair around every launch on the context's stream and is timed by the wall clock as well
+    (`ms_per_step_profiled`), so that the mean event interval of the dominant kernel (`kernel_us`)
+    and a wall time over the very same steps stand side by side."""
+    step = w["step"]
+    ctx.L.futhark_context_pause_profiling(ctx.ptr)
+    t_pre = time.perf_counter()
+    while time.perf_counter() - t_pre < prewarm_seconds:
+        for _ in range(10):
+            step()
+        ctx.sync()
+    for _ in range(warmup):
+        step()
+    ctx.sync()
+
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    ctx.sync()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / steps
+
+    ctx.report()  # drop whatever was recorded before
+    ctx.L.futhark_context_unpause_profiling(ctx.ptr)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    ctx.sync()
+    ms_profiled = (time.perf_counter() - t0) * 1e3 / steps
+    ctx.L.futhark_context_pause_profiling(ctx.ptr)
+    report = json.loads(ctx.report())
+    durs = [e["duration"] for e in report["events"] if e["name"] == w["kernel"]]
+    # events of one step (a step may launch the kernel more than once: count per step)
+    per_step = len(durs) / steps if durs else 0
+    kernel_us = float(np.sum(durs)) / steps if durs else float("nan")
+    kernel_us_min = float(np.min(durs)) * per_step if durs else float("nan")
+    kernel_us_ci95 = (float(1.96 * np.std(durs, ddof=1) / np.sqrt(len(durs))) * per_step
+                      if len(durs) > 1 else 0.0)
+
+    if w["bound"] == "hbm":
+        work, unit, peak, scale = w["bytes"], "GB/s", HBM_PEAK_GBS, 1e9
+    else:
+        work, unit, peak, scale = w["flops"], "TFLOP/s", MFMA_PEAK_TFLOPS[w["dtype"]], 1e12
+    value = work / (ms_per_step * 1e-3) / scale
+    achieved = work / (kernel_us * 1e-6) / scale
+    return {
+        "value": round(value, 3), "unit": unit, "ms_per_step": round(ms_per_step, 5),
+        "ms_per_step_profiled": round(ms_profiled, 5), "work": work,
+        "roofline": {"bound": w["bound"], "achieved": round(achieved, 3), "peak": peak,
+                     "unit": unit, "frac": round(achieved / peak, 4),
+                     "traffic": measured_traffic_bytes(w["name"]),
+                     "kernel": w["kernel"], "kernel_us": round(kernel_us, 3),
+                     "kernel_us_min": round(kernel_us_min, 3),
+                     "kernel_us_ci95": round(kernel_us_ci95, 3)},
+    }
+
+
+def release(ctx, w) -> None:
+    """Frees a workload's resident inputs and what the pool kept for it."""
+    for a in w.get("keep", []):
+        a.free()
+    w.clear()
+    ctx.clear_caches()
 
 
 def main() -> None:
@@ -330,6 +402,11 @@ def main() -> None:
                          "scan/reduce/segscan/segred workloads only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--no-suite", action="store_true",
+                    help="measure the named workload only (profiling runs); by default the "
+                         "other BASELINE configurations are measured after it and reported "
+                         "under `suite` in the same JSON line")
+    ap.add_argument("--suite-steps", type=int, default=20)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run the plain copy kernel (fa_copy, 256 MiB) a few times, so "
                          "that a rocprofv3 --pmc run of this command holds a dispatch of known "
@@ -344,47 +421,8 @@ def main() -> None:
     ctx = Context(profiling=True)
     ctx.L.futhark_context_pause_profiling(ctx.ptr)
     w = make_workload(args.workload, ctx)
-    step = w["step"]
-
-    t_pre = time.perf_counter()
-    while time.perf_counter() - t_pre < args.prewarm_seconds:
-        for _ in range(10):
-            step()
-        ctx.sync()
-    for _ in range(args.warmup):
-        step()
-    ctx.sync()
-
-    # Timed region 1: whole-job throughput, wall clock around K steps.
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    ctx.sync()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-
-    # Timed region 2: the same K steps with a HIP event pair around every kernel
-    # launch, recorded on the context's stream (futhark_context_report).
-    ctx.L.futhark_context_unpause_profiling(ctx.ptr)
-    for _ in range(args.steps):
-        step()
-    ctx.sync()
-    report = json.loads(ctx.report())
-    durs = [e["duration"] for e in report["events"] if e["name"] == w["kernel"]]
-    kernel_us = float(np.mean(durs)) if durs else float("nan")
-    kernel_us_min = float(np.min(durs)) if durs else float("nan")
-    kernel_us_ci95 = float(1.96 * np.std(durs, ddof=1) / np.sqrt(len(durs))) if len(durs) > 1 else 0.0
-
-    if w["bound"] == "hbm":
-        work, unit, peak = w["bytes"], "GB/s", HBM_PEAK_GBS
-        value = work / (ms_per_step * 1e-3) / 1e9
-        achieved = work / (kernel_us * 1e-6) / 1e9
-        metric = "achieved GB/s"
-    else:
-        work, unit, peak = w["flops"], "TFLOP/s", MFMA_PEAK_TFLOPS[w["dtype"]]
-        value = work / (ms_per_step * 1e-3) / 1e12
-        achieved = work / (kernel_us * 1e-6) / 1e12
-        metric = "achieved TFLOP/s"
+    w["name"] = args.workload
+    m = measure(ctx, w, args.steps, args.warmup, args.prewarm_seconds)
 
     cpu = None
     if not args.no_cpu_baseline and "cpu" in w:
@@ -424,26 +462,51 @@ def main() -> None:
         for _ in range(5):
             assert k.fa_copy(ctx.stream, dst.device_ptr, src.device_ptr, nbytes) == 0
         ctx.sync()
+        src.free()
+        dst.free()
 
+    bound, dtype, describe = w["bound"], w["dtype"], w["describe"]
+    elements = w.get("elements")
+    metric = "achieved GB/s" if bound == "hbm" else "achieved TFLOP/s"
     out = {
         "metric": f"{metric} ({args.workload}), 1xMI355X",
-        "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 5), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": w["dtype"], "data": "synthetic",
-        "config": {"workload": w["describe"], "name": args.workload,
-                   "algorithmic_bytes_per_step" if w["bound"] == "hbm" else "flop_per_step": work,
-                   **({"elements_per_s": round(w["elements"] / (ms_per_step * 1e-3), 1)}
-                      if "elements" in w else {})},
-        "roofline": {"bound": w["bound"], "achieved": round(achieved, 3), "peak": peak,
-                     "unit": unit, "frac": round(achieved / peak, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "kernel": w["kernel"], "kernel_us": round(kernel_us, 3),
-                     "kernel_us_min": round(kernel_us_min, 3),
-                     "kernel_us_ci95": round(kernel_us_ci95, 3)},
+        "value": m["value"], "unit": m["unit"], "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": m["ms_per_step"],
+        "ms_per_step_profiled": m["ms_per_step_profiled"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": dtype, "data": "synthetic",
+        "config": {"workload": describe, "name": args.workload,
+                   "algorithmic_bytes_per_step" if bound == "hbm" else "flop_per_step": m["work"],
+                   **({"elements_per_s": round(elements / (m["ms_per_step"] * 1e-3), 1)}
+                      if elements else {})},
+        "roofline": m["roofline"],
         "cpu_baseline": cpu,
     }
     if server is not None:
         out["server"] = server
+
+    if not args.no_suite:
+        release(ctx, w)
+        suite = {}
+        for name in SUITE:
+            if name == args.workload:
+                continue
+            t_w = time.perf_counter()
+            sw = make_workload(name, ctx)
+            sw["name"] = name
+            sm = measure(ctx, sw, args.suite_steps, 3, 0.3 if sw["bound"] == "mfma" else 0.1)
+            entry = {"value": sm["value"], "unit": sm["unit"], "ms_per_step": sm["ms_per_step"],
+                     "ms_per_step_profiled": sm["ms_per_step_profiled"], "dtype": sw["dtype"],
+                     "workload": sw["describe"], "work_per_step": sm["work"],
+                     "roofline": sm["roofline"]}
+            if "elements" in sw:
+                entry["elements_per_s"] = round(sw["elements"] / (sm["ms_per_step"] * 1e-3), 1)
+            suite[name] = entry
+            release(ctx, sw)
+            print(f"[bench] {name}: {sm['value']} {sm['unit']}, kernel {sm['roofline']['kernel_us']} us, "
+                  f"frac {sm['roofline']['frac']} ({time.perf_counter() - t_w:.1f} s)",
+                  file=sys.stderr, flush=True)
+        out["suite"] = suite
+        out["suite_steps"] = args.suite_steps
     print(json.dumps(out))
     ctx.close()
 

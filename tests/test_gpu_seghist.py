@@ -99,10 +99,13 @@ def test_config3_full_size_i32(ctx, H, dist):
         h.free()
 
 
-@pytest.mark.parametrize("H", [256, 65536])
-def test_config3_full_size_f32(ctx, H):
+@pytest.mark.parametrize("H", [256, 65536, 1 << 22])
+@pytest.mark.parametrize("dist", ["uniform", "zipf"])
+def test_config3_full_size_f32(ctx, H, dist):
+    """f32 (+) and f32 max at 2^27 for every bin count and index distribution of the
+    configuration: max bit-exact, sums within 1e-5 of the f64-accumulated oracle."""
     n = 1 << 27
-    is_ = dg.hist_indices(48, n, H, "uniform")
+    is_ = dg.hist_indices(48, n, H, dist)
     ws = dg.uniform_f32(50, n)
     i, w = ctx.new("i32_1d", is_), ctx.new("f32_1d", ws)
     out = ctx.call("hist_max_f32", ["f32_1d"], H, i, w)
@@ -111,6 +114,12 @@ def test_config3_full_size_f32(ctx, H):
     out = ctx.call("hist_add_f32", ["f32_1d"], H, i, w)
     got, ref = out.values(), oracle.hist("add", "f32", H, is_, ws, "f64acc")
     assert np.all(np.abs(got - ref) <= 1e-5 * np.abs(ref))
+    # size-independent property: the bins add up to the sum of the in-range weights
+    ok = (is_ >= 0) & (is_ < H)
+    total = float(ws[ok].astype(np.float64).sum())
+    assert abs(float(got.astype(np.float64).sum()) - total) <= 1e-5 * total
+    for h in (i, w, out):
+        h.free()
 
 
 # ------------------------------------------------------------ segmented histograms
