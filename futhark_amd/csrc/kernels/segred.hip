@@ -29,7 +29,9 @@ constexpr int SEGRED_BLOCK = 1024;
 // (2^24 elements: 15.7 us for 2 and more).
 constexpr int SEGRED_UNROLL = 2;
 constexpr int SEGRED_MAX_GRID = 1024;
-constexpr size_t SEGRED_HEADER_BYTES = 256;
+// The header is shared with the scan kernel (its ticket counters live in the
+// first 8 KiB of the same scratch buffer); partials follow it.
+constexpr size_t SEGRED_HEADER_BYTES = 8192;
 
 static int segred_grid_limit() {
   static int limit = 0;
