@@ -29,14 +29,13 @@
 
 namespace fa {
 
-// Descriptors per lane in a look-back window of 64 lanes.  The look-back of a
-// tile starts a round after its predecessors published their aggregates, so
-// the first window finds them; wider windows measured slower (more loads per
-// round trip: 2^26 f32, 1 -> 99 us, 2 -> 105 us, 4 -> 121 us).
-#ifndef FA_SCAN_LB
-#define FA_SCAN_LB 1
-#endif
-constexpr int SCAN_LB = FA_SCAN_LB;
+// Look-back windows are one descriptor per lane, 64 tiles.  Two or four per
+// lane (128 or 256 tiles per round trip) measured slower on 2^26 f32 (93 ->
+// 100 -> 121 us), narrower first windows (8, 16, 32 tiles) no faster.
+//
+// Cache policy, measured on 2^26 f32 with flags: values are loaded with the
+// default policy (non-temporal: scan 93 -> 108 us), flag bytes non-temporal
+// (default: 113 instead of 98 us), results stored non-temporal (default: 119).
 
 constexpr uint32_t ST_X = 0;  // nothing published
 constexpr uint32_t ST_A = 1;  // aggregate of the tile
@@ -53,10 +52,7 @@ constexpr uint32_t ST_P = 2;  // inclusive prefix up to the end of the tile
 // long as at least that many blocks get to run at the same time, which the
 // number (8) is small enough for: a block occupies one CU.
 constexpr size_t SCAN_HEADER_BYTES = 8192;
-#ifndef FA_SCAN_COUNTERS
-#define FA_SCAN_COUNTERS 8
-#endif
-constexpr int SCAN_MAX_COUNTERS = FA_SCAN_COUNTERS;
+constexpr int SCAN_MAX_COUNTERS = 8;
 constexpr int SCAN_COUNTER_STRIDE = 64;  // in 32-bit words
 constexpr size_t SCAN_DESC_BYTES = 16;
 
@@ -176,11 +172,19 @@ template <class T> constexpr int ss_buffer_bytes(bool flags) {
 // 16 bytes per lane from global memory straight into LDS: lane l's data lands
 // at lds_addr + 16 l.  The compiler does not know of this load; whoever reads
 // the bytes waits for vmcnt first.
+// NT selects the non-temporal cache policy.
+template <bool NT>
 __device__ __forceinline__ void ss_load_to_lds(const void *gaddr, uint32_t lds_addr) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(
-                   __builtin_amdgcn_readfirstlane(lds_addr)),
-               "v"(gaddr)
-               : "memory");
+  if constexpr (NT)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(
+                     __builtin_amdgcn_readfirstlane(lds_addr)),
+                 "v"(gaddr)
+                 : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(
+                     __builtin_amdgcn_readfirstlane(lds_addr)),
+                 "v"(gaddr)
+                 : "memory");
 }
 
 // Waits until at most `younger` vector memory operations of this wave are
@@ -290,21 +294,17 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
     bool ticket_drawn = false;
     auto look_back = [&](int64_t tile) -> Pair {
       Pair acc = {Op::identity(), 0u};
-      // The window is SCAN_LB descriptors per lane, 64 * SCAN_LB tiles.
-      int64_t j = tile - 1;  // newest tile of the window
+      // A window is the `width` tiles up to tile j, one descriptor per lane, in
+      // the highest lanes.
+      int64_t j = tile - 1;
+      int width = WAVE;
       while (true) {
-        const int64_t first_idx = j - (int64_t)(WAVE * SCAN_LB - 1) + (int64_t)lane * SCAN_LB;
-        // Fold this lane's descriptors in tile order; one with a published
-        // prefix (or a segment start) restarts the fold.  All descriptors of
-        // the lane are requested before any is examined, so a window costs one
-        // round trip however many the lane holds.
-        uint32_t st[SCAN_LB], fg[SCAN_LB];
-        T v[SCAN_LB];
-        bool ok[SCAN_LB];
-        DescWords raw[SCAN_LB];
-#pragma unroll
-        for (int k = 0; k < SCAN_LB; k++)
-          raw[k] = first_idx + k < 0 ? DescWords{0ull, 0ull} : desc_load<T>(desc, first_idx + k);
+        const int64_t idx = j - (int64_t)(WAVE - 1 - lane);
+        const bool active = lane >= WAVE - width && idx >= 0;
+        uint32_t st = idx < 0 ? ST_P : ST_A, fg = 0u;  // before tile 0: an empty prefix
+        T v = Op::identity();
+        DescWords raw = {0ull, 0ull};
+        if (active) raw = desc_load<T>(desc, idx);
         // The round's ticket is drawn behind the first window's loads: vector
         // memory operations return in order, and the loads must not wait for
         // the atomic's round trip.
@@ -312,35 +312,17 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
           if (lane == 0) drawn = atomicAdd(ticket, 1u);
           ticket_drawn = true;
         }
-#pragma unroll
-        for (int k = 0; k < SCAN_LB; k++) {
-          st[k] = ST_P;
-          fg[k] = 0u;
-          v[k] = Op::identity();
-          ok[k] = first_idx + k < 0 || desc_decode<T>(raw[k], epoch, st[k], fg[k], v[k]);
-        }
-#pragma unroll
-        for (int k = 0; k < SCAN_LB; k++) {
-          while (!ok[k]) {
+        if (active) {
+          while (!desc_decode<T>(raw, epoch, st, fg, v)) {
             __builtin_amdgcn_s_sleep(1);
-            ok[k] = desc_decode<T>(desc_load<T>(desc, first_idx + k), epoch, st[k], fg[k], v[k]);
+            raw = desc_load<T>(desc, idx);
           }
         }
-        Pair part = {Op::identity(), 0u};
-        bool term = false;
-#pragma unroll
-        for (int k = 0; k < SCAN_LB; k++) {
-          const Pair e = {v[k], SEG ? fg[k] : 0u};
-          if (st[k] == ST_P) {
-            part = e;
-          } else {
-            if constexpr (SEG) part = seg_apply<T, Op>(part, e);
-            else part.v = Op::apply(part.v, v[k]);
-          }
-          term = term || (st[k] == ST_P) || (SEG && fg[k]);
-        }
+        // A published prefix (or, in a segmented scan, a segment start) ends the
+        // walk: lanes before the last such lane do not count.
+        const bool term = lane >= WAVE - width && (st == ST_P || (SEG && fg));
         const uint64_t mask = __ballot(term);
-        Pair mine = part;
+        Pair mine = {v, SEG ? fg : 0u};
         if (mask) {
           const int first = 63 - __builtin_clzll(mask);
           if (lane < first) {
@@ -359,7 +341,8 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
           acc.v = Op::apply(win.v, acc.v);
         }
         if (mask) break;
-        j -= WAVE * SCAN_LB;
+        j -= width;
+        width = WAVE;
       }
       return acc;
     };
@@ -485,7 +468,7 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
       const int m = 8 * wave + j;
       const int off = (8 * m + io_thread) * SS_THREAD_BYTES + io_unit[j & 1] * 16;
       if (dma) {
-        ss_load_to_lds(src + off, lds_base + b * BUFFER + m * 1024);
+        ss_load_to_lds<false>(src + off, lds_base + b * BUFFER + m * 1024);
       } else {
         const int64_t idx = t0 + off / (int)sizeof(T);
         Vec16<T> v;
@@ -510,7 +493,7 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
         }
         const int foff = fbase + thread_in_wave * EPT + half * 16;
         if (dma) {
-          ss_load_to_lds(flags + t0 + foff, lds_base + b * BUFFER + SS_TILE_BYTES + fbase + q * 1024);
+          ss_load_to_lds<true>(flags + t0 + foff, lds_base + b * BUFFER + SS_TILE_BYTES + fbase + q * 1024);
         } else {
           V4 w4;
 #pragma unroll
