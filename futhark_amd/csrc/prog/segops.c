@@ -237,17 +237,14 @@ static int do_reduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
   uint32_t epoch = 0;
   void *scratch = rts_scan_scratch(ctx, fa_segred_scratch_bytes(t), &epoch);
   if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
-  struct memblock_device res = {0};
-  int err = rts_memblock_alloc(ctx, &res, (int64_t)es, "reduce.res");
-  if (err != 0) return err;
+  /* The kernel stores the one result into the context's pinned host slot. */
   struct rts_event *ev = rts_kernel_begin(
       ctx, "segred_nonseg", rts_msgprintf("{\"n\":%lld,\"bytes\":%lld}", (long long)n,
                                           (long long)(n * (int64_t)es)));
-  int code = fa_segred_nonseg(ctx->stream, t, op, in->mem.mem, n, res.mem, scratch,
+  int code = fa_segred_nonseg(ctx->stream, t, op, in->mem.mem, n, ctx->scalar_stage, scratch,
                               ctx->scan_scratch_bytes, epoch);
-  err = rts_kernel_end(ctx, ev, "segred_nonseg", code);
-  if (err == 0) err = rts_copy_d2h(ctx, out, res.mem, es);
-  rts_memblock_unref(ctx, &res, "reduce.res");
+  int err = rts_kernel_end(ctx, ev, "segred_nonseg", code);
+  if (err == 0) err = rts_take_scalar(ctx, out, es);
   return err;
 }
 

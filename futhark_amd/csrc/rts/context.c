@@ -244,6 +244,9 @@ static int backend_setup(struct futhark_context *ctx) {
   hipStream_t s;
   if (hip_check(ctx, hipStreamCreate(&s), "hipStreamCreate") != 0) return 1;
   ctx->stream = (void *)s;
+  if (hip_check(ctx, hipHostMalloc(&ctx->scalar_stage, 256, hipHostMallocDefault),
+                "hipHostMalloc (scalar slot)") != 0)
+    return 1;
   if (ctx->logging) {
     fprintf(ctx->log, "Device: %s, %d CUs, %zu B LDS per block, %zu B L2, %s memory\n",
             ctx->device_name, ctx->num_cus, ctx->max_shared_memory, ctx->l2_cache_bytes,
@@ -387,6 +390,13 @@ int rts_copy_d2h(struct futhark_context *ctx, void *dst, const void *src, size_t
   if (bytes == 0) return 0;
   return hip_check(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost,
                                        (hipStream_t)ctx->stream), "hipMemcpyAsync (D2H)");
+}
+int rts_take_scalar(struct futhark_context *ctx, void *dst, size_t bytes) {
+  if (bytes > 256) return 1;
+  int err = hip_check(ctx, hipStreamSynchronize((hipStream_t)ctx->stream), "hipStreamSynchronize");
+  if (err != 0) return err;
+  memcpy(dst, ctx->scalar_stage, bytes);
+  return 0;
 }
 int rts_copy_d2d(struct futhark_context *ctx, void *dst, const void *src, size_t bytes) {
   if (bytes == 0) return 0;
@@ -577,6 +587,7 @@ void futhark_context_free(struct futhark_context *ctx) {
   if (ctx->stream != NULL) {
     (void)hipStreamSynchronize((hipStream_t)ctx->stream);
     if (ctx->scan_scratch) (void)hipFree(ctx->scan_scratch);
+    if (ctx->scalar_stage) (void)hipHostFree(ctx->scalar_stage);
     (void)rts_gpu_free_all(ctx);
     (void)hipStreamDestroy((hipStream_t)ctx->stream);
   }

@@ -163,6 +163,12 @@ struct futhark_context {
   size_t scan_scratch_bytes;
   uint32_t scan_epoch;
 
+  /* a pinned host slot (hipHostMalloc, 256 bytes) the device can write: a kernel
+   * that produces one scalar stores it here, and the entry point hands it to
+   * the caller after the stream has drained, without a copy operation
+   * (a copy into pageable memory costs about 20 us per call). */
+  void *scalar_stage;
+
   /* deferred error from an asynchronous call, reported at the next sync */
   int pending_error;
 };
@@ -188,6 +194,8 @@ int rts_memblock_set(struct futhark_context *ctx, struct memblock_device *lhs,
 /* copies on the context's stream; asynchronous (hip.h:790-862) */
 int rts_copy_h2d(struct futhark_context *ctx, void *dst, const void *src, size_t bytes);
 int rts_copy_d2h(struct futhark_context *ctx, void *dst, const void *src, size_t bytes);
+/* waits for the stream, then copies `bytes` (at most 256) from the pinned scalar slot to dst */
+int rts_take_scalar(struct futhark_context *ctx, void *dst, size_t bytes);
 int rts_copy_d2d(struct futhark_context *ctx, void *dst, const void *src, size_t bytes);
 int rts_memset0(struct futhark_context *ctx, void *dst, size_t bytes);
 
