@@ -247,6 +247,46 @@ def make_workload(name: str, ctx):
             ctx.call("transpose_f32", ["f32_2d"], x).free()
         w.update(step=step, bytes=2 * rows * cols * 4, kernel="map_transpose_4b", dtype=t, bound="hbm",
                  keep=[x], describe=f"transpose of [{rows}][{cols}]{t} (map_transpose_4b)")
+    elif name.startswith("mfma_peak_"):
+        # mfma_peak_f16: registers-only MFMA rate on operands distributed like bmm_*_1x4096's
+        import ctypes as C
+        from futhark_amd import lib_path
+        t = name.split("_")[2]
+        m = 4096
+        vals = dg.normal_f32(64, 4096, 1.0 / np.sqrt(m))
+        bits = dg.to_f16_bits(vals) if t == "f16" else dg.to_bf16_bits(vals)
+        ops = ctx.new("u16_1d", bits)
+        sink = ctx.new("f32_1d", np.zeros(4, np.float32))
+        k = C.CDLL(str(lib_path("libfuthark_amd_kernels.so")))
+        k.fa_mfma_probe.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p,
+                                    C.POINTER(C.c_double)]
+        hip = C.CDLL("libamdhip64.so")
+        blocks, iters = 256, 2000
+        flop = C.c_double(0.0)
+        code = {"f16": 6, "bf16": 7}[t]
+        ev0, ev1 = C.c_void_p(), C.c_void_p()
+        assert hip.hipEventCreate(C.byref(ev0)) == 0 and hip.hipEventCreate(C.byref(ev1)) == 0
+        durations = []
+
+        def step():
+            timed = not w.get("paused", True)
+            if timed:
+                hip.hipEventRecord(ev0, C.c_void_p(ctx.stream))
+            rc = k.fa_mfma_probe(ctx.stream, code, ops.device_ptr, blocks, iters, sink.device_ptr,
+                                 C.byref(flop))
+            assert rc == 0, rc
+            if timed:
+                hip.hipEventRecord(ev1, C.c_void_p(ctx.stream))
+                hip.hipEventSynchronize(ev1)
+                ms = C.c_float(0.0)
+                hip.hipEventElapsedTime(C.byref(ms), ev0, ev1)
+                durations.append(ms.value * 1e3)
+        step()
+        ctx.sync()
+        w.update(step=step, flops=flop.value, kernel="mfma_probe", dtype=t, bound="mfma",
+                 keep=[ops, sink], own_events=durations,
+                 describe=f"registers-only MFMA 32x32x16 {t} (f32 accumulate), {blocks} blocks x 4 waves x "
+                          f"{iters} rounds of 16 MFMAs, operands N(0,1)/sqrt({m})")
     else:
         raise SystemExit(f"unknown workload {name}")
     return w
@@ -315,6 +355,7 @@ SUITE = [
     "hist_add_f32_H256_uniform_2p27", "hist_add_f32_H256_zipf_2p27", "hist_max_f32_H65536_uniform_2p27",
     "sort_u32_2p26", "sort_u64i32_2p26",
     "bmm_f16_1x4096", "bmm_bf16_1x4096", "bmm_f32_1x4096", "bmm_f16_64x512", "bmm_f32_64x512",
+    "mfma_peak_f16", "mfma_peak_bf16",
 ]
 
 
@@ -343,14 +384,19 @@ def measure(ctx, w, steps: int, warmup: int, prewarm_seconds: float):
 
     ctx.report()  # drop whatever was recorded before
     ctx.L.futhark_context_unpause_profiling(ctx.ptr)
+    w["paused"] = False
     t0 = time.perf_counter()
     for _ in range(steps):
         step()
     ctx.sync()
     ms_profiled = (time.perf_counter() - t0) * 1e3 / steps
+    w["paused"] = True
     ctx.L.futhark_context_pause_profiling(ctx.ptr)
     report = json.loads(ctx.report())
     durs = [e["duration"] for e in report["events"] if e["name"] == w["kernel"]]
+    if "own_events" in w:  # a workload outside the program library times its launches itself
+        durs = list(w["own_events"])
+        del w["own_events"][:]
     # events of one step (a step may launch the kernel more than once: count per step)
     per_step = len(durs) / steps if durs else 0
     kernel_us = float(np.sum(durs)) / steps if durs else float("nan")

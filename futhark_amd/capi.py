@@ -129,6 +129,12 @@ class Segops:
         L.futhark_entry_scan_compose_i32.argtypes = [vp, pp, vp]
         L.futhark_entry_exscan_compose_i32.argtypes = [vp, pp, vp]
         L.futhark_entry_segscan_compose_i32.argtypes = [vp, pp, vp, vp]
+        L.futhark_entry_reduce_argmax_i32.argtypes = [vp, pp, vp]
+        L.futhark_entry_scan_argmax_i32.argtypes = [vp, pp, vp]
+        L.futhark_entry_hist_argmax_i32.argtypes = [vp, pp, i64, vp, vp]
+        L.futhark_entry_reduce_compose_i32.argtypes = [vp, pp, vp]
+        L.futhark_entry_sumsq_f32.argtypes = [vp, vp, vp]
+        L.futhark_entry_scan_norm_f32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u64.argtypes = [vp, pp, vp]
         for name, (k, v) in OPAQUE_PAIRS.items():

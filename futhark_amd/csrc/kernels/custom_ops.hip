@@ -1,0 +1,152 @@
+// Per-program operators: SegOps instantiated with operators and fused maps
+// that are not in the library's fixed set, written against the public
+// template header alone (include/futhark_amd_segops.hpp).  Each stands for
+// what the reference's code generators emit when a program brings its own
+// lambda:
+//   * an operator over a tuple -- argmax over (value, index) pairs, reduce and
+//     scan (tuples in SegBinOps: src/Futhark/IR/SegOp.hs:138-155);
+//   * a map fused in front of a reduction -- reduce (+) 0 (map (\x -> x*x) xs),
+//     and argmax over zip xs (iota n), where the pair is made on the way in;
+//   * maps fused on both sides of a scan (the SegPostOp of
+//     SegScan/SinglePass.hs:841-876) -- map sqrt (scan (+) 0 (map (\x -> x*x) xs));
+//   * a reduction whose operator does not commute (SegRed.hs:836-921) --
+//     composition of affine maps;
+//   * reduce_by_index with a tuple operator, which has to lock its bins
+//     (ImpGen/GPU/Base.hs:769-842) -- argmax per bin.
+#include "futhark_amd_segops.hpp"
+
+namespace {
+
+using namespace fa;
+
+// (value, index) under "the larger value wins, the smaller index among equal
+// values": commutative and associative; neutral (lowest, highest).
+struct ValIdx {
+  int32_t v, i;
+};
+struct OpArgmax {
+  static constexpr bool commutative = true;
+  static __host__ __device__ __forceinline__ ValIdx identity() { return ValIdx{INT32_MIN, INT32_MAX}; }
+  static __host__ __device__ __forceinline__ ValIdx apply(ValIdx a, ValIdx b) {
+    const bool take_a = a.v > b.v || (a.v == b.v && a.i < b.i);
+    return take_a ? a : b;
+  }
+};
+struct ZipIndex {  // zip xs (iota n)
+  static __device__ __forceinline__ ValIdx apply(int32_t x, int64_t i) { return ValIdx{x, (int32_t)i}; }
+};
+struct PairAsIs {
+  static __device__ __forceinline__ ValIdx apply(ValIdx p, int64_t) { return p; }
+};
+struct AffineAsIs {
+  static __device__ __forceinline__ AffineI32 apply(AffineI32 f, int64_t) { return f; }
+};
+struct SquareF32 {
+  static __device__ __forceinline__ float apply(float x, int64_t) { return x * x; }
+  static __device__ __forceinline__ float apply(float x) { return x * x; }
+};
+struct SqrtF32 {
+  static __device__ __forceinline__ float apply(float x) { return __builtin_sqrtf(x); }
+};
+
+// The same operator on the {a, b} pair the locked histogram works with.
+struct ValIdxAB {
+  int32_t a, b;
+};
+struct OpArgmaxAB {
+  static constexpr bool commutative = true;
+  static __host__ __device__ __forceinline__ ValIdxAB identity() { return ValIdxAB{INT32_MIN, INT32_MAX}; }
+  static __host__ __device__ __forceinline__ ValIdxAB apply(ValIdxAB x, ValIdxAB y) {
+    const bool take_x = x.a > y.a || (x.a == y.a && x.b < y.b);
+    return take_x ? x : y;
+  }
+};
+struct ZipIndexAB {
+  static __device__ __forceinline__ ValIdxAB apply(int32_t x, int64_t i) { return ValIdxAB{x, (int32_t)i}; }
+};
+
+// [H][2]i32 from the two component arrays.
+__global__ void zip_pairs_kernel(const int32_t *a, const int32_t *b, int32_t *out, int64_t H) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < H) {
+    out[2 * i] = a[i];
+    out[2 * i + 1] = b[i];
+  }
+}
+__global__ void unzip_pairs_kernel(const int32_t *in, int32_t *a, int32_t *b, int64_t H) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < H) {
+    a[i] = in[2 * i];
+    b[i] = in[2 * i + 1];
+  }
+}
+
+}  // namespace
+
+extern "C" int fa_reduce_argmax_i32(fa_stream_t stream, const int32_t *xs, int64_t n, int32_t *out2,
+                                    void *scratch, size_t scratch_bytes, uint32_t epoch) {
+  return launch_reduce<int32_t, ValIdx, ZipIndex, OpArgmax>((hipStream_t)stream, xs, n, (ValIdx *)out2,
+                                                            scratch, scratch_bytes, epoch);
+}
+
+extern "C" int fa_reduce_compose_i32(fa_stream_t stream, const int32_t *abs, int64_t n, int32_t *out2,
+                                     void *scratch, size_t scratch_bytes, uint32_t epoch) {
+  if (!is_aligned(abs, 8)) return FA_EALIGN;
+  return launch_reduce<AffineI32, AffineI32, AffineAsIs, OpCompose>(
+      (hipStream_t)stream, (const AffineI32 *)abs, n, (AffineI32 *)out2, scratch, scratch_bytes, epoch);
+}
+
+extern "C" int fa_sumsq_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
+                            void *scratch, size_t scratch_bytes, uint32_t epoch) {
+  return launch_reduce<float, float, SquareF32, OpAdd<float>>((hipStream_t)stream, xs, n, out, scratch,
+                                                              scratch_bytes, epoch);
+}
+
+extern "C" int fa_scan_argmax_i32(fa_stream_t stream, const int32_t *pairs, const uint8_t *flags,
+                                  int64_t n, int exclusive, int32_t *out, void *scratch,
+                                  size_t scratch_bytes, uint32_t epoch) {
+  if (n < 0 || (n > 0 && (pairs == nullptr || out == nullptr || scratch == nullptr))) return FA_EINVAL;
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
+  return launch_scan<ValIdx, OpArgmax>((hipStream_t)stream, pairs, flags, (int64_t)0, n, exclusive, out,
+                                       scratch, scratch_bytes, epoch);
+}
+
+extern "C" int fa_scan_norm_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
+                                void *scratch, size_t scratch_bytes, uint32_t epoch) {
+  if (n < 0 || (n > 0 && (xs == nullptr || out == nullptr || scratch == nullptr))) return FA_EINVAL;
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
+  return launch_scan<float, OpAdd<float>, SquareF32, SqrtF32>((hipStream_t)stream, xs, nullptr,
+                                                              (int64_t)0, n, 0, out, scratch,
+                                                              scratch_bytes, epoch);
+}
+
+extern "C" size_t fa_hist_argmax_workspace_bytes(int64_t H) {
+  if (H < 0) return 0;
+  return (size_t)(3 * H) * 4 + 256;  // two component arrays and the lock words
+}
+
+extern "C" int64_t fa_hist_argmax_max_bins(void) { return HL_MAX_BINS; }
+
+// dest: [H][2]i32 (value, index) pairs, updated in place.
+extern "C" int fa_hist_argmax_i32(fa_stream_t stream, const int32_t *is, const int32_t *xs, int64_t n,
+                                  int32_t *dest, int64_t H, void *workspace, size_t workspace_bytes) {
+  if (n < 0 || H < 0 || H > HL_MAX_BINS) return FA_EINVAL;
+  if (H == 0) return 0;
+  if (dest == nullptr || workspace == nullptr || (n > 0 && (is == nullptr || xs == nullptr)))
+    return FA_EINVAL;
+  if (workspace_bytes < fa_hist_argmax_workspace_bytes(H)) return FA_ESCRATCH;
+  hipStream_t st = (hipStream_t)stream;
+  int32_t *a = (int32_t *)workspace, *b = a + H;
+  uint32_t *locks = (uint32_t *)(b + H);
+  const dim3 grid((unsigned)ceil_div(H, (int64_t)256));
+  hipLaunchKernelGGL(unzip_pairs_kernel, grid, dim3(256), 0, st, dest, a, b, H);
+  int rc = launch_status();
+  if (rc != 0) return rc;
+  rc = fa_replicate(stream, 4, locks, H, 0);
+  if (rc != 0) return rc;
+  rc = launch_hist_locked<int32_t, int32_t, int32_t, ValIdxAB, ZipIndexAB, OpArgmaxAB, int32_t>(
+      st, is, xs, n, a, b, locks, H);
+  if (rc != 0) return rc;
+  hipLaunchKernelGGL(zip_pairs_kernel, grid, dim3(256), 0, st, a, b, dest, H);
+  return launch_status();
+}

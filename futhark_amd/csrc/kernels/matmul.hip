@@ -667,6 +667,60 @@ extern "C" int fa_matmul_ws(fa_stream_t stream, fa_dtype in_t, const void *A, co
   return launch_status();
 }
 
+// ------------------------------------------------------------ MFMA rate probe
+// What the matrix cores sustain on registers alone: every wave loads one A and
+// one B fragment (16 bytes each) from `operands` and then issues `iters` rounds
+// of 16 independent 32x32x16 MFMAs into 256 accumulator registers, the inner
+// tile of matmul16_kernel without its loads and LDS reads.  The figure depends
+// on the operand values (power management lowers the clock when the multiplier
+// inputs toggle), so the caller supplies operands distributed like its
+// matrices.  One 256-thread block per CU and launch.
+namespace fa {
+template <bool BF16>
+__global__ __launch_bounds__(256) void mfma_probe_kernel(const uint16_t *__restrict__ operands,
+                                                         int iters, float *sink) {
+  using Frag = __attribute__((ext_vector_type(4))) uint32_t;
+  const Frag a = reinterpret_cast<const Frag *>(operands)[threadIdx.x];
+  const Frag b = reinterpret_cast<const Frag *>(operands)[256 + threadIdx.x];
+  f32x16 acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[i][e] = 0.0f;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+      if constexpr (BF16)
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bit_cast<bf16x8>(a), bit_cast<bf16x8>(b), acc[i], 0, 0, 0);
+      else
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bit_cast<f16x8>(a), bit_cast<f16x8>(b), acc[i], 0, 0, 0);
+    }
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 16; i++)
+#pragma unroll
+    for (int e = 0; e < 16; e++) s += acc[i][e];
+  if (s == 12345.678f) sink[0] = s;  // keeps the loop alive
+}
+}  // namespace fa
+
+extern "C" int fa_mfma_probe(fa_stream_t stream, fa_dtype in_t, const void *operands, int blocks,
+                             int iters, float *sink, double *flop) {
+  if (in_t != FA_F16 && in_t != FA_BF16) return FA_ENOTSUP;
+  if (operands == nullptr || sink == nullptr || blocks < 1 || iters < 1) return FA_EINVAL;
+  if (!is_aligned(operands, 16)) return FA_EALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  if (in_t == FA_F16)
+    hipLaunchKernelGGL((mfma_probe_kernel<false>), dim3(blocks), dim3(256), 0, st,
+                       (const uint16_t *)operands, iters, sink);
+  else
+    hipLaunchKernelGGL((mfma_probe_kernel<true>), dim3(blocks), dim3(256), 0, st,
+                       (const uint16_t *)operands, iters, sink);
+  if (flop != nullptr) *flop = (double)blocks * 4.0 * iters * 16.0 * (2.0 * 32 * 32 * 16);
+  return launch_status();
+}
+
 extern "C" int fa_matmul(fa_stream_t stream, fa_dtype in_t, const void *A, const void *B, float *C,
                          int64_t batch, int64_t M, int64_t N, int64_t K) {
   return matmul_direct(stream, in_t, A, B, C, batch, M, N, K);

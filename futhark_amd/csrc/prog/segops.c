@@ -707,6 +707,156 @@ int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhar
   return ret;
 }
 
+/* ---- SegOps with operators and fused maps of their own (per-program lambdas):
+ * instantiated in csrc/kernels/custom_ops.hip from the public kernel templates. */
+
+/* A reduction to one element; `dev_out` is where the kernel stores it. */
+typedef int (*custom_reduce_fn)(fa_stream_t, const void *, int64_t, void *, void *, size_t, uint32_t);
+static int do_custom_reduce(struct futhark_context *ctx, custom_reduce_fn fn, const char *name,
+                            const struct fut_array *in, int64_t n, void *dev_out) {
+  uint32_t epoch = 0;
+  void *scratch = rts_scan_scratch(ctx, fa_segred_scratch_bytes(FA_I64), &epoch);
+  if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
+  struct rts_event *ev = rts_kernel_begin(ctx, name, rts_msgprintf("{\"n\":%lld}", (long long)n));
+  int code = fn(ctx->stream, in->mem.mem, n, dev_out, scratch, ctx->scan_scratch_bytes, epoch);
+  return rts_kernel_end(ctx, ev, name, code);
+}
+static int reduce_argmax_fn(fa_stream_t s, const void *xs, int64_t n, void *out, void *sc, size_t sb,
+                            uint32_t e) {
+  return fa_reduce_argmax_i32(s, (const int32_t *)xs, n, (int32_t *)out, sc, sb, e);
+}
+static int reduce_compose_fn(fa_stream_t s, const void *xs, int64_t n, void *out, void *sc, size_t sb,
+                             uint32_t e) {
+  return fa_reduce_compose_i32(s, (const int32_t *)xs, n, (int32_t *)out, sc, sb, e);
+}
+static int sumsq_fn(fa_stream_t s, const void *xs, int64_t n, void *out, void *sc, size_t sb,
+                    uint32_t e) {
+  return fa_sumsq_f32(s, (const float *)xs, n, (float *)out, sc, sb, e);
+}
+
+/* A reduction whose result is a pair of i32, returned as a [2]i32 array. */
+static int do_pair_reduce(struct futhark_context *ctx, custom_reduce_fn fn, const char *name,
+                          struct fut_array **out, const struct fut_array *in) {
+  const int64_t two = 2;
+  struct fut_array *res = out_array(ctx, 8, 1, &two, "pair.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  int err = do_custom_reduce(ctx, fn, name, in, in->shape[0], res->mem.mem);
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
+int futhark_entry_reduce_argmax_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
+                                    const struct futhark_i32_1d *in0) {
+  ENTER(ctx);
+  int ret = do_pair_reduce(ctx, reduce_argmax_fn, "segred_argmax", (struct fut_array **)out0, &in0->a);
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_reduce_compose_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
+                                     const struct futhark_i32_2d *in0) {
+  ENTER(ctx);
+  int ret = in0->a.shape[1] != 2
+                ? bad_sizes(ctx, "reduce_compose_i32")
+                : do_pair_reduce(ctx, reduce_compose_fn, "segred_compose", (struct fut_array **)out0,
+                                 &in0->a);
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_sumsq_f32(struct futhark_context *ctx, float *out0, const struct futhark_f32_1d *in0) {
+  ENTER(ctx);
+  int ret = do_custom_reduce(ctx, sumsq_fn, "segred_sumsq", &in0->a, in0->a.shape[0], ctx->scalar_stage);
+  if (ret == 0) ret = rts_take_scalar(ctx, out0, 4);
+  LEAVE(ctx);
+  return ret;
+}
+
+static int do_custom_scan(struct futhark_context *ctx, struct fut_array **out,
+                          const struct fut_array *in, int norm, const char *entry) {
+  const int64_t n = in->shape[0];
+  if (!norm && in->shape[1] != 2) return bad_sizes(ctx, entry);
+  uint32_t epoch = 0;
+  const size_t sbytes = fa_segscan_scratch_bytes(norm ? FA_F32 : FA_I64, n);
+  void *scratch = rts_scan_scratch(ctx, sbytes, &epoch);
+  if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
+  struct fut_array *res = out_array(ctx, n * (norm ? 4 : 8), norm ? 1 : 2, in->shape, "scan.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  struct rts_event *ev = rts_kernel_begin(ctx, "segscan", rts_msgprintf("{\"n\":%lld}", (long long)n));
+  int code = norm ? fa_scan_norm_f32(ctx->stream, (const float *)in->mem.mem, n, (float *)res->mem.mem,
+                                     scratch, ctx->scan_scratch_bytes, epoch)
+                  : fa_scan_argmax_i32(ctx->stream, (const int32_t *)in->mem.mem, NULL, n, 0,
+                                       (int32_t *)res->mem.mem, scratch, ctx->scan_scratch_bytes, epoch);
+  int err = rts_kernel_end(ctx, ev, "segscan", code);
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
+int futhark_entry_scan_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                  const struct futhark_i32_2d *in0) {
+  ENTER(ctx);
+  int ret = do_custom_scan(ctx, (struct fut_array **)out0, &in0->a, 0, "scan_argmax_i32");
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_scan_norm_f32(struct futhark_context *ctx, struct futhark_f32_1d **out0,
+                                const struct futhark_f32_1d *in0) {
+  ENTER(ctx);
+  int ret = do_custom_scan(ctx, (struct fut_array **)out0, &in0->a, 1, "scan_norm_f32");
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_hist_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                  const int64_t in0, const struct futhark_i32_1d *in1,
+                                  const struct futhark_i32_1d *in2) {
+  ENTER(ctx);
+  int ret = 0;
+  const int64_t k = in0, n = in1->a.shape[0];
+  if (in2->a.shape[0] != n) {
+    ret = bad_sizes(ctx, "hist_argmax_i32");
+  } else if (k < 0 || k > fa_hist_argmax_max_bins()) {
+    rts_set_error(ctx, rts_msgprintf("hist_argmax_i32: between 0 and %lld bins, got %lld\n",
+                                     (long long)fa_hist_argmax_max_bins(), (long long)k));
+    ret = FUTHARK_PROGRAM_ERROR;
+  } else {
+    const int64_t shape[2] = {k, 2};
+    struct fut_array *res = out_array(ctx, k * 8, 2, shape, "hist.out");
+    if (res == NULL) {
+      ret = FUTHARK_OUT_OF_MEMORY;
+    } else {
+      /* every bin starts as the neutral pair (i32.lowest, i32.highest) */
+      const uint64_t ne = ((uint64_t)(uint32_t)INT32_MAX << 32) | (uint32_t)INT32_MIN;
+      struct memblock_device ws = {0};
+      ret = rts_memblock_alloc(ctx, &ws, (int64_t)fa_hist_argmax_workspace_bytes(k), "hist.workspace");
+      if (ret == 0) {
+        struct rts_event *ev = rts_kernel_begin(
+            ctx, "seghist_locked", rts_msgprintf("{\"n\":%lld,\"bins\":%lld}", (long long)n, (long long)k));
+        int code = fa_replicate(ctx->stream, 8, res->mem.mem, k, ne);
+        if (code == 0)
+          code = fa_hist_argmax_i32(ctx->stream, (const int32_t *)in1->a.mem.mem,
+                                    (const int32_t *)in2->a.mem.mem, n, (int32_t *)res->mem.mem, k,
+                                    ws.mem, (size_t)ws.size);
+        ret = rts_kernel_end(ctx, ev, "seghist_locked", code);
+        rts_memblock_unref(ctx, &ws, "hist.workspace");
+      }
+      if (ret != 0) drop_array(ctx, res);
+      else *out0 = (struct futhark_i32_2d *)res;
+    }
+  }
+  LEAVE(ctx);
+  return ret;
+}
+
 #define DEFINE_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(DEFINE_SEGOP_ENTRIES, T, CT)
 FUTHARK_FOR_EACH_NUM_TYPE(DEFINE_FOR_TYPE)
 #define DEFINE_BITOPS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(DEFINE_SEGOP_ENTRIES, T, CT)

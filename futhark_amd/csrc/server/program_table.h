@@ -233,6 +233,25 @@ static int e_scan_compose_i32(struct futhark_context *c, struct value *o, struct
 static int e_exscan_compose_i32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_exscan_compose_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]));
 }
+static int e_reduce_argmax_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_reduce_argmax_i32(c, (struct futhark_i32_1d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_scan_argmax_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_scan_argmax_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_hist_argmax_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_hist_argmax_i32(c, (struct futhark_i32_2d **)&o->u.arr, i[0]->u.i64,
+                                       ARRP(i[1]), ARRP(i[2]));
+}
+static int e_reduce_compose_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_reduce_compose_i32(c, (struct futhark_i32_1d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_sumsq_f32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_sumsq_f32(c, &o->u.f32, ARRP(i[0]));
+}
+static int e_scan_norm_f32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_scan_norm_f32(c, (struct futhark_f32_1d **)&o->u.arr, ARRP(i[0]));
+}
 static int e_segscan_compose_i32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_segscan_compose_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]),
                                            ARRP(i[1]));
@@ -321,6 +340,12 @@ static const struct entry entries[] = {
     {"exscan_compose_i32", e_exscan_compose_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
     {"segscan_compose_i32", e_segscan_compose_i32, "[][]i32", 1, 2, {"[]u8", "[][]i32"}, {0},
      {NULL}},
+    {"reduce_argmax_i32", e_reduce_argmax_i32, "[]i32", 1, 1, {"[]i32"}, {0}, {NULL}},
+    {"scan_argmax_i32", e_scan_argmax_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
+    {"hist_argmax_i32", e_hist_argmax_i32, "[][]i32", 1, 3, {"i64", "[]i32", "[]i32"}, {0}, {NULL}},
+    {"reduce_compose_i32", e_reduce_compose_i32, "[]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
+    {"sumsq_f32", e_sumsq_f32, "f32", 0, 1, {"[]f32"}, {0}, {NULL}},
+    {"scan_norm_f32", e_scan_norm_f32, "[]f32", 1, 1, {"[]f32"}, {0}, {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {MATMUL_PARAM, NULL}},
     {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {MATMUL_PARAM, NULL}},
     {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {NULL}},

@@ -73,6 +73,12 @@ def entry_points() -> dict:
         _entry("scan_compose_i32", "[][]i32", [("abs", "[][]i32")]),
         _entry("exscan_compose_i32", "[][]i32", [("abs", "[][]i32")]),
         _entry("segscan_compose_i32", "[][]i32", [("flags", "[]u8"), ("abs", "[][]i32")]),
+        _entry("reduce_argmax_i32", "[]i32", [("xs", "[]i32")]),
+        _entry("scan_argmax_i32", "[][]i32", [("vis", "[][]i32")]),
+        _entry("hist_argmax_i32", "[][]i32", [("k", "i64"), ("is", "[]i32"), ("xs", "[]i32")]),
+        _entry("reduce_compose_i32", "[]i32", [("abs", "[][]i32")]),
+        _entry("sumsq_f32", "f32", [("xs", "[]f32")]),
+        _entry("scan_norm_f32", "[]f32", [("xs", "[]f32")]),
         _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")], [MATMUL_PARAM]),
         _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")], [MATMUL_PARAM]),
         _entry("radix_sort_u32", "[]u32", [("keys", "[]u32")]),

@@ -312,6 +312,51 @@ int fa_replicate(fa_stream_t stream, int elem_bytes, void *dst, int64_t n,
 int fa_iota(fa_stream_t stream, fa_dtype t, void *dst, int64_t n,
             int64_t start, int64_t step);
 
+/* ---------------------------------------------- per-program operators (proofs)
+ * SegOps instantiated from include/futhark_amd_segops.hpp with operators and
+ * fused maps outside the fixed set above (csrc/kernels/custom_ops.hip); they
+ * stand for the kernels the reference generates for a program's own lambdas
+ * (SegBinOp with tuples and SegPostOp, src/Futhark/IR/SegOp.hs:138-155).
+ * Scratch and epoch as for fa_segred_nonseg / fa_segscan.
+ *   argmax on (value, index) pairs of i32: the larger value, the smaller index
+ *   among equal values; neutral (INT32_MIN, INT32_MAX).
+ *   fa_reduce_argmax_i32: over zip xs (iota n), the pair made on the way in; out2: 2 x i32
+ *   fa_scan_argmax_i32:   pairs [n][2]i32 in and out, optionally segmented by flags
+ *   fa_reduce_compose_i32: fold of affine maps (FA_COMPOSE, not commutative) in
+ *                          element order (SegRed.hs:836-921); out2: 2 x i32
+ *   fa_sumsq_f32:         reduce (+) 0 (map (\x -> x*x) xs)
+ *   fa_scan_norm_f32:     map sqrt (scan (+) 0 (map (\x -> x*x) xs))
+ *   fa_hist_argmax_i32:   reduce_by_index with argmax into dest [H][2]i32 (updated
+ *                         in place), bins locked while updated because the tuple's
+ *                         components live in two arrays (ImpGen/GPU/Base.hs:769-842);
+ *                         H <= fa_hist_argmax_max_bins(); workspace of
+ *                         fa_hist_argmax_workspace_bytes(H) bytes, contents irrelevant. */
+int fa_reduce_argmax_i32(fa_stream_t stream, const int32_t *xs, int64_t n, int32_t *out2,
+                         void *scratch, size_t scratch_bytes, uint32_t epoch);
+int fa_scan_argmax_i32(fa_stream_t stream, const int32_t *pairs, const uint8_t *flags, int64_t n,
+                       int exclusive, int32_t *out, void *scratch, size_t scratch_bytes,
+                       uint32_t epoch);
+int fa_reduce_compose_i32(fa_stream_t stream, const int32_t *abs, int64_t n, int32_t *out2,
+                          void *scratch, size_t scratch_bytes, uint32_t epoch);
+int fa_sumsq_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
+                 void *scratch, size_t scratch_bytes, uint32_t epoch);
+int fa_scan_norm_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
+                     void *scratch, size_t scratch_bytes, uint32_t epoch);
+size_t fa_hist_argmax_workspace_bytes(int64_t H);
+int64_t fa_hist_argmax_max_bins(void);
+int fa_hist_argmax_i32(fa_stream_t stream, const int32_t *is, const int32_t *xs, int64_t n,
+                       int32_t *dest, int64_t H, void *workspace, size_t workspace_bytes);
+
+/* Measurement aid (no counterpart in the reference): the rate the matrix cores
+ * sustain on registers alone.  `blocks` blocks of four waves each issue `iters`
+ * rounds of sixteen independent 32x32x16 MFMAs (f16 or bf16 in, f32 accumulate)
+ * on fragments read once from `operands` (8 KiB of 16-bit values, distributed
+ * like the caller's matrices: the sustained clock depends on them).  *flop, if
+ * not NULL, receives the number of floating-point operations of the launch;
+ * `sink` is one float the kernel may write. */
+int fa_mfma_probe(fa_stream_t stream, fa_dtype in_t, const void *operands, int blocks,
+                  int iters, float *sink, double *flop);
+
 /* Plain device copy kernel used for calibration of bandwidth counters. */
 int fa_copy(fa_stream_t stream, void *dst, const void *src, size_t bytes);
 

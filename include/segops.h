@@ -321,6 +321,36 @@ int futhark_entry_exscan_compose_i32(struct futhark_context *ctx, struct futhark
 int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
                                       const struct futhark_u8_1d *in0,
                                       const struct futhark_i32_2d *in1);
+
+/* SegOps whose operator or fused maps are the program's own (kernels
+ * instantiated from include/futhark_amd_segops.hpp):
+ *   def argmax (v1: i32, i1: i32) (v2: i32, i2: i32) =
+ *     if v1 > v2 || (v1 == v2 && i1 < i2) then (v1, i1) else (v2, i2)
+ *   entry reduce_argmax_i32 [n] (xs: [n]i32) : [2]i32 =
+ *     let (v, i) = reduce_comm argmax (i32.lowest, i32.highest) (zip xs (map i32.i64 (iota n)))
+ *     in [v, i]
+ *   entry scan_argmax_i32 (vis: [][2]i32) : [][2]i32 =     -- rows (value, index)
+ *     scan argmax (i32.lowest, i32.highest) (map (\r -> (r[0], r[1])) vis) |> map (\(v, i) -> [v, i])
+ *   entry hist_argmax_i32 (k: i64) (is: []i32) (xs: []i32) : [k][2]i32 =
+ *     hist argmax (i32.lowest, i32.highest) k (map i64.i32 is) (zip xs (map i32.i64 (indices xs)))
+ *     |> map (\(v, i) -> [v, i])                           -- k at most 8192
+ *   entry reduce_compose_i32 (abs: [][2]i32) : [2]i32 =    -- compose as above; does not commute
+ *     let (a, b) = reduce compose (1, 0) (map (\r -> (r[0], r[1])) abs) in [a, b]
+ *   entry sumsq_f32 (xs: []f32) : f32 = reduce (+) 0 (map (\x -> x * x) xs)
+ *   entry scan_norm_f32 (xs: []f32) : []f32 = map f32.sqrt (scan (+) 0 (map (\x -> x * x) xs)) */
+int futhark_entry_reduce_argmax_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
+                                    const struct futhark_i32_1d *in0);
+int futhark_entry_scan_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                  const struct futhark_i32_2d *in0);
+int futhark_entry_hist_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                  const int64_t in0, const struct futhark_i32_1d *in1,
+                                  const struct futhark_i32_1d *in2);
+int futhark_entry_reduce_compose_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
+                                     const struct futhark_i32_2d *in0);
+int futhark_entry_sumsq_f32(struct futhark_context *ctx, float *out0,
+                            const struct futhark_f32_1d *in0);
+int futhark_entry_scan_norm_f32(struct futhark_context *ctx, struct futhark_f32_1d **out0,
+                                const struct futhark_f32_1d *in0);
 int futhark_entry_bmm_bf16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
                            const struct futhark_u16_3d *in0, const struct futhark_u16_3d *in1);
 int futhark_entry_matmul_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,

@@ -153,6 +153,62 @@ def scan_compose_i32(abs_, flags=None, exclusive: bool = False):
     return out
 
 
+def scan_argmax_i32(vis, flags=None, exclusive: bool = False):
+    """scan of (value, index) pairs [n][2]i32 under argmax (larger value, then smaller index)."""
+    vis = _arr(vis, np.int32).reshape(-1, 2)
+    out = np.empty_like(vis)
+    f = None if flags is None else _arr(flags, np.uint8)
+    fn = lib().orc_scan_argmax_i32_lit
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p]
+    fn(None if f is None else _p(f), _p(vis), vis.shape[0], int(exclusive), _p(out))
+    return out
+
+
+def reduce_argmax_i32(xs):
+    """reduce argmax (i32.lowest, i32.highest) (zip xs (iota n)) as [v, i]: the last scan element."""
+    xs = _arr(xs, np.int32)
+    if xs.size == 0:
+        return np.array([np.iinfo(np.int32).min, np.iinfo(np.int32).max], np.int32)
+    vis = np.stack([xs, np.arange(xs.size, dtype=np.int32)], axis=1)
+    return scan_argmax_i32(vis)[-1].copy()
+
+
+def hist_argmax_i32(k: int, is_, xs):
+    """hist argmax ne k is (zip xs (indices xs)) as [k][2]i32."""
+    is_, xs = _arr(is_, np.int32), _arr(xs, np.int32)
+    ii = np.iinfo(np.int32)
+    dest = np.empty((k, 2), np.int32)
+    dest[:, 0], dest[:, 1] = ii.min, ii.max
+    fn = lib().orc_hist_argmax_i32_lit
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64]
+    fn(_p(dest), k, _p(is_), _p(xs), xs.size)
+    return dest
+
+
+def reduce_compose_i32(abs_):
+    """reduce compose (1, 0) abs: the last element of the scan, (1, 0) for no elements."""
+    abs_ = _arr(abs_, np.int32).reshape(-1, 2)
+    if abs_.shape[0] == 0:
+        return np.array([1, 0], np.int32)
+    return scan_compose_i32(abs_)[-1].copy()
+
+
+def sumsq_f32(xs, variant: str = "lit"):
+    """reduce (+) 0 (map (\\x -> x*x) xs): squares in f32, sum sequential in f32 ("lit") or in f64."""
+    xs = _arr(xs, np.float32)
+    sq = xs * xs
+    return reduce("add", "f32", sq, variant)
+
+
+def scan_norm_f32(xs, variant: str = "lit"):
+    """map f32.sqrt (scan (+) 0 (map (\\x -> x*x) xs))."""
+    xs = _arr(xs, np.float32)
+    sq = xs * xs
+    return np.sqrt(scan("add", "f32", sq, variant)).astype(np.float32)
+
+
 def rbi_vec(op: str, t: str, dest, is_, vss):
     """reduce_by_index dest (map2 op) (replicate m ne) is vss on a copy of dest ([H][m])."""
     _, dt = _CT[t]

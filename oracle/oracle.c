@@ -196,6 +196,32 @@ void orc_scan_compose_i32_lit(const uint8_t *flags, const int32_t *abs, int64_t 
   }
 }
 
+/* The argmax operator on (value, index) pairs of i32: the larger value wins,
+ * among equal values the smaller index; neutral (INT32_MIN, INT32_MAX).  Scan,
+ * reduce and reduce_by_index with it are the same left-to-right loops as above
+ * (FirstOrderTransform.hs:505-560 for hist, :613-656 for scan); a tuple is just
+ * two accumulators (the loops carry one variable per component). */
+static void argmax_i32(int32_t *v, int32_t *i, int32_t v2, int32_t i2) {
+  if (!(*v > v2 || (*v == v2 && *i < i2))) { *v = v2; *i = i2; }
+}
+void orc_scan_argmax_i32_lit(const uint8_t *flags, const int32_t *vis, int64_t n, int exclusive,
+                             int32_t *out) {
+  int32_t v = INT32_MIN, ix = INT32_MAX;
+  for (int64_t i = 0; i < n; i++) {
+    if (flags != NULL && flags[i] != 0) { v = INT32_MIN; ix = INT32_MAX; }
+    if (exclusive) { out[2 * i] = v; out[2 * i + 1] = ix; }
+    argmax_i32(&v, &ix, vis[2 * i], vis[2 * i + 1]);
+    if (!exclusive) { out[2 * i] = v; out[2 * i + 1] = ix; }
+  }
+}
+void orc_hist_argmax_i32_lit(int32_t *dest /* [H][2] */, int64_t H, const int32_t *is,
+                             const int32_t *xs, int64_t n) {
+  for (int64_t i = 0; i < n; i++) {
+    const int64_t b = (int64_t)is[i];
+    if (b >= 0 && b < H) argmax_i32(&dest[2 * b], &dest[2 * b + 1], xs[i], (int32_t)i);
+  }
+}
+
 /* hist / reduce_by_index alone for the other integer types */
 #define DEFINE_RBI(OP, S, T)                                                                   \
   void orc_rbi_##OP##_##S##_lit(T *dest, int64_t H, const int32_t *is, const T *vs,            \

@@ -1,0 +1,82 @@
+"""GPU parity for SegOps with a program's own operators and fused maps (the
+kernels of csrc/kernels/custom_ops.hip, instantiated from the public template
+header): tuple operator argmax in reduce, scan and reduce_by_index (bins locked),
+a reduction that does not commute, maps fused before a reduction and on both
+sides of a scan.  Integers bit-exact; f32 within 1e-5 of the f64-accumulated oracle."""
+import numpy as np
+import pytest
+
+import oracle
+from futhark_amd import FutharkError, datagen as dg
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 2, 63, 64, 65, 1023, 4096, 4097, 100003, (1 << 20) + 7, (1 << 24) + 1]
+
+
+def test_reduce_argmax(ctx):
+    for n in SIZES:
+        xs = dg.uniform_int(21, n, -1000, 1000)          # ties are common
+        a = ctx.new("i32_1d", xs)
+        out = ctx.call("reduce_argmax_i32", ["i32_1d"], a)
+        assert out.values().tolist() == oracle.reduce_argmax_i32(xs).tolist(), n
+        a.free(); out.free()
+    # the maximum at the very end, at the very start, and everywhere
+    n = (1 << 22) + 3
+    for where in (n - 1, 0):
+        xs = np.zeros(n, np.int32); xs[where] = 7
+        assert ctx.call("reduce_argmax_i32", ["i32_1d"], ctx.new("i32_1d", xs)).values().tolist() == [7, where]
+    assert ctx.call("reduce_argmax_i32", ["i32_1d"], ctx.new("i32_1d", np.full(n, 5, np.int32))).values().tolist() == [5, 0]
+
+
+def test_scan_argmax(ctx):
+    for n in SIZES[:-1]:
+        xs = dg.uniform_int(22, n, -100000, 100000)
+        vis = np.stack([xs, np.arange(n, dtype=np.int32)], axis=1)
+        a = ctx.new("i32_2d", vis.reshape(n, 2))
+        out = ctx.call("scan_argmax_i32", ["i32_2d"], a)
+        assert np.array_equal(out.values(), oracle.scan_argmax_i32(vis)), n
+        a.free(); out.free()
+    with pytest.raises(FutharkError):
+        ctx.call("scan_argmax_i32", ["i32_2d"], ctx.new("i32_2d", np.zeros((5, 3), np.int32)))
+
+
+def test_reduce_with_an_operator_that_does_not_commute(ctx):
+    rng = np.random.default_rng(3)
+    for n in SIZES:
+        abs_ = rng.integers(-2 ** 31, 2 ** 31, (n, 2)).astype(np.int32)
+        a = ctx.new("i32_2d", abs_.reshape(n, 2))
+        out = ctx.call("reduce_compose_i32", ["i32_1d"], a)
+        assert out.values().tolist() == oracle.reduce_compose_i32(abs_).tolist(), n
+        a.free(); out.free()
+    # swapping two neighbours changes the result, so operand order is really checked
+    abs_ = np.array([[2, 3], [5, 7]], np.int32)
+    assert oracle.reduce_compose_i32(abs_).tolist() != oracle.reduce_compose_i32(abs_[::-1]).tolist()
+
+
+def test_maps_fused_into_reduce_and_scan(ctx):
+    for n in SIZES:
+        xs = (dg.uniform_f32(23, n) * 4 - 2).astype(np.float32)
+        a = ctx.new("f32_1d", xs)
+        got = ctx.call("sumsq_f32", [np.float32], a)
+        want = oracle.sumsq_f32(xs, "f64acc")
+        assert abs(float(got) - float(want)) <= 1e-5 * abs(float(want)) + 1e-30, n
+        out = ctx.call("scan_norm_f32", ["f32_1d"], a)
+        wn = oracle.scan_norm_f32(xs, "f64acc")
+        assert np.all(np.abs(out.values().astype(np.float64) - wn) <= 1e-5 * np.abs(wn) + 1e-30), n
+        a.free(); out.free()
+
+
+def test_hist_with_a_tuple_operator_locks_its_bins(ctx):
+    rng = np.random.default_rng(4)
+    for n, H in [(0, 5), (1, 1), (1000, 7), (100003, 256), ((1 << 22) + 5, 256), ((1 << 22) + 5, 8192),
+                 (300000, 1), (5, 0)]:
+        xs = rng.integers(-50, 50, n).astype(np.int32)           # ties in every bin
+        is_ = dg.hist_indices(24, n, max(H, 1), "zipf") if n else np.zeros(0, np.int32)
+        out = ctx.call("hist_argmax_i32", ["i32_2d"], H, ctx.new("i32_1d", is_), ctx.new("i32_1d", xs))
+        assert out.shape == (H, 2)
+        assert np.array_equal(out.values(), oracle.hist_argmax_i32(H, is_, xs)), (n, H)
+        out.free()
+    with pytest.raises(FutharkError):
+        ctx.call("hist_argmax_i32", ["i32_2d"], 8193, ctx.new("i32_1d", np.zeros(4, np.int32)),
+                 ctx.new("i32_1d", np.zeros(4, np.int32)))

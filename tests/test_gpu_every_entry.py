@@ -41,9 +41,13 @@ def make_inputs(name, e, rng):
         t = el(types[0])
         return [_vals(rng, t, (4, 5)), rng.integers(-1, 5, N).astype(np.int64),
                 rng.integers(-1, 6, N).astype(np.int64), _vals(rng, t, N)]
-    if name.endswith("compose_i32"):
+    if name.endswith("compose_i32") or name == "scan_argmax_i32":
         ab = _vals(rng, "i32", (N, 2))
         return ([(rng.random(N) < 0.2).astype(np.uint8)] if fam == "segscan" else []) + [ab]
+    if name == "hist_argmax_i32":
+        return [np.array(5, np.int64), rng.integers(-1, 7, N).astype(np.int32), _vals(rng, "i32", N)]
+    if name in ("sumsq_f32", "scan_norm_f32"):
+        return [_vals(rng, "f32", N)]
     if fam in ("reduce", "scan", "exscan"):
         return [_vals(rng, el(types[0]), N)]
     if fam == "segscan":

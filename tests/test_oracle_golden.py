@@ -362,3 +362,53 @@ def test_affine_composition_scan_is_the_iterated_map():
     two = np.array([[2, 3], [5, 7]], np.int32)
     assert oracle.scan_compose_i32(two)[1].tolist() == [10, 22]          # 5 * (2x + 3) + 7
     assert oracle.scan_compose_i32(two[::-1])[1].tolist() == [10, 17]    # 2 * (5x + 7) + 3
+
+
+def test_tuple_operator_oracles_are_pinned_by_closed_forms():
+    """argmax on (value, index) pairs and the fused maps: each against what numpy fixes.
+    reduce argmax (zip xs iota) is numpy's argmax (first of equal maxima); the running one
+    is maximum.accumulate with the position of its first occurrence; per bin, the maximum
+    of the bin's values and the first position holding it."""
+    rng = np.random.default_rng(5)
+    for n in (1, 2, 17, 1000, 4099):
+        xs = rng.integers(-50, 50, n).astype(np.int32)      # many ties
+        assert oracle.reduce_argmax_i32(xs).tolist() == [int(xs.max()), int(np.argmax(xs))]
+        vis = np.stack([xs, np.arange(n, dtype=np.int32)], axis=1)
+        sc = oracle.scan_argmax_i32(vis)
+        run = np.maximum.accumulate(xs)
+        assert np.array_equal(sc[:, 0], run)
+        first = np.array([int(np.argmax(xs[:i + 1])) for i in range(n)]) if n <= 1000 else None
+        if first is not None:
+            assert np.array_equal(sc[:, 1], first)
+        ex = oracle.scan_argmax_i32(vis, exclusive=True)
+        assert ex[0].tolist() == [np.iinfo(np.int32).min, np.iinfo(np.int32).max]
+        assert np.array_equal(ex[1:], sc[:-1])
+        flags = (rng.integers(0, 7, n) == 0).astype(np.uint8)
+        seg = oracle.scan_argmax_i32(vis, flags)
+        starts = np.flatnonzero(flags).tolist()
+        bounds = sorted(set([0] + starts + [n]))
+        for a, b in zip(bounds[:-1], bounds[1:]):
+            assert np.array_equal(seg[a:b], oracle.scan_argmax_i32(vis[a:b]))
+        H = 13
+        is_ = rng.integers(-2, H + 2, n).astype(np.int32)
+        h = oracle.hist_argmax_i32(H, is_, xs)
+        for b in range(H):
+            sel = np.flatnonzero(is_ == b)
+            want = [np.iinfo(np.int32).min, np.iinfo(np.int32).max] if sel.size == 0 else \
+                [int(xs[sel].max()), int(sel[np.argmax(xs[sel])])]
+            assert h[b].tolist() == want
+    assert oracle.reduce_argmax_i32(np.zeros(0, np.int32)).tolist() == [-2 ** 31, 2 ** 31 - 1]
+    # the fold of affine maps applied to a probe value is the maps applied one after the other
+    abs_ = rng.integers(-9, 9, (200, 2)).astype(np.int32)
+    a, b = (int(v) for v in oracle.reduce_compose_i32(abs_))
+    x = 12345
+    for fa, fb in abs_.tolist():
+        x = (fa * x + fb) % (1 << 32)
+    assert (a * 12345 + b) % (1 << 32) == x
+    assert oracle.reduce_compose_i32(np.zeros((0, 2), np.int32)).tolist() == [1, 0]
+    # sums of squares and running norms against float64 numpy
+    xs = rng.standard_normal(5000).astype(np.float32)
+    assert abs(float(oracle.sumsq_f32(xs, "f64acc")) - float(np.dot(xs.astype(np.float64), xs.astype(np.float64)))) \
+        <= 1e-6 * float(np.dot(xs.astype(np.float64), xs.astype(np.float64)))
+    want = np.sqrt(np.cumsum(xs.astype(np.float64) ** 2))
+    assert np.all(np.abs(oracle.scan_norm_f32(xs, "f64acc") - want) <= 1e-6 * want)
