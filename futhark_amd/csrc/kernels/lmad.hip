@@ -95,8 +95,11 @@ __global__ __launch_bounds__(256) void transpose_tile_kernel(T *__restrict__ dst
                                                              int64_t rows, int64_t cols) {
   constexpr int TS = 64;
   __shared__ T tile[TS][TS + 1];
-  const int64_t b = blockIdx.z;
-  const int64_t r0 = (int64_t)blockIdx.y * TS, c0 = (int64_t)blockIdx.x * TS;
+  // grid.x enumerates the tiles of one matrix row by row (the second and third
+  // grid dimensions hold 65535 at most), grid.y the matrices of the batch.
+  const int64_t b = blockIdx.y;
+  const int64_t tiles_x = (cols + TS - 1) / TS;
+  const int64_t r0 = ((int64_t)blockIdx.x / tiles_x) * TS, c0 = ((int64_t)blockIdx.x % tiles_x) * TS;
   const T *s = src + b * rows * cols;
   T *d = dst + b * rows * cols;
   const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;  // 64 x 4
@@ -130,8 +133,11 @@ __global__ __launch_bounds__(256) void transpose_tile_vec_kernel(T *__restrict__
   constexpr int LANES = TS / V;         // lanes across one tile row
   constexpr int STEP = 256 / LANES;     // tile rows covered per pass
   __shared__ T tile[TS][TS + 1];
-  const int64_t b = blockIdx.z;
-  const int64_t r0 = (int64_t)blockIdx.y * TS, c0 = (int64_t)blockIdx.x * TS;
+  // grid.x enumerates the tiles of one matrix row by row (the second and third
+  // grid dimensions hold 65535 at most), grid.y the matrices of the batch.
+  const int64_t b = blockIdx.y;
+  const int64_t tiles_x = (cols + TS - 1) / TS;
+  const int64_t r0 = ((int64_t)blockIdx.x / tiles_x) * TS, c0 = ((int64_t)blockIdx.x % tiles_x) * TS;
   const T *s = src + b * rows * cols;
   T *d = dst + b * rows * cols;
   const int tx = threadIdx.x % LANES, ty = threadIdx.x / LANES;
@@ -161,7 +167,14 @@ template <class T>
 static int launch_map_transpose(hipStream_t st, T *dst, const T *src, int64_t batch, int64_t rows,
                                 int64_t cols) {
   if (batch == 0 || rows == 0 || cols == 0) return 0;
-  if (batch > 65535) return FA_EINVAL;
+  if (batch > 65535) {  // the grid's second dimension holds 65535: take the batch in pieces
+    for (int64_t b0 = 0; b0 < batch; b0 += 65535) {
+      const int64_t nb = batch - b0 < 65535 ? batch - b0 : 65535;
+      const int rc = launch_map_transpose<T>(st, dst + b0 * rows * cols, src + b0 * rows * cols, nb, rows, cols);
+      if (rc != 0) return rc;
+    }
+    return 0;
+  }
   if (rows <= 32 || cols <= 32) {
     const bool short_rows = rows <= cols;
     const int64_t longest = short_rows ? cols : rows;
@@ -177,8 +190,8 @@ static int launch_map_transpose(hipStream_t st, T *dst, const T *src, int64_t ba
     return launch_status();
   }
   const int64_t gx = ceil_div(cols, (int64_t)64), gy = ceil_div(rows, (int64_t)64);
-  if (gx > INT32_MAX || gy > 65535) return FA_EINVAL;
-  const dim3 grid((unsigned)gx, (unsigned)gy, (unsigned)batch);
+  if (gx * gy > INT32_MAX) return FA_EINVAL;  // more than 2^43 elements in one matrix
+  const dim3 grid((unsigned)(gx * gy), (unsigned)batch);
   constexpr int V = 16 / (int)sizeof(T);
   if (sizeof(T) >= 4 && rows % V == 0 && cols % V == 0 && is_aligned(dst, 16) &&
       is_aligned(src, 16))

@@ -287,7 +287,10 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
     if (i < tile_n) {
       const K k = kbuf[i];
       dst[j] = s_tab[fn(k, pass)] + (uint32_t)i;
-      kout[dst[j]] = k;
+      // The offsets come from this library's own histogram and scan; should
+      // they ever be wrong, a store outside the output would fault the GPU,
+      // whereas a dropped key is a wrong result the caller can see.
+      if ((int64_t)dst[j] < n) kout[dst[j]] = k;
     }
   }
   if constexpr (VB != 0) {
@@ -302,7 +305,7 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
 #pragma unroll
     for (int j = 0; j < RS_KPT; j++) {
       const int i = j * RS_BLOCK + tid;
-      if (i < tile_n) vout[dst[j]] = vbuf[i];
+      if (i < tile_n && (int64_t)dst[j] < n) vout[dst[j]] = vbuf[i];
     }
   }
 }

@@ -339,6 +339,32 @@ extern "C" size_t fa_segred_irregular_scratch_bytes(fa_dtype t, int64_t n) {
   return sri_scratch_bytes(ceil_div(n, tile));
 }
 
+namespace fa {
+// Segments must be in order, disjoint and inside [0, n): one thread per segment
+// looks at itself and its successor and raises *failure otherwise.
+__global__ __launch_bounds__(256) void segments_check_kernel(const int64_t *__restrict__ offsets,
+                                                             const int64_t *__restrict__ lens,
+                                                             int64_t m, int64_t n, int32_t *failure,
+                                                             int32_t code) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= m) return;
+  const int64_t o = offsets[i], l = lens[i];
+  bool ok = o >= 0 && l >= 0 && o <= n && l <= n - o;
+  if (ok && i + 1 < m) ok = o + l <= offsets[i + 1];
+  if (!ok) *failure = code;
+}
+}  // namespace fa
+
+extern "C" int fa_segments_check(fa_stream_t stream, const int64_t *offsets, const int64_t *lens,
+                                 int64_t m, int64_t n, int32_t *failure, int32_t code) {
+  if (m < 0 || n < 0 || failure == nullptr || (m > 0 && (offsets == nullptr || lens == nullptr)))
+    return FA_EINVAL;
+  if (m == 0) return 0;
+  hipLaunchKernelGGL(fa::segments_check_kernel, dim3((unsigned)ceil_div(m, (int64_t)256)), dim3(256), 0,
+                     (hipStream_t)stream, offsets, lens, m, n, failure, code);
+  return launch_status();
+}
+
 extern "C" int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op, const void *vs,
                                    int64_t n, const int64_t *offsets, const int64_t *lens,
                                    int64_t m, void *out, void *scratch, size_t scratch_bytes) {

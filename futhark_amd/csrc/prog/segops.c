@@ -282,6 +282,14 @@ static int do_segred(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
                      const char *entry) {
   const int64_t m = offsets->shape[0], n = vs->shape[0];
   if (lens->shape[0] != m) return bad_sizes(ctx, entry);
+  /* The kernels are memory-safe whatever the segments are, but their result is
+     only defined for ordered, disjoint segments inside the array: anything
+     else makes the next synchronisation fail, as an index out of bounds does
+     in a compiled program. */
+  int chk = fa_segments_check(ctx->stream, (const int64_t *)offsets->mem.mem,
+                              (const int64_t *)lens->mem.mem, m, n, RTS_FAILURE_WORD(ctx),
+                              RTS_FAILURE_SEGMENTS);
+  if (chk != 0) return rts_kernel_end(ctx, NULL, "segments_check", chk);
   struct fut_array *res = out_array(ctx, m * (int64_t)es, 1, &m, "segred.out");
   if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
   /* Plain workspace from the pool; not the look-back scratch of the scans,
@@ -425,6 +433,10 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
     rts_set_error(ctx, rts_msgprintf("Error: negative histogram size %lld.\n", (long long)k));
     return FUTHARK_PROGRAM_ERROR;
   }
+  if (k > INT64_MAX / (int64_t)es) {
+    rts_set_error(ctx, rts_msgprintf("Error: %lld bins do not fit in memory.\n", (long long)k));
+    return FUTHARK_OUT_OF_MEMORY;
+  }
   struct fut_array *res = out_array(ctx, k * (int64_t)es, 1, &k, "hist.dest");
   if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
   int err = 0;
@@ -464,6 +476,12 @@ static int do_seghist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t 
   if (k < 0) {
     rts_set_error(ctx, rts_msgprintf("Error: negative histogram size %lld.\n", (long long)k));
     return FUTHARK_PROGRAM_ERROR;
+  }
+  /* m * k * es must be a size that exists before anything is done with it */
+  if (m > 0 && k > (INT64_MAX / (int64_t)es) / m) {
+    rts_set_error(ctx, rts_msgprintf("Error: %lld histograms of %lld bins do not fit in memory.\n",
+                                     (long long)m, (long long)k));
+    return FUTHARK_OUT_OF_MEMORY;
   }
   const int64_t dims[2] = {m, k};
   struct fut_array *res = out_array(ctx, m * k * (int64_t)es, 2, dims, "seghist.dest");

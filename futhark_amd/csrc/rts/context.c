@@ -247,6 +247,7 @@ static int backend_setup(struct futhark_context *ctx) {
   if (hip_check(ctx, hipHostMalloc(&ctx->scalar_stage, 256, hipHostMallocDefault),
                 "hipHostMalloc (scalar slot)") != 0)
     return 1;
+  memset(ctx->scalar_stage, 0, 256);
   if (ctx->logging) {
     fprintf(ctx->log, "Device: %s, %d CUs, %zu B LDS per block, %zu B L2, %s memory\n",
             ctx->device_name, ctx->num_cus, ctx->max_shared_memory, ctx->l2_cache_bytes,
@@ -543,6 +544,19 @@ int futhark_context_sync(struct futhark_context *ctx) {
     int p = ctx->pending_error;
     ctx->pending_error = 0;
     return p;
+  }
+  if (ctx->scalar_stage != NULL) {
+    volatile int32_t *failure = RTS_FAILURE_WORD(ctx);
+    const int32_t code = *failure;
+    if (code != 0) {
+      *failure = 0;
+      rts_set_error(ctx, rts_msgprintf(
+          code == RTS_FAILURE_SEGMENTS
+              ? "Error: segments are not in order, overlap or leave the array (offsets[i] + lens[i] "
+                "<= offsets[i+1] <= n required).\n"
+              : "Error: a kernel reported failure %d.\n", (int)code));
+      return FUTHARK_PROGRAM_ERROR;
+    }
   }
   return FUTHARK_SUCCESS;
 }

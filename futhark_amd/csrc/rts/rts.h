@@ -168,6 +168,11 @@ struct futhark_context {
    * the caller after the stream has drained, without a copy operation
    * (a copy into pageable memory costs about 20 us per call). */
   void *scalar_stage;
+  /* a word of that slot (byte 128) kernels raise when the program must fail, as
+   * the reference's global_failure (rts/c/gpu.h): checked and cleared at every
+   * synchronisation, which then returns FUTHARK_PROGRAM_ERROR */
+#define RTS_FAILURE_WORD(ctx) ((int32_t *)((char *)(ctx)->scalar_stage + 128))
+#define RTS_FAILURE_SEGMENTS 1
 
   /* deferred error from an asynchronous call, reported at the next sync */
   int pending_error;

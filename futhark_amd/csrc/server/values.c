@@ -481,8 +481,15 @@ int fv_read_value(FILE *f, const struct fv_primtype *t, int rank, int64_t *shape
 
 int fv_end_of_input(FILE *f) {
   /* blanks and `--` comments may follow the last value (end_of_input,
-   * rts/c/values.h:713-722); whatever else is found stays in the stream */
+   * rts/c/values.h:713-722); whatever else is found stays in the stream.  A `-`
+   * that does not open a comment takes two characters to recognise, and ISO C
+   * promises only one character of push-back: on a stream that can seek, the
+   * position before the `-` is restored instead; on a pipe the second push-back
+   * is left to the C library (glibc keeps it), and should it be refused the
+   * answer is still right, only the `-` is gone from the stream. */
   for (;;) {
+    fpos_t before;
+    const int can_seek = fgetpos(f, &before) == 0;
     int c = getc(f);
     if (c == EOF) return 0;
     if (isspace(c)) continue;
@@ -492,6 +499,7 @@ int fv_end_of_input(FILE *f) {
         while (c2 != EOF && c2 != '\n') c2 = getc(f);
         continue;
       }
+      if (can_seek && fsetpos(f, &before) == 0) return 1;
       if (c2 != EOF) ungetc(c2, f);
     }
     ungetc(c, f);

@@ -201,6 +201,14 @@ int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op,
                         const int64_t *offsets, const int64_t *lens, int64_t m,
                         void *out, void *scratch, size_t scratch_bytes);
 
+/* Checks what fa_segred_irregular requires of its segments (in order, disjoint,
+ * inside [0, n)): stores `code` into *failure (device-visible memory, e.g. a
+ * pinned host word) when they are not, and leaves it alone otherwise.  A
+ * compiled Futhark program reports an out-of-bounds index at the next
+ * synchronisation in the same way (global_failure, rts/c/gpu.h). */
+int fa_segments_check(fa_stream_t stream, const int64_t *offsets, const int64_t *lens,
+                      int64_t m, int64_t n, int32_t *failure, int32_t code);
+
 /* ----------------------------------------------------------------- SegHist
  * `reduce_by_index dest op ne is vs` (prelude/soacs.fut:132-146): for every i
  * with 0 <= is[i] < H, dest[is[i]] = dest[is[i]] op vs[i]; other indices are

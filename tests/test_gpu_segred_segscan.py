@@ -416,3 +416,28 @@ def test_reduce_after_scans_on_one_scratch(segops_lib, t):
                 assert c.call(f"reduce_add_{t}", [NP[t]], s) == oracle.reduce("add", t, small)
             for _ in range(3):
                 assert c.call(f"reduce_add_{t}", [NP[t]], a) == oracle.reduce("add", t, xs), pad
+
+
+def test_segred_reports_segments_that_are_not_segments(segops_lib):
+    """Offsets and lengths that overlap, run backwards or leave the array are an error a
+    compiled program reports at the next synchronisation; good ones right after work."""
+    from futhark_amd import Context, FutharkError
+    n = 1000
+    xs = _data("i32", n, 9)
+    bad_cases = [([0, 10], [20, 5]),          # the first runs into the second
+                 ([50, 10], [5, 5]),          # out of order
+                 ([0, 990], [10, 20]),        # past the end
+                 ([-1, 10], [5, 5]),          # before the start
+                 ([0, 10], [5, -2])]          # a negative length
+    with Context(segops_lib) as c:
+        v = c.new("i32_1d", xs)
+        for offs, lens in bad_cases:
+            o, l = c.new("i64_1d", np.array(offs, np.int64)), c.new("i64_1d", np.array(lens, np.int64))
+            with pytest.raises(FutharkError) as e:
+                out = c.call("segred_add_i32", ["i32_1d"], o, l, v)
+                c.sync()
+            assert e.value.code == 2 and "segments" in e.value.message
+        o, l = c.new("i64_1d", np.array([0, 10, 500], np.int64)), c.new("i64_1d", np.array([10, 0, 500], np.int64))
+        out = c.call("segred_add_i32", ["i32_1d"], o, l, v)
+        c.sync()
+        assert np.array_equal(out.values(), oracle.segred("add", "i32", np.array([0, 10, 500]), np.array([10, 0, 500]), xs))

@@ -159,8 +159,12 @@ def test_map_transpose_shapes(ctx, es):
     k = _K()
     dt = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[es]
     rng = np.random.default_rng(es)
-    for batch, rows, cols in [(1, 1, 1), (1, 64, 64), (3, 65, 127), (2, 1, 5000), (2, 5000, 1),
-                              (1, 17, 4099), (1, 4099, 31), (5, 33, 33), (1, 1000, 1000)]:
+    shapes = [(1, 1, 1), (1, 64, 64), (3, 65, 127), (2, 1, 5000), (2, 5000, 1),
+              (1, 17, 4099), (1, 4099, 31), (5, 33, 33), (1, 1000, 1000)]
+    if es == 4:
+        # more than 65535 tiles down, and more matrices than a launch grid's second dimension holds
+        shapes += [(1, 65536 * 64 + 70, 33), (70001, 3, 5), (65600, 40, 34)]
+    for batch, rows, cols in shapes:
         x = rng.integers(0, 255, (batch, rows, cols)).astype(dt)
         s = ctx.new("u8_1d", x.reshape(-1).view(np.uint8))
         d = ctx.new("u8_1d", np.zeros(x.size * es, np.uint8))
