@@ -73,6 +73,20 @@ static inline int rs_prepare(hipStream_t st, const RsScratch &sc) {
 // element by element.
 constexpr int RS_HIST_TILES = 8;
 
+// h[d] += one for every lane.  Sorted or small keys and skewed histogram
+// indices give most lanes of a wave the same digit, and 64 atomics on one LDS
+// word are taken one after the other (a pass over keys with one digit ran at
+// 183 us against 50 us); so the lanes that share the first lane's digit are
+// counted with a ballot and added once.
+__device__ __forceinline__ void rs_count(uint32_t *h, uint32_t d, uint32_t one) {
+  const uint32_t d0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)d);
+  const uint64_t same = __ballot(d == d0);
+  if (d != d0)
+    atomicAdd(&h[d], one);
+  else if (lane_id() == 0)
+    atomicAdd(&h[d0], one * (uint32_t)__builtin_popcountll(same));
+}
+
 template <class K, class DigitFn>
 __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__ keys, int64_t n,
                                                            DigitFn fn, int pass, uint32_t *counts,
@@ -116,7 +130,7 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__
 #pragma unroll
       for (int r = 0; r < ROWS; r++)
 #pragma unroll
-        for (int e = 0; e < VEC; e++) atomicAdd(&h[i][fn(cur[r].e[e], pass)], one);
+        for (int e = 0; e < VEC; e++) rs_count(&h[i][0], fn(cur[r].e[e], pass), one);
 #pragma unroll
       for (int r = 0; r < ROWS; r++) cur[r] = nxt[r];
     }

@@ -510,21 +510,37 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
     const int nb = (int)((H - bin0) < range_bins ? (H - bin0) : range_bins);
     for (int i = threadIdx.x; i < nb; i += HIST_BLOCK) sh[i] = OpA::identity();
     __syncthreads();
-    int64_t i = lo + threadIdx.x;
-    for (; i + 3 * HIST_BLOCK < hi; i += 4 * HIST_BLOCK) {
-      U b[4];
-      T v[4];
+    auto update = [&](U b, T v) { lds_update<A, OpA>(&sh[(int)((int64_t)b - bin0)], (A)v); };
+    // [lo, hi) = loose elements up to a multiple of four, groups of four read
+    // with 16-byte non-temporal loads (two groups of a thread in flight),
+    // loose elements at the end.
+    int64_t a = (lo + 3) & ~(int64_t)3;
+    if (a > hi) a = hi;
+    for (int64_t i = lo + threadIdx.x; i < a; i += HIST_BLOCK) update(pis[i], pvs[i]);
+    const int64_t groups = (hi - a) / 4;
+    int64_t g = threadIdx.x;
+    for (; g + HIST_BLOCK < groups; g += 2 * HIST_BLOCK) {
+      U b[2][4];
+      T v[2][4];
 #pragma unroll
-      for (int q = 0; q < 4; q++) {
-        b[q] = pis[i + q * HIST_BLOCK];
-        v[q] = pvs[i + q * HIST_BLOCK];
+      for (int q = 0; q < 2; q++) {
+        load_elems4(b[q], pis + a + (g + q * HIST_BLOCK) * 4);
+        load_elems4(v[q], pvs + a + (g + q * HIST_BLOCK) * 4);
       }
 #pragma unroll
-      for (int q = 0; q < 4; q++)
-        lds_update<A, OpA>(&sh[(int)((int64_t)b[q] - bin0)], (A)v[q]);
+      for (int q = 0; q < 2; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) update(b[q][e], v[q][e]);
     }
-    for (; i < hi; i += HIST_BLOCK)
-      lds_update<A, OpA>(&sh[(int)((int64_t)pis[i] - bin0)], (A)pvs[i]);
+    if (g < groups) {
+      U b[4];
+      T v[4];
+      load_elems4(b, pis + a + g * 4);
+      load_elems4(v, pvs + a + g * 4);
+#pragma unroll
+      for (int e = 0; e < 4; e++) update(b[e], v[e]);
+    }
+    for (int64_t i = a + groups * 4 + threadIdx.x; i < hi; i += HIST_BLOCK) update(pis[i], pvs[i]);
     __syncthreads();
     for (int q = threadIdx.x; q < nb; q += HIST_BLOCK) {
       const A acc = sh[q];
