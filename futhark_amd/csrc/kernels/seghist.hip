@@ -398,24 +398,36 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
 // value.  LDS operations of one wave complete in order, so a round sees the
 // writes of the one before.  The 16 histograms of a block are combined at the
 // end and flushed with one device atomic per non-zero bin.
+//
+// A bin with many takers (skewed indices) would need as many rounds as it has
+// lanes; so a wave keeps 2^copies_log2 copies of its histogram where LDS
+// allows, lane l using copy l mod 2^copies_log2, and only lanes of the same
+// copy take turns (H = 256, Zipf indices: 640 -> 382 us per 2^27 pairs).
 template <class T, class I>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
     const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t H,
-    int index_bits) {
+    int index_bits, int copies_log2) {
   extern __shared__ __align__(16) unsigned char s_raw[];
   T *sh = reinterpret_cast<T *>(s_raw);
   constexpr int VEC = 4;
   constexpr int WAVES = HIST_BLOCK / WAVE;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / WAVE));
   const int nb = (int)H;
+  const int copies = 1 << copies_log2;
   // volatile: the compiler must not carry a bin across the rounds below in a register
-  volatile T *mine = sh + (size_t)wave * nb;
-  for (int i = threadIdx.x; i < nb * WAVES; i += HIST_BLOCK) sh[i] = T(0);
+  volatile T *mine = sh + ((size_t)wave * nb << copies_log2);
+  for (int i = threadIdx.x; i < nb * WAVES * copies; i += HIST_BLOCK) sh[i] = T(0);
   __syncthreads();
+  const uint32_t my_copy = (uint32_t)lane_id() & (uint32_t)(copies - 1);
+  // the lanes of my copy: every copies-th bit, starting at my_copy
+  uint32_t copy_mask = 0u;
+  for (int l = (int)my_copy; l < 32; l += copies) copy_mask |= 1u << l;
 
   auto update = [&](int64_t bin, T v) {
     const bool valid = (uint64_t)bin < (uint64_t)H;
     const uint32_t b = valid ? (uint32_t)bin : 0u;
+    // The match is left to the compiler here: the hand-scheduled one of the
+    // radix scatter (rs_match2) made this kernel slower (345 against 295 us).
     uint32_t differ_lo = 0u, differ_hi = 0u;
     for (int bit = 0; bit < index_bits; bit++) {
       const uint32_t me = (uint32_t)(((int32_t)(b << (31 - bit))) >> 31);  // 0 or ~0
@@ -423,14 +435,16 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
       differ_lo |= (uint32_t)m ^ me;
       differ_hi |= (uint32_t)(m >> 32) ^ me;
     }
+    const uint32_t peers_lo = ~differ_lo, peers_hi = ~differ_hi;
     const uint64_t vm = __ballot(valid);
-    const uint32_t peers_lo = ~differ_lo & (uint32_t)vm, peers_hi = ~differ_hi & (uint32_t)(vm >> 32);
-    // this lane's turn among the lanes with its bin; lanes without a bin never get one
-    const int turn =
-        valid ? (int)__builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u)) : -1;
-    const int group = __builtin_popcount(peers_lo) + __builtin_popcount(peers_hi);
+    const uint32_t lo = peers_lo & (uint32_t)vm & copy_mask;
+    const uint32_t hi = peers_hi & (uint32_t)(vm >> 32) & copy_mask;
+    // this lane's turn among the lanes with its bin and copy; lanes without a bin never get one
+    const int turn = valid ? (int)__builtin_amdgcn_mbcnt_hi(hi, __builtin_amdgcn_mbcnt_lo(lo, 0u)) : -1;
+    const int group = __builtin_popcount(lo) + __builtin_popcount(hi);
+    const uint32_t slot = (b << copies_log2) + my_copy;
     for (int r = 0; __ballot(valid && group > r) != 0; r++) {
-      if (turn == r) mine[b] = mine[b] + v;
+      if (turn == r) mine[slot] = mine[slot] + v;
       __builtin_amdgcn_wave_barrier();
     }
   };
@@ -464,8 +478,9 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
   }
   __syncthreads();
   for (int r = threadIdx.x; r < nb; r += HIST_BLOCK) {
-    T acc = sh[r];
-    for (int w = 1; w < WAVES; w++) acc += sh[(size_t)w * nb + r];
+    T acc = T(0);
+    for (int w = 0; w < WAVES; w++)
+      for (int c = 0; c < copies; c++) acc += sh[(((size_t)w * nb + r) << copies_log2) + c];
     if (!bits_equal(acc, T(0))) global_update<T, OpAdd<T>>(dest + r, acc);
   }
 }
@@ -615,6 +630,8 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
 // Sums of floats into at most this many bytes of bins per wave go through
 // seghist_wave_private_kernel.
 constexpr int HIST_WAVE_PRIVATE_BYTES = HIST_LDS_BYTES / (HIST_BLOCK / WAVE);
+constexpr int HIST_WAVE_COPIES_MAX = 4;
+
 
 template <class T, class I>
 static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
@@ -626,10 +643,15 @@ static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, in
   static const hipError_t raised = hipFuncSetAttribute(
       (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
   if (raised != hipSuccess) return (int)raised;
-  const size_t lds = (size_t)H * sizeof(T) * (HIST_BLOCK / WAVE);
+  // as many copies per wave (at most HIST_WAVE_COPIES_MAX) as leave room for two blocks on a CU
+  const size_t one = (size_t)H * sizeof(T) * (HIST_BLOCK / WAVE);
+  int copies_log2 = 0;
+  while ((1 << copies_log2) < HIST_WAVE_COPIES_MAX && (one << (copies_log2 + 1)) * 2 + 4096 <= 160 * 1024)
+    copies_log2++;
+  const size_t lds = one << copies_log2;
   const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
   hipLaunchKernelGGL(kernel, dim3(hist_num_cus() * per_cu), dim3(HIST_BLOCK), lds, st, is, vs, n,
-                     dest, H, index_bits);
+                     dest, H, index_bits, copies_log2);
   return launch_status();
 }
 
