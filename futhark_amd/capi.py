@@ -116,6 +116,7 @@ class Segops:
                 getattr(L, f"futhark_entry_vecreduce_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_seghist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
                 getattr(L, f"futhark_entry_scanrows_{op}_{t}").argtypes = [vp, pp, vp]
+                getattr(L, f"futhark_entry_vecscan_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
                 getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
                 getattr(L, f"futhark_entry_rbi_vec_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
@@ -135,6 +136,7 @@ class Segops:
         L.futhark_entry_reduce_compose_i32.argtypes = [vp, pp, vp]
         L.futhark_entry_sumsq_f32.argtypes = [vp, vp, vp]
         L.futhark_entry_scan_norm_f32.argtypes = [vp, pp, vp]
+        L.futhark_entry_rows_fraction_f32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u64.argtypes = [vp, pp, vp]
         for name, (k, v) in OPAQUE_PAIRS.items():

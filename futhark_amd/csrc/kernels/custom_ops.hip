@@ -150,3 +150,78 @@ extern "C" int fa_hist_argmax_i32(fa_stream_t stream, const int32_t *is, const i
   hipLaunchKernelGGL(zip_pairs_kernel, grid, dim3(256), 0, st, a, b, dest, H);
   return launch_status();
 }
+
+// ===========================================================================
+// SegOps inside a block (the reference's intra-block level,
+// ImpGen/GPU/Block.hs:357-615: a SegRed, a SegScan and a SegMap over one row,
+// all run by the threads of the block that owns the row, the row's values never
+// leaving the CU between them):
+//   map (\r -> let t = reduce (+) 0 r in map (/ t) (scan (+) 0 r)) xss
+// One block per row at a time.  The row's sum is a block reduction; the scan
+// walks the row in chunks of IB_CHUNK elements, four consecutive elements per
+// thread, with a wave scan of the threads' sums, the waves' sums combined
+// through LDS, and the carry of the chunks before kept by every thread.
+constexpr int IB_BLOCK = 256;
+constexpr int IB_VEC = 4;
+constexpr int IB_CHUNK = IB_BLOCK * IB_VEC;
+
+struct IbScan {
+  float excl;   // sum of the values of the threads before this one
+  float total;  // sum over the block
+};
+__device__ __forceinline__ IbScan ib_block_scan(float v, float *lds) {
+  const int lane = lane_id(), wave = threadIdx.x / WAVE;
+  const float incl = wave_incl_scan<float, OpAdd<float>>(v);
+  const float excl = wave_shift_up1<float, OpAdd<float>>(incl);
+  if (lane == WAVE - 1) lds[wave] = incl;
+  __syncthreads();
+  float before = 0.0f, total = 0.0f;
+#pragma unroll
+  for (int w = 0; w < IB_BLOCK / WAVE; w++) {
+    const float s = lds[w];
+    if (w < wave) before += s;
+    total += s;
+  }
+  __syncthreads();  // lds is free again
+  return IbScan{before + excl, total};
+}
+
+__global__ __launch_bounds__(IB_BLOCK) void rows_fraction_kernel(const float *__restrict__ xss,
+                                                                 int64_t m, int64_t k,
+                                                                 float *__restrict__ out) {
+  __shared__ float lds[IB_BLOCK / WAVE];
+  for (int64_t row = blockIdx.x; row < m; row += gridDim.x) {
+    const float *r = xss + row * k;
+    float *o = out + row * k;
+    float part = 0.0f;
+    for (int64_t i = threadIdx.x; i < k; i += IB_BLOCK) part += r[i];
+    const float total = ib_block_scan(part, lds).total;
+    float carry = 0.0f;
+    for (int64_t c0 = 0; c0 < k; c0 += IB_CHUNK) {
+      const int64_t i0 = c0 + (int64_t)threadIdx.x * IB_VEC;
+      float x[IB_VEC];
+      float run = 0.0f;
+#pragma unroll
+      for (int e = 0; e < IB_VEC; e++) {
+        run += i0 + e < k ? r[i0 + e] : 0.0f;  // the second read of the row comes from cache
+        x[e] = run;
+      }
+      const IbScan s = ib_block_scan(run, lds);
+#pragma unroll
+      for (int e = 0; e < IB_VEC; e++)
+        if (i0 + e < k) o[i0 + e] = (carry + s.excl + x[e]) / total;
+      carry += s.total;
+    }
+  }
+}
+
+extern "C" int fa_rows_fraction_f32(fa_stream_t stream, const float *xss, int64_t m, int64_t k,
+                                    float *out) {
+  if (m < 0 || k < 0) return FA_EINVAL;
+  if (m == 0 || k == 0) return 0;
+  if (xss == nullptr || out == nullptr) return FA_EINVAL;
+  const int64_t grid = m < 256 * 8 ? m : 256 * 8;
+  hipLaunchKernelGGL(rows_fraction_kernel, dim3((unsigned)grid), dim3(IB_BLOCK), 0,
+                     (hipStream_t)stream, xss, m, k, out);
+  return launch_status();
+}

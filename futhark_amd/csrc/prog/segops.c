@@ -394,6 +394,54 @@ static int do_scanrows(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t
   return 0;
 }
 
+/* `scan (map2 op) (replicate k ne) xss` for xss : [n][k]T: column j of the
+ * result is the scan of column j.  The single-pass scan takes operators on
+ * scalars (the reference's own refuses array operators too,
+ * SegScan/SinglePass.hs canBeSinglePass, and falls back to two passes over
+ * the rows); here the matrix is transposed, its rows are scanned with the
+ * single-pass kernel, and the result is transposed back, so that every access
+ * to HBM is a coalesced one. */
+static int do_vecscan(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
+                      struct fut_array **out, const struct fut_array *in) {
+  const int64_t n = in->shape[0], k = in->shape[1];
+  if (k != 0 && n > INT64_MAX / (int64_t)es / k) {
+    rts_set_error(ctx, rts_msgprintf("vecscan: %lld rows of %lld elements do not fit an int64 size\n",
+                                     (long long)n, (long long)k));
+    return 1;
+  }
+  const int64_t dims[2] = {n, k};
+  struct fut_array *res = out_array(ctx, n * k * (int64_t)es, 2, dims, "vecscan.out");
+  if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
+  if (n == 0 || k == 0) {
+    *out = res;
+    return 0;
+  }
+  uint32_t epoch = 0;
+  const size_t sbytes = fa_segscan_scratch_bytes(t, n * k);
+  void *scratch = rts_scan_scratch(ctx, sbytes, &epoch);
+  struct memblock_device tmp = {0};
+  int err = scratch == NULL ? (ctx->error ? FUTHARK_OUT_OF_MEMORY : 1) : 0;
+  if (err == 0) err = rts_memblock_alloc(ctx, &tmp, n * k * (int64_t)es, "vecscan.transposed");
+  if (err == 0) {
+    /* res holds the transposed input first, the result at the end */
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "vecscan", rts_msgprintf("{\"rows\":%lld,\"vector_size\":%lld}", (long long)n, (long long)k));
+    int code = fa_map_transpose(ctx->stream, (int)es, res->mem.mem, in->mem.mem, 1, n, k);
+    if (code == 0)
+      code = fa_segscan_rows(ctx->stream, t, op, res->mem.mem, k, n, 0, tmp.mem, scratch,
+                             ctx->scan_scratch_bytes, epoch);
+    if (code == 0) code = fa_map_transpose(ctx->stream, (int)es, res->mem.mem, tmp.mem, 1, k, n);
+    err = rts_kernel_end(ctx, ev, "vecscan", code);
+  }
+  rts_memblock_unref(ctx, &tmp, "vecscan.transposed");
+  if (err != 0) {
+    drop_array(ctx, res);
+    return err;
+  }
+  *out = res;
+  return 0;
+}
+
 /* Bit pattern of the neutral element: 0 for add, or, xor; all ones for and;
  * T.lowest / T.highest for max / min (prelude/math.fut: the smallest / largest
  * integer of the type, -inf / +inf for floats). */
@@ -640,6 +688,15 @@ static int do_rbi_shaped(struct futhark_context *ctx, fa_dtype t, fa_op op, size
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }                                                                                           \
+  int futhark_entry_vecscan_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_2d **out0,                        \
+                                       const struct futhark_##T##_2d *in0) {                  \
+    ENTER(ctx);                                                                               \
+    int ret =                                                                                 \
+        do_vecscan(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, &in0->a);     \
+    LEAVE(ctx);                                                                               \
+    return ret;                                                                               \
+  }                                                                                           \
   int futhark_entry_seghist_##OP##_##T(struct futhark_context *ctx,                           \
                                        struct futhark_##T##_2d **out0, const int64_t in0,     \
                                        const struct futhark_i32_2d *in1,                      \
@@ -830,6 +887,34 @@ int futhark_entry_scan_norm_f32(struct futhark_context *ctx, struct futhark_f32_
                                 const struct futhark_f32_1d *in0) {
   ENTER(ctx);
   int ret = do_custom_scan(ctx, (struct fut_array **)out0, &in0->a, 1, "scan_norm_f32");
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_rows_fraction_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
+                                    const struct futhark_f32_2d *in0) {
+  ENTER(ctx);
+  const struct fut_array *in = &in0->a;
+  const int64_t m = in->shape[0], k = in->shape[1];
+  int ret = 0;
+  struct fut_array *res = NULL;
+  if (k != 0 && m > INT64_MAX / 4 / k) {
+    rts_set_error(ctx, rts_msgprintf("rows_fraction_f32: %lld rows of %lld elements do not fit an int64 size\n",
+                                     (long long)m, (long long)k));
+    ret = 1;
+  } else if ((res = out_array(ctx, m * k * 4, 2, in->shape, "rows_fraction.out")) == NULL) {
+    ret = FUTHARK_OUT_OF_MEMORY;
+  } else {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "intrablock_rows",
+        rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)k));
+    int code = fa_rows_fraction_f32(ctx->stream, (const float *)in->mem.mem, m, k, (float *)res->mem.mem);
+    ret = rts_kernel_end(ctx, ev, "intrablock_rows", code);
+    if (ret != 0)
+      drop_array(ctx, res);
+    else
+      *out0 = (struct futhark_f32_2d *)res;
+  }
   LEAVE(ctx);
   return ret;
 }

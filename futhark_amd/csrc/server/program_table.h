@@ -187,6 +187,11 @@ struct entry {
     return futhark_entry_scanrows_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,         \
                                              ARRP(i[0]));                                      \
   }                                                                                            \
+  static int e_vecscan_##OP##_##T(struct futhark_context *c, struct value *o,                  \
+                                  struct value **i) {                                          \
+    return futhark_entry_vecscan_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,          \
+                                            ARRP(i[0]));                                       \
+  }                                                                                            \
   static int e_seghist_##OP##_##T(struct futhark_context *c, struct value *o,                  \
                                   struct value **i) {                                          \
     return futhark_entry_seghist_##OP##_##T(c, (struct futhark_##T##_2d **)&o->u.arr,          \
@@ -248,6 +253,9 @@ static int e_reduce_compose_i32(struct futhark_context *c, struct value *o, stru
 }
 static int e_sumsq_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_sumsq_f32(c, &o->u.f32, ARRP(i[0]));
+}
+static int e_rows_fraction_f32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_rows_fraction_f32(c, (struct futhark_f32_2d **)&o->u.arr, ARRP(i[0]));
 }
 static int e_scan_norm_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_scan_norm_f32(c, (struct futhark_f32_1d **)&o->u.arr, ARRP(i[0]));
@@ -312,6 +320,7 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
    {SEGRED_PARAM, NULL}},                                                                       \
   {"vecreduce_" #OP "_" #T, e_vecreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},   \
   {"scanrows_" #OP "_" #T, e_scanrows_##OP##_##T, "[][]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},   \
+  {"vecscan_" #OP "_" #T, e_vecscan_##OP##_##T, "[][]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},     \
   {"seghist_" #OP "_" #T, e_seghist_##OP##_##T, "[][]" #T, 1, 3,                                \
    {"i64", "[][]i32", "[][]" #T}, {0}, {HIST_PARAM, NULL}},                                     \
   {"rbi_vec_" #OP "_" #T, e_rbi_vec_##OP##_##T, "[][]" #T, 1, 3,                                \
@@ -346,6 +355,7 @@ static const struct entry entries[] = {
     {"reduce_compose_i32", e_reduce_compose_i32, "[]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
     {"sumsq_f32", e_sumsq_f32, "f32", 0, 1, {"[]f32"}, {0}, {NULL}},
     {"scan_norm_f32", e_scan_norm_f32, "[]f32", 1, 1, {"[]f32"}, {0}, {NULL}},
+    {"rows_fraction_f32", e_rows_fraction_f32, "[][]f32", 1, 1, {"[][]f32"}, {0}, {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {MATMUL_PARAM, NULL}},
     {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {MATMUL_PARAM, NULL}},
     {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {NULL}},

@@ -52,6 +52,7 @@ def entry_points() -> dict:
                 _entry(f"segreduce_{op}_{t}", a, [("xss", "[]" + a)], [SEGRED_PARAM]),
                 _entry(f"vecreduce_{op}_{t}", a, [("xss", "[]" + a)]),
                 _entry(f"scanrows_{op}_{t}", "[]" + a, [("xss", "[]" + a)]),
+                _entry(f"vecscan_{op}_{t}", "[]" + a, [("xss", "[]" + a)]),
                 _entry(f"seghist_{op}_{t}", "[]" + a,
                        [("k", "i64"), ("iss", "[][]i32"), ("vss", "[]" + a)], [HIST_PARAM]),
                 _entry(f"rbi_vec_{op}_{t}", "[]" + a,
@@ -79,6 +80,7 @@ def entry_points() -> dict:
         _entry("reduce_compose_i32", "[]i32", [("abs", "[][]i32")]),
         _entry("sumsq_f32", "f32", [("xs", "[]f32")]),
         _entry("scan_norm_f32", "[]f32", [("xs", "[]f32")]),
+        _entry("rows_fraction_f32", "[][]f32", [("xss", "[][]f32")]),
         _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")], [MATMUL_PARAM]),
         _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")], [MATMUL_PARAM]),
         _entry("radix_sort_u32", "[]u32", [("keys", "[]u32")]),

@@ -350,6 +350,11 @@ int fa_sumsq_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
                  void *scratch, size_t scratch_bytes, uint32_t epoch);
 int fa_scan_norm_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
                      void *scratch, size_t scratch_bytes, uint32_t epoch);
+/* map (\r -> let t = reduce (+) 0 r in map (/ t) (scan (+) 0 r)) xss for
+ * xss : [m][k]f32: a reduction, a scan and a map over a row by the block that
+ * owns it.  Replaces: the intra-block SegOps of a kernel at block level
+ * (src/Futhark/CodeGen/ImpGen/GPU/Block.hs:357-615). */
+int fa_rows_fraction_f32(fa_stream_t stream, const float *xss, int64_t m, int64_t k, float *out);
 size_t fa_hist_argmax_workspace_bytes(int64_t H);
 int64_t fa_hist_argmax_max_bins(void);
 int fa_hist_argmax_i32(fa_stream_t stream, const int32_t *is, const int32_t *xs, int64_t n,

@@ -23,6 +23,7 @@
  *   entry segreduce_OP_T (xss: [][]T) : []T    = map (reduce OP NE) xss
  *   entry vecreduce_OP_T (xss: [n][k]T) : [k]T = reduce (map2 OP) (replicate k NE) xss
  *   entry scanrows_OP_T (xss: [][]T) : [][]T   = map (scan OP NE) xss
+ *   entry vecscan_OP_T (xss: [n][k]T) : [n][k]T = scan (map2 OP) (replicate k NE) xss
  *   entry hist_OP_T (k: i64) (is: []i32) (vs: []T) : [k]T =
  *     hist OP NE k (map i64.i32 is) vs           -- prelude/soacs.fut:132-146
  *   entry seghist_OP_T (k: i64) (iss: [][]i32) (vss: [][]T) : [][]T =
@@ -258,6 +259,9 @@ FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
   int futhark_entry_scanrows_##OP##_##T(struct futhark_context *ctx,                          \
                                         struct futhark_##T##_2d **out0,                       \
                                         const struct futhark_##T##_2d *in0);                  \
+  int futhark_entry_vecscan_##OP##_##T(struct futhark_context *ctx,                           \
+                                       struct futhark_##T##_2d **out0,                        \
+                                       const struct futhark_##T##_2d *in0);                   \
   int futhark_entry_seghist_##OP##_##T(struct futhark_context *ctx,                           \
                                        struct futhark_##T##_2d **out0, const int64_t in0,     \
                                        const struct futhark_i32_2d *in1,                      \
@@ -337,7 +341,10 @@ int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhar
  *   entry reduce_compose_i32 (abs: [][2]i32) : [2]i32 =    -- compose as above; does not commute
  *     let (a, b) = reduce compose (1, 0) (map (\r -> (r[0], r[1])) abs) in [a, b]
  *   entry sumsq_f32 (xs: []f32) : f32 = reduce (+) 0 (map (\x -> x * x) xs)
- *   entry scan_norm_f32 (xs: []f32) : []f32 = map f32.sqrt (scan (+) 0 (map (\x -> x * x) xs)) */
+ *   entry scan_norm_f32 (xs: []f32) : []f32 = map f32.sqrt (scan (+) 0 (map (\x -> x * x) xs))
+ *   entry rows_fraction_f32 (xss: [][]f32) : [][]f32 =
+ *     map (\r -> let t = reduce (+) 0 r in map (/ t) (scan (+) 0 r)) xss
+ *                                   -- SegOps at block level, ImpGen/GPU/Block.hs:357-615 */
 int futhark_entry_reduce_argmax_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
                                     const struct futhark_i32_1d *in0);
 int futhark_entry_scan_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
@@ -351,6 +358,8 @@ int futhark_entry_sumsq_f32(struct futhark_context *ctx, float *out0,
                             const struct futhark_f32_1d *in0);
 int futhark_entry_scan_norm_f32(struct futhark_context *ctx, struct futhark_f32_1d **out0,
                                 const struct futhark_f32_1d *in0);
+int futhark_entry_rows_fraction_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
+                                    const struct futhark_f32_2d *in0);
 int futhark_entry_bmm_bf16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
                            const struct futhark_u16_3d *in0, const struct futhark_u16_3d *in1);
 int futhark_entry_matmul_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,

@@ -209,6 +209,20 @@ def scan_norm_f32(xs, variant: str = "lit"):
     return np.sqrt(scan("add", "f32", sq, variant)).astype(np.float32)
 
 
+def rows_fraction_f32(xss, variant: str = "lit"):
+    """map (\\r -> let t = reduce (+) 0 r in map (/ t) (scan (+) 0 r)) xss: per row, the running
+    sums divided by the row's sum, in f32 (division as IEEE: a row that sums to zero gives
+    NaN or infinities)."""
+    xss = _arr(xss, np.float32)
+    out = np.empty_like(xss)
+    for r in range(xss.shape[0]):
+        row = np.ascontiguousarray(xss[r])
+        t = np.float32(reduce("add", "f32", row, variant))
+        with np.errstate(divide="ignore", invalid="ignore"):
+            out[r] = (scan("add", "f32", row, variant).astype(np.float32) / t).astype(np.float32)
+    return out
+
+
 def rbi_vec(op: str, t: str, dest, is_, vss):
     """reduce_by_index dest (map2 op) (replicate m ne) is vss on a copy of dest ([H][m])."""
     _, dt = _CT[t]
@@ -246,6 +260,19 @@ def scanrows(op: str, t: str, xss, variant: str = "lit"):
     out = np.empty_like(xss)
     for r in range(xss.shape[0]):
         out[r] = scan(op, t, xss[r], variant)
+    return out
+
+
+def vecscan(op: str, t: str, xss, variant: str = "lit"):
+    """scan (map2 op) (replicate k ne) xss for xss : [n][k]t, evaluated as the
+    sequential loop of FirstOrderTransform.hs:613-656 with the vector operator:
+    acc = replicate k ne; for i < n: acc = map2 op acc xss[i]; out[i] = acc.
+    Column j of the result therefore is the scan of column j."""
+    _, dt = _CT[t]
+    xss = _arr(xss, dt)
+    out = np.empty_like(xss)
+    for j in range(xss.shape[1] if xss.ndim == 2 else 0):
+        out[:, j] = scan(op, t, np.ascontiguousarray(xss[:, j]), variant)
     return out
 
 

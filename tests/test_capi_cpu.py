@@ -45,7 +45,7 @@ def test_program_library_exports_the_generated_api():
             declared.add(f"futhark_{f}_{kind}")
     for t in NUM_TYPES:
         for op in ops_for(t):
-            for e in ("reduce", "scan", "exscan", "segscan", "segred", "segreduce", "vecreduce", "rbi_vec", "rbi_2d", "scanrows", "seghist", "hist", "rbi"):
+            for e in ("reduce", "scan", "exscan", "segscan", "segred", "segreduce", "vecreduce", "rbi_vec", "rbi_2d", "scanrows", "vecscan", "seghist", "hist", "rbi"):
                 declared.add(f"futhark_entry_{e}_{op}_{t}")
     declared = {d for d in declared if not d.endswith("_")}
     missing = declared - _exports(lib_path())

@@ -80,3 +80,26 @@ def test_hist_with_a_tuple_operator_locks_its_bins(ctx):
     with pytest.raises(FutharkError):
         ctx.call("hist_argmax_i32", ["i32_2d"], 8193, ctx.new("i32_1d", np.zeros(4, np.int32)),
                  ctx.new("i32_1d", np.zeros(4, np.int32)))
+
+
+def test_segops_inside_a_block(ctx):
+    """rows_fraction_f32: a reduction, a scan and a map over each row by one block.  Rows
+    shorter than a wave, off the four elements a thread takes, longer than a chunk of the
+    scan, more rows than blocks, empty in either dimension; a row that sums to zero divides
+    as IEEE says.  Tolerance 1e-5 relative (positive data, f32 sums in another order)."""
+    for m, k in [(1, 1), (5, 3), (7, 64), (3, 1023), (4, 1024), (3, 1025), (2, 40001), (5000, 17),
+                 (0, 4), (4, 0)]:
+        xss = (dg.uniform_f32(25, m * k) + np.float32(0.01)).reshape(m, k)
+        out = ctx.call("rows_fraction_f32", ["f32_2d"], ctx.new("f32_2d", xss))
+        got = out.values()
+        assert got.shape == (m, k)
+        want = oracle.rows_fraction_f32(xss, "f64acc")
+        assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-5 * np.abs(want) + 1e-30), (m, k)
+        if m and k:
+            assert np.all(np.abs(got[:, -1] - 1.0) <= 1e-5)
+    z = np.zeros((2, 5), np.float32)
+    z[1] = [1, -1, 2, -2, 0]
+    got = ctx.call("rows_fraction_f32", ["f32_2d"], ctx.new("f32_2d", z)).values()
+    want = oracle.rows_fraction_f32(z)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
+    assert np.array_equal(np.sign(got[np.isinf(got)]), np.sign(want[np.isinf(want)]))

@@ -48,6 +48,8 @@ def make_inputs(name, e, rng):
         return [np.array(5, np.int64), rng.integers(-1, 7, N).astype(np.int32), _vals(rng, "i32", N)]
     if name in ("sumsq_f32", "scan_norm_f32"):
         return [_vals(rng, "f32", N)]
+    if name == "rows_fraction_f32":
+        return [np.abs(_vals(rng, "f32", (6, 7))) + np.float32(1)]
     if fam in ("reduce", "scan", "exscan"):
         return [_vals(rng, el(types[0]), N)]
     if fam == "segscan":
@@ -55,7 +57,7 @@ def make_inputs(name, e, rng):
     if fam == "segred":
         lens = np.array([10, 0, 20, 7], np.int64)
         return [np.array([0, 10, 10, 30], np.int64), lens, _vals(rng, el(types[2]), N)]
-    if fam in ("segreduce", "scanrows", "vecreduce"):
+    if fam in ("segreduce", "scanrows", "vecreduce", "vecscan"):
         return [_vals(rng, el(types[0]), (6, 7))]
     if fam == "hist":
         return [np.array(5, np.int64), rng.integers(-1, 7, N).astype(np.int32), _vals(rng, el(types[2]), N)]

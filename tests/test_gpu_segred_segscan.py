@@ -441,3 +441,25 @@ def test_segred_reports_segments_that_are_not_segments(segops_lib):
         out = c.call("segred_add_i32", ["i32_1d"], o, l, v)
         c.sync()
         assert np.array_equal(out.values(), oracle.segred("add", "i32", np.array([0, 10, 500]), np.array([10, 0, 500]), xs))
+
+
+@pytest.mark.parametrize("t,op", [("i32", "add"), ("f32", "max"), ("i64", "add"), ("f32", "add"),
+                                  ("i32", "xor")])
+def test_scan_with_a_vector_operator(ctx, t, op):
+    """scan (map2 op) (replicate k ne) xss: column j of the result is the scan of column j.
+    Shapes: one column (an ordinary scan), few and many columns, more rows than a tile of the row
+    scan holds, sizes off every tile of the transposes, empty in either dimension."""
+    for n, k in [(1, 1), (1000, 1), (7, 3), (1, 300), (1000, 4), (333, 33), (40001, 5), (70, 1000),
+                 (20000, 64), (0, 4), (4, 0)]:
+        xss = _data(t, n * k, 17).reshape(n, k)
+        out = ctx.call(f"vecscan_{op}_{t}", [f"{t}_2d"], ctx.new(f"{t}_2d", xss))
+        got = out.values()
+        assert got.shape == (n, k)
+        if t == "f32" and op == "add":
+            _close(got.reshape(-1), np.cumsum(xss.astype(np.float64), axis=0).reshape(-1))
+        else:
+            assert np.array_equal(got, oracle.vecscan(op, t, xss)), (n, k)
+        # the last row is what the reduction with the same operator gives
+        if n > 0 and k > 0 and not (t == "f32" and op == "add"):
+            red = ctx.call(f"vecreduce_{op}_{t}", [f"{t}_1d"], ctx.new(f"{t}_2d", xss)).values()
+            assert np.array_equal(got[-1], red), (n, k)

@@ -412,3 +412,40 @@ def test_tuple_operator_oracles_are_pinned_by_closed_forms():
         <= 1e-6 * float(np.dot(xs.astype(np.float64), xs.astype(np.float64)))
     want = np.sqrt(np.cumsum(xs.astype(np.float64) ** 2))
     assert np.all(np.abs(oracle.scan_norm_f32(xs, "f64acc") - want) <= 1e-6 * want)
+
+
+def test_vector_operator_scan_oracle_is_pinned():
+    """vecscan is the scalar scan (pinned by the reference's scan0/exscan0/scan4 vectors above)
+    applied per column.  What could go wrong is the axis: a shape that is not square, rows that
+    are all alike (closed form (i+1)(j+1)), numpy's own cumulative sum down the rows, and the
+    last row against the reduction with the same operator."""
+    n, k = 5, 3
+    xss = np.tile(np.arange(1, k + 1, dtype=np.int32), (n, 1))
+    got = oracle.vecscan("add", "i32", xss)
+    assert got.shape == (n, k)
+    assert got.tolist() == [[(i + 1) * (j + 1) for j in range(k)] for i in range(n)]
+    rng = np.random.default_rng(5)
+    yss = rng.integers(-1000, 1000, (37, 11)).astype(np.int64)
+    assert np.array_equal(oracle.vecscan("add", "i64", yss), np.cumsum(yss, axis=0))
+    assert np.array_equal(oracle.vecscan("max", "i64", yss), np.maximum.accumulate(yss, axis=0))
+    assert np.array_equal(oracle.vecscan("add", "i64", yss)[-1], oracle.vecreduce("add", "i64", yss))
+    assert oracle.vecscan("add", "i32", np.zeros((0, 4), np.int32)).shape == (0, 4)
+    assert oracle.vecscan("add", "i32", np.zeros((4, 0), np.int32)).shape == (4, 0)
+
+
+def test_rows_fraction_oracle_is_pinned():
+    """Closed forms: a row of ones gives (i+1)/k; the last column is 1; rows do not mix
+    (a transposed loop would); scaling a row by a power of two changes nothing."""
+    k = 8
+    ones = np.ones((3, k), np.float32)
+    got = oracle.rows_fraction_f32(ones)
+    assert np.array_equal(got, np.tile((np.arange(1, k + 1) / k).astype(np.float32), (3, 1)))
+    rng = np.random.default_rng(9)
+    xss = (rng.random((4, 37)) + 0.5).astype(np.float32)
+    got = oracle.rows_fraction_f32(xss, "f64acc")
+    want = np.cumsum(xss.astype(np.float64), axis=1) / xss.astype(np.float64).sum(axis=1)[:, None]
+    assert np.all(np.abs(got - want) <= 1e-6)
+    assert np.all(np.abs(got[:, -1] - 1) <= 1e-6)
+    assert np.array_equal(oracle.rows_fraction_f32(xss * np.float32(4)), oracle.rows_fraction_f32(xss))
+    one_row = oracle.rows_fraction_f32(xss[2:3])
+    assert np.array_equal(one_row[0], oracle.rows_fraction_f32(xss)[2])
