@@ -206,6 +206,32 @@ def make_workload(name: str, ctx):
             ctx.call(f"scanrows_{op}_{t}", [f"{t}_2d"], a).free()
         w.update(step=step, bytes=2 * m * k * dt().itemsize, kernel="segscan_rows", dtype=t,
                  bound="hbm", keep=[a], describe=f"scan ({op}) of every row of [{m}][{k}]{t}")
+    elif name.startswith("vecscan_"):
+        # vecscan_add_f32_65536x1024: scan (map2 op) (replicate k ne) xss, xss : [n][k]
+        _, op, t, shape = name.split("_")
+        n, k = (int(x) for x in shape.split("x"))
+        w["elements"] = n * k
+        dt = {"f32": np.float32, "i32": np.int32, "i64": np.int64, "f64": np.float64}[t]
+        xss = (dg.uniform_f32(38, n * k) if t[0] == "f" else dg.uniform_int(39, n * k, -1000, 1000)
+               ).astype(dt).reshape(n, k)
+        a = ctx.new(f"{t}_2d", xss)
+
+        def step():
+            ctx.call(f"vecscan_{op}_{t}", [f"{t}_2d"], a).free()
+        w.update(step=step, bytes=2 * n * k * dt().itemsize, kernel="vecscan", dtype=t, bound="hbm",
+                 keep=[a], describe=f"scan with vectorised operator (map2 {op}) of [{n}][{k}]{t}")
+    elif name.startswith("rowsfraction_"):
+        # rowsfraction_f32_65536x1024: reduce, scan and map over every row inside one block
+        _, t, shape = name.split("_")
+        m, k = (int(x) for x in shape.split("x"))
+        w["elements"] = m * k
+        xss = (dg.uniform_f32(38, m * k) + np.float32(0.01)).reshape(m, k)
+        a = ctx.new("f32_2d", xss)
+
+        def step():
+            ctx.call("rows_fraction_f32", ["f32_2d"], a).free()
+        w.update(step=step, bytes=2 * m * k * 4, kernel="intrablock_rows", dtype=t, bound="hbm",
+                 keep=[a], describe=f"row sums, row scans and a division inside a block, [{m}][{k}]{t}")
     elif name.startswith("segreduce_"):
         # segreduce_add_f32_65536x1024: regular segments, map (reduce op ne) xss
         _, op, t, shape = name.split("_")

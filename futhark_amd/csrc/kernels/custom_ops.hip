@@ -190,26 +190,48 @@ __global__ __launch_bounds__(IB_BLOCK) void rows_fraction_kernel(const float *__
                                                                  int64_t m, int64_t k,
                                                                  float *__restrict__ out) {
   __shared__ float lds[IB_BLOCK / WAVE];
+  const bool vectors = k % IB_VEC == 0 && ((uintptr_t)xss | (uintptr_t)out) % 16 == 0;
   for (int64_t row = blockIdx.x; row < m; row += gridDim.x) {
     const float *r = xss + row * k;
     float *o = out + row * k;
     float part = 0.0f;
-    for (int64_t i = threadIdx.x; i < k; i += IB_BLOCK) part += r[i];
+    if (vectors) {
+      for (int64_t i = (int64_t)threadIdx.x * IB_VEC; i < k; i += IB_CHUNK) {
+        const Vec16<float> v = load_vec16(r + i);
+        part += (v.e[0] + v.e[1]) + (v.e[2] + v.e[3]);
+      }
+    } else {
+      for (int64_t i = threadIdx.x; i < k; i += IB_BLOCK) part += r[i];
+    }
     const float total = ib_block_scan(part, lds).total;
     float carry = 0.0f;
     for (int64_t c0 = 0; c0 < k; c0 += IB_CHUNK) {
       const int64_t i0 = c0 + (int64_t)threadIdx.x * IB_VEC;
+      // the second read of the row comes from cache; rows of whole 16-byte
+      // vectors are read and written as such
+      const bool whole = vectors && i0 + IB_VEC <= k;
       float x[IB_VEC];
-      float run = 0.0f;
+      if (whole) {
+        const Vec16<float> v = load_vec16(r + i0);
 #pragma unroll
-      for (int e = 0; e < IB_VEC; e++) {
-        run += i0 + e < k ? r[i0 + e] : 0.0f;  // the second read of the row comes from cache
-        x[e] = run;
+        for (int e = 0; e < IB_VEC; e++) x[e] = v.e[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < IB_VEC; e++) x[e] = i0 + e < k ? r[i0 + e] : 0.0f;
       }
-      const IbScan s = ib_block_scan(run, lds);
 #pragma unroll
-      for (int e = 0; e < IB_VEC; e++)
-        if (i0 + e < k) o[i0 + e] = (carry + s.excl + x[e]) / total;
+      for (int e = 1; e < IB_VEC; e++) x[e] += x[e - 1];
+      const IbScan s = ib_block_scan(x[IB_VEC - 1], lds);
+      if (whole) {
+        Vec16<float> v;
+#pragma unroll
+        for (int e = 0; e < IB_VEC; e++) v.e[e] = (carry + s.excl + x[e]) / total;
+        store_vec16(o + i0, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < IB_VEC; e++)
+          if (i0 + e < k) o[i0 + e] = (carry + s.excl + x[e]) / total;
+      }
       carry += s.total;
     }
   }

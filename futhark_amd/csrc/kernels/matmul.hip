@@ -28,9 +28,6 @@ typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef short i16x4 __attribute__((ext_vector_type(4)));
 
-#ifndef MM_C_STORE
-#define MM_C_STORE(p, v) (*(p) = (v))
-#endif
 constexpr int MM_BM = 256, MM_BN = 256;
 constexpr int MM_XCDS = 8;
 constexpr int MM_GROUP_M = 4;
@@ -309,7 +306,8 @@ __global__ __launch_bounds__(MM16_THREADS) void matmul16_kernel(const uint16_t *
         const int row =
             bm + wm * (MM16_MT * 32) + mt * 32 + (e >> 2) * 8 + (lane >> 5) * 4 + (e & 3);
         const int col = bn + wn * (MM16_NT * 32) + nt * 32 + (lane & 31);
-        MM_C_STORE(&Cb[(int64_t)row * N + col], acc[mt][nt][e]);
+        // C is not read again by this kernel: non-temporal stores (122.7 -> 121.0 us at 4096^3)
+        __builtin_nontemporal_store(acc[mt][nt][e], &Cb[(int64_t)row * N + col]);
       }
 }
 
