@@ -117,11 +117,27 @@ __device__ __forceinline__ void load_to_lds_16(const char *uniform_base, uint32_
                : "memory");
 }
 
-template <bool BF16>
-__global__ __launch_bounds__(MM16_THREADS) void matmul16_kernel(const uint16_t *__restrict__ A,
-                                                                const uint16_t *__restrict__ B,
-                                                                float *__restrict__ C, int M,
-                                                                int N, int K) {
+// BM x BN: the block's tile of C; WAVES_M x WAVES_N: how its waves share it.
+// 256 x 256 with 2 x 2 waves is the kernel for large products (one block per
+// CU, the least LDS traffic per MFMA); 128 x 128 with 1 x 2 waves takes shapes
+// that are multiples of 128 only.
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void matmul16_kernel(
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ B, float *__restrict__ C, int M,
+    int N, int K) {
+  constexpr int MM16_WAVES = WAVES_M * WAVES_N;
+  constexpr int MM16_WAVES_N = WAVES_N;
+  constexpr int MM_BM = BM, MM_BN = BN;
+  constexpr int MM16_A_TILE_BYTES = BM * MM16_A_ROW_BYTES;
+  constexpr int MM16_B_ROW_BYTES = BN * 2;
+  constexpr int MM16_B_TILE_BYTES = MM16_BK * MM16_B_ROW_BYTES;
+  constexpr int MM16_STAGE_BYTES = MM16_A_TILE_BYTES + MM16_B_TILE_BYTES;
+  constexpr int MM16_MT = BM / (WAVES_M * 32), MM16_NT = BN / (WAVES_N * 32);
+  constexpr int MM16_CHUNKS = MM16_A_TILE_BYTES / 1024 / MM16_WAVES;  // 1 KiB loads per wave, per operand
+  static_assert(MM16_B_TILE_BYTES == MM16_A_TILE_BYTES, "as many chunks of B as of A");
+  constexpr int B_UNITS = MM16_B_ROW_BYTES / 16;  // 16-byte units per row of the B tile
+  constexpr int B_ROWS = 1024 / MM16_B_ROW_BYTES;  // rows of the B tile per 1 KiB chunk
+  static_assert((B_ROWS * MM16_WAVES) % 4 == 0, "a lane's swizzle term is the same in all its chunks");
   extern __shared__ __align__(16) unsigned char lds[];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -136,20 +152,20 @@ __global__ __launch_bounds__(MM16_THREADS) void matmul16_kernel(const uint16_t *
   float *Cb = C + batch * (int64_t)M * N;
 
   // Loads.  Chunk c of the A tile is rows 8c..8c+7 (1 KiB of LDS), chunk c of
-  // the B tile is rows 2c, 2c+1.  Wave w moves chunks w, w + WAVES, ...; since
+  // the B tile is rows B_ROWS c .. B_ROWS c + B_ROWS - 1.  Wave w moves chunks w, w + WAVES, ...; since
   // WAVES is even the swizzle term of a lane's row does not depend on the
   // chunk, so a lane's chunks differ by a constant stride in global memory.
   static_assert(MM16_WAVES % 2 == 0, "swizzle terms assume an even chunk stride");
   const int a_r = lane >> 3, a_slot = lane & 7;
   const int a_unit = a_slot ^ (((wave & 1) << 2) | (a_r >> 1));  // ((8 w + a_r) >> 1) & 7
-  const int b_r = lane >> 5, b_slot = lane & 31;
-  const int b_unit = b_slot ^ ((((wave & 1) << 1) | b_r) << 2);  // ((2 w + b_r) & 3) << 2
+  const int b_r = lane / B_UNITS, b_slot = lane % B_UNITS;
+  const int b_unit = b_slot ^ (((B_ROWS * wave + b_r) & 3) << 2);  // row k of the tile: (k & 3) << 2
   const char *a_src = reinterpret_cast<const char *>(Ab + (int64_t)(bm + wave * 8) * K);
-  const char *b_src = reinterpret_cast<const char *>(Bb + (int64_t)(wave * 2) * N + bn);
+  const char *b_src = reinterpret_cast<const char *>(Bb + (int64_t)(wave * B_ROWS) * N + bn);
   const uint32_t a_lane = (uint32_t)(a_r * K * 2 + a_unit * 16);  // K, N < 2^27 elements
   const uint32_t b_lane = (uint32_t)(b_r * N * 2 + b_unit * 16);
   const int64_t a_chunk_step = (int64_t)MM16_WAVES * 8 * K * 2;
-  const int64_t b_chunk_step = (int64_t)MM16_WAVES * 2 * N * 2;
+  const int64_t b_chunk_step = (int64_t)MM16_WAVES * B_ROWS * N * 2;
   const int64_t b_tile_step = (int64_t)MM16_BK * N * 2;
   const uint32_t lds_base =
       (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)lds;
@@ -553,11 +569,13 @@ struct MmPlan {
 
 static size_t mm_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
+static bool mm16_small_tiles_fit(int64_t M, int64_t N, int64_t K);
 static MmPlan mm_plan(fa_dtype in_t, int64_t batch, int64_t M, int64_t N, int64_t K) {
   MmPlan p = {};
   const int bk = in_t == FA_F32 ? MM32_BK : MM16_BK;
   const size_t es = in_t == FA_F32 ? 4 : 2;
-  p.direct_tiled = M % MM_BM == 0 && N % MM_BN == 0 && K % bk == 0 && K > 0;
+  p.direct_tiled = (M % MM_BM == 0 && N % MM_BN == 0 && K % bk == 0 && K > 0) ||
+                   (in_t != FA_F32 && mm16_small_tiles_fit(M, N, K));
   if (p.direct_tiled || batch * M * N == 0 || K == 0) return p;
   p.Mp = ceil_div(M, (int64_t)MM_BM) * MM_BM;
   p.Np = ceil_div(N, (int64_t)MM_BN) * MM_BN;
@@ -575,6 +593,31 @@ static MmPlan mm_plan(fa_dtype in_t, int64_t batch, int64_t M, int64_t N, int64_
   return p;
 }
 
+// Launch of one geometry of the 16-bit kernel.
+template <bool BF16, int BM, int BN, int WAVES_M, int WAVES_N>
+static int launch_mm16(hipStream_t st, const uint16_t *A, const uint16_t *B, float *C, int64_t batch,
+                       int64_t M, int64_t N, int64_t K) {
+  constexpr int lds = 2 * (BM * MM16_A_ROW_BYTES + MM16_BK * BN * 2);
+  auto kernel = matmul16_kernel<BF16, BM, BN, WAVES_M, WAVES_N>;
+  static const int raised = raise_lds(kernel, lds);
+  if (raised) return raised;
+  if (M / BM > 65535) return FA_EINVAL;
+  const dim3 grid((unsigned)(N / BN), (unsigned)(M / BM), (unsigned)batch);
+  hipLaunchKernelGGL(kernel, grid, dim3(64 * WAVES_M * WAVES_N), lds, st, A, B, C, (int)M, (int)N,
+                     (int)K);
+  return launch_status();
+}
+
+// 128 x 128 tiles serve shapes that are multiples of 128 but not of 256 without
+// padded copies.  They are not faster where both fit, not even for products
+// with few k-steps per tile: b = 64, M = N = K = 512 f16 takes 43 us with them
+// against 34 us with 256 x 256 tiles (two blocks share a CU, but every block
+// moves twice the bytes from L2 into LDS per flop, and reads LDS a third more
+// often per MFMA).
+static bool mm16_small_tiles_fit(int64_t M, int64_t N, int64_t K) {
+  return M % 128 == 0 && N % 128 == 0 && K % MM16_BK == 0 && K > 0;
+}
+
 static int matmul_direct(fa_stream_t stream, fa_dtype in_t, const void *A, const void *B, float *C,
                          int64_t batch, int64_t M, int64_t N, int64_t K) {
   if (batch < 0 || M < 0 || N < 0 || K < 0) return FA_EINVAL;
@@ -584,28 +627,25 @@ static int matmul_direct(fa_stream_t stream, fa_dtype in_t, const void *A, const
   if (batch > 65535 || M > INT32_MAX || N > INT32_MAX || K > INT32_MAX) return FA_EINVAL;
   hipStream_t st = (hipStream_t)stream;
   const int bk = in_t == FA_F32 ? MM32_BK : MM16_BK;
-  const bool tiled = M % MM_BM == 0 && N % MM_BN == 0 && K % bk == 0 && K > 0 &&
-                     is_aligned(A, 16) && is_aligned(B, 16) && is_aligned(C, 16);
+  const bool aligned = is_aligned(A, 16) && is_aligned(B, 16) && is_aligned(C, 16);
+  const bool tiled = M % MM_BM == 0 && N % MM_BN == 0 && K % bk == 0 && K > 0 && aligned;
+  if (in_t != FA_F32 && aligned && !tiled && mm16_small_tiles_fit(M, N, K)) {
+    const uint16_t *a = (const uint16_t *)A, *b = (const uint16_t *)B;
+    return in_t == FA_F16 ? launch_mm16<false, 128, 128, 1, 2>(st, a, b, C, batch, M, N, K)
+                          : launch_mm16<true, 128, 128, 1, 2>(st, a, b, C, batch, M, N, K);
+  }
   if (tiled) {
-    const dim3 grid((unsigned)(N / MM_BN), (unsigned)(M / MM_BM), (unsigned)batch);
-    int rc = 0;
     if (in_t == FA_F32) {
+      const dim3 grid((unsigned)(N / MM_BN), (unsigned)(M / MM_BM), (unsigned)batch);
       static const int raised = raise_lds(matmul32_kernel, 2 * MM32_STAGE_BYTES);
-      if ((rc = raised)) return rc;
+      if (raised) return raised;
       hipLaunchKernelGGL(matmul32_kernel, grid, dim3(MM_THREADS), 2 * MM32_STAGE_BYTES, st,
                          (const float *)A, (const float *)B, C, (int)M, (int)N, (int)K);
-    } else if (in_t == FA_F16) {
-      static const int raised = raise_lds(matmul16_kernel<false>, 2 * MM16_STAGE_BYTES);
-      if ((rc = raised)) return rc;
-      hipLaunchKernelGGL((matmul16_kernel<false>), grid, dim3(MM16_THREADS), 2 * MM16_STAGE_BYTES, st,
-                         (const uint16_t *)A, (const uint16_t *)B, C, (int)M, (int)N, (int)K);
-    } else {
-      static const int raised = raise_lds(matmul16_kernel<true>, 2 * MM16_STAGE_BYTES);
-      if ((rc = raised)) return rc;
-      hipLaunchKernelGGL((matmul16_kernel<true>), grid, dim3(MM16_THREADS), 2 * MM16_STAGE_BYTES, st,
-                         (const uint16_t *)A, (const uint16_t *)B, C, (int)M, (int)N, (int)K);
+      return launch_status();
     }
-    return launch_status();
+    const uint16_t *a = (const uint16_t *)A, *b = (const uint16_t *)B;
+    return in_t == FA_F16 ? launch_mm16<false, 256, 256, 2, 2>(st, a, b, C, batch, M, N, K)
+                          : launch_mm16<true, 256, 256, 2, 2>(st, a, b, C, batch, M, N, K);
   }
   const dim3 grid((unsigned)ceil_div(N, 64), (unsigned)ceil_div(M, 64), (unsigned)batch);
   if (grid.y > 65535) return FA_EINVAL;

@@ -37,6 +37,7 @@ def _check(got, Af, Bf, tol):
 def test_shapes(ctx, t, tol):
     for b, M, N, K in [(1, 2, 2, 3), (3, 17, 29, 13), (2, 64, 64, 64), (1, 100, 70, 130),
                        (1, 256, 256, 32), (1, 256, 256, 64), (2, 256, 512, 96), (1, 512, 256, 512),
+                       (1, 128, 128, 64), (3, 384, 128, 192), (1, 640, 896, 128),  # 128 x 128 tiles
                        (1, 5, 7, 0), (0, 4, 4, 4)]:
         Ain, Bin, Af, Bf, kind = _inputs(t, b, M, N, K)
         out = ctx.call(f"bmm_{t}", ["f32_3d"], ctx.new(kind, Ain), ctx.new(kind, Bin))
