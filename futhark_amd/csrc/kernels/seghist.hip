@@ -403,7 +403,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
 // lanes; so a wave keeps 2^copies_log2 copies of its histogram where LDS
 // allows, lane l using copy l mod 2^copies_log2, and only lanes of the same
 // copy take turns (H = 256, Zipf indices: 640 -> 382 us per 2^27 pairs).
-template <class T, class I>
+template <class T, class I, int INDEX_BITS /* 0: as many as `index_bits` says, not unrolled */>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
     const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t H,
     int index_bits, int copies_log2) {
@@ -429,11 +429,17 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
     // The match is left to the compiler here: the hand-scheduled one of the
     // radix scatter (rs_match2) made this kernel slower (345 against 295 us).
     uint32_t differ_lo = 0u, differ_hi = 0u;
-    for (int bit = 0; bit < index_bits; bit++) {
+    auto match_bit = [&](int bit) {
       const uint32_t me = (uint32_t)(((int32_t)(b << (31 - bit))) >> 31);  // 0 or ~0
       const uint64_t m = __ballot(me != 0u);
       differ_lo |= (uint32_t)m ^ me;
       differ_hi |= (uint32_t)(m >> 32) ^ me;
+    };
+    if constexpr (INDEX_BITS > 0) {
+#pragma unroll
+      for (int bit = 0; bit < INDEX_BITS; bit++) match_bit(bit);
+    } else {
+      for (int bit = 0; bit < index_bits; bit++) match_bit(bit);
     }
     const uint32_t peers_lo = ~differ_lo, peers_hi = ~differ_hi;
     const uint64_t vm = __ballot(valid);
@@ -636,13 +642,14 @@ constexpr int HIST_WAVE_COPIES_MAX = 4;
 template <class T, class I>
 static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
                                     int64_t H) {
+  // The match loop over the index bits is unrolled (8 bits for up to 256 bins,
+  // else 11: HIST_WAVE_PRIVATE_BYTES / 4 = 2048 bins at most) except for 4-byte
+  // sums into up to 256 bins, where the unrolled loop costs registers and with
+  // them time (H = 256 f32: 309 against 297 us; H = 2048 f32: 428 against
+  // 465 us, H = 256 f64: 372 against 392 us in favour of unrolling).
+  static_assert(HIST_WAVE_PRIVATE_BYTES / 4 <= (1 << 11), "eleven index bits cover every bin");
   int index_bits = 1;
   while (((int64_t)1 << index_bits) < H) index_bits++;
-  auto kernel = seghist_wave_private_kernel<T, I>;
-  // Initialised once, under the lock C++ gives function-local statics.
-  static const hipError_t raised = hipFuncSetAttribute(
-      (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
-  if (raised != hipSuccess) return (int)raised;
   // as many copies per wave (at most HIST_WAVE_COPIES_MAX) as leave room for two blocks on a CU
   const size_t one = (size_t)H * sizeof(T) * (HIST_BLOCK / WAVE);
   int copies_log2 = 0;
@@ -650,8 +657,24 @@ static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, in
     copies_log2++;
   const size_t lds = one << copies_log2;
   const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
-  hipLaunchKernelGGL(kernel, dim3(hist_num_cus() * per_cu), dim3(HIST_BLOCK), lds, st, is, vs, n,
-                     dest, H, index_bits, copies_log2);
+  const dim3 grid(hist_num_cus() * per_cu);
+#define FA_WAVE_PRIVATE(BITS)                                                                  \
+  do {                                                                                         \
+    auto kernel = seghist_wave_private_kernel<T, I, BITS>;                                     \
+    /* Initialised once, under the lock C++ gives function-local statics. */                   \
+    static const hipError_t raised = hipFuncSetAttribute(                                      \
+        (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);     \
+    if (raised != hipSuccess) return (int)raised;                                              \
+    hipLaunchKernelGGL(kernel, grid, dim3(HIST_BLOCK), lds, st, is, vs, n, dest, H, index_bits, \
+                       copies_log2);                                                           \
+  } while (0)
+  if (H > 256)
+    FA_WAVE_PRIVATE(11);
+  else if (sizeof(T) == 8)
+    FA_WAVE_PRIVATE(8);
+  else
+    FA_WAVE_PRIVATE(0);
+#undef FA_WAVE_PRIVATE
   return launch_status();
 }
 
