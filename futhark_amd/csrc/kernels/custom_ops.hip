@@ -226,7 +226,7 @@ __global__ __launch_bounds__(IB_BLOCK) void rows_fraction_kernel(const float *__
         Vec16<float> v;
 #pragma unroll
         for (int e = 0; e < IB_VEC; e++) v.e[e] = (carry + s.excl + x[e]) / total;
-        store_vec16(o + i0, v);
+        store_vec16_nt(o + i0, v);
       } else {
 #pragma unroll
         for (int e = 0; e < IB_VEC; e++)
