@@ -237,11 +237,71 @@ __global__ __launch_bounds__(IB_BLOCK) void rows_fraction_kernel(const float *__
   }
 }
 
+// Rows of at most IB_WAVE_ROW_MAX elements: one wave per row, four rows to a
+// block, no barrier at all (a block per 256-byte row spends its time in the
+// four barriers of ib_block_scan: [2^20][64] took 833 us).
+constexpr int IB_WAVE_ROW_MAX = 256;  // at 1024 the block kernel is faster (81 against 96 us for [65536][1024])
+__global__ __launch_bounds__(IB_BLOCK) void rows_fraction_wave_kernel(const float *__restrict__ xss,
+                                                                      int64_t m, int64_t k,
+                                                                      float *__restrict__ out) {
+  const int lane = lane_id();
+  const int64_t waves = (int64_t)gridDim.x * (IB_BLOCK / WAVE);
+  const bool vectors = k % IB_VEC == 0 && ((uintptr_t)xss | (uintptr_t)out) % 16 == 0;
+  for (int64_t row = (int64_t)blockIdx.x * (IB_BLOCK / WAVE) + threadIdx.x / WAVE; row < m;
+       row += waves) {
+    const float *r = xss + row * k;
+    float *o = out + row * k;
+    // pass one: the row's sum; pass two: scan and divide (the row comes from cache)
+    float part = 0.0f;
+    for (int64_t i = (int64_t)lane * IB_VEC; i < k; i += WAVE * IB_VEC) {
+#pragma unroll
+      for (int e = 0; e < IB_VEC; e++) part += i + e < k ? r[i + e] : 0.0f;
+    }
+    const float total = read_lane(wave_incl_scan<float, OpAdd<float>>(part), WAVE - 1);
+    float carry = 0.0f;
+    for (int64_t c0 = 0; c0 < k; c0 += WAVE * IB_VEC) {
+      const int64_t i0 = c0 + (int64_t)lane * IB_VEC;
+      const bool whole = vectors && i0 + IB_VEC <= k;
+      float x[IB_VEC];
+      if (whole) {
+        const Vec16<float> v = load_vec16(r + i0);
+#pragma unroll
+        for (int e = 0; e < IB_VEC; e++) x[e] = v.e[e];
+      } else {
+#pragma unroll
+        for (int e = 0; e < IB_VEC; e++) x[e] = i0 + e < k ? r[i0 + e] : 0.0f;
+      }
+#pragma unroll
+      for (int e = 1; e < IB_VEC; e++) x[e] += x[e - 1];
+      const float incl = wave_incl_scan<float, OpAdd<float>>(x[IB_VEC - 1]);
+      const float excl = wave_shift_up1<float, OpAdd<float>>(incl);
+      if (whole) {
+        Vec16<float> v;
+#pragma unroll
+        for (int e = 0; e < IB_VEC; e++) v.e[e] = (carry + excl + x[e]) / total;
+        store_vec16_nt(o + i0, v);
+      } else {
+#pragma unroll
+        for (int e = 0; e < IB_VEC; e++)
+          if (i0 + e < k) o[i0 + e] = (carry + excl + x[e]) / total;
+      }
+      carry += read_lane(incl, WAVE - 1);
+    }
+  }
+}
+
 extern "C" int fa_rows_fraction_f32(fa_stream_t stream, const float *xss, int64_t m, int64_t k,
                                     float *out) {
   if (m < 0 || k < 0) return FA_EINVAL;
   if (m == 0 || k == 0) return 0;
   if (xss == nullptr || out == nullptr) return FA_EINVAL;
+  if (k <= IB_WAVE_ROW_MAX) {
+    const int64_t blocks = ceil_div(m, (int64_t)(IB_BLOCK / WAVE));
+    const int64_t grid = blocks < 256 * 8 ? blocks : 256 * 8;
+    hipLaunchKernelGGL(rows_fraction_wave_kernel, dim3((unsigned)grid), dim3(IB_BLOCK), 0,
+                       (hipStream_t)stream, xss, m, k, out);
+    return launch_status();
+  }
   const int64_t grid = m < 256 * 8 ? m : 256 * 8;
   hipLaunchKernelGGL(rows_fraction_kernel, dim3((unsigned)grid), dim3(IB_BLOCK), 0,
                      (hipStream_t)stream, xss, m, k, out);

@@ -397,10 +397,12 @@ static int do_scanrows(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t
 /* `scan (map2 op) (replicate k ne) xss` for xss : [n][k]T: column j of the
  * result is the scan of column j.  The single-pass scan takes operators on
  * scalars (the reference's own refuses array operators too,
- * SegScan/SinglePass.hs canBeSinglePass, and falls back to two passes over
- * the rows); here the matrix is transposed, its rows are scanned with the
- * single-pass kernel, and the result is transposed back, so that every access
- * to HBM is a coalesced one. */
+ * SegScan/SinglePass.hs canBeSinglePass, and falls back to two passes).  Rows
+ * of whole 1 KiB strips go to fa_vecscan (fold per chunk of rows, prefixes
+ * over the chunks, scan per chunk: no transposed copy); for every other shape
+ * the matrix is transposed, its rows are scanned with the single-pass kernel,
+ * and the result is transposed back, so that every access to HBM is a
+ * coalesced one. */
 static int do_vecscan(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
                       struct fut_array **out, const struct fut_array *in) {
   const int64_t n = in->shape[0], k = in->shape[1];
@@ -416,6 +418,25 @@ static int do_vecscan(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t 
     *out = res;
     return 0;
   }
+  const size_t direct_bytes = fa_vecscan_workspace_bytes(t, n, k);
+  if (direct_bytes > 0) { /* rows of whole 1 KiB strips: no transposed copy */
+    struct memblock_device ws = {0};
+    int err = rts_memblock_alloc(ctx, &ws, (int64_t)direct_bytes, "vecscan.workspace");
+    if (err == 0) {
+      struct rts_event *ev = rts_kernel_begin(
+          ctx, "vecscan", rts_msgprintf("{\"rows\":%lld,\"vector_size\":%lld,\"transposed\":false}",
+                                        (long long)n, (long long)k));
+      int code = fa_vecscan(ctx->stream, t, op, in->mem.mem, n, k, res->mem.mem, ws.mem, direct_bytes);
+      err = rts_kernel_end(ctx, ev, "vecscan", code);
+    }
+    rts_memblock_unref(ctx, &ws, "vecscan.workspace");
+    if (err != 0) {
+      drop_array(ctx, res);
+      return err;
+    }
+    *out = res;
+    return 0;
+  }
   uint32_t epoch = 0;
   const size_t sbytes = fa_segscan_scratch_bytes(t, n * k);
   void *scratch = rts_scan_scratch(ctx, sbytes, &epoch);
@@ -425,7 +446,7 @@ static int do_vecscan(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t 
   if (err == 0) {
     /* res holds the transposed input first, the result at the end */
     struct rts_event *ev = rts_kernel_begin(
-        ctx, "vecscan", rts_msgprintf("{\"rows\":%lld,\"vector_size\":%lld}", (long long)n, (long long)k));
+        ctx, "vecscan", rts_msgprintf("{\"rows\":%lld,\"vector_size\":%lld,\"transposed\":true}", (long long)n, (long long)k));
     int code = fa_map_transpose(ctx->stream, (int)es, res->mem.mem, in->mem.mem, 1, n, k);
     if (code == 0)
       code = fa_segscan_rows(ctx->stream, t, op, res->mem.mem, k, n, 0, tmp.mem, scratch,

@@ -289,6 +289,20 @@ int fa_matmul_ws(fa_stream_t stream, fa_dtype in_t,
                  int64_t batch, int64_t M, int64_t N, int64_t K,
                  void *workspace, size_t workspace_bytes);
 
+/* Scan with a vector operator: out[i][j] = xss[0][j] op ... op xss[i][j] for
+ * xss, out : [n][k], without a transposed copy.  Replaces: the SegScan of
+ * `scan (map2 op) (replicate k ne) xss`, which the reference compiles with its
+ * two-pass scan (src/Futhark/CodeGen/ImpGen/GPU/SegScan/TwoPass.hs; the
+ * single-pass kernel refuses array operators, SegScan/SinglePass.hs
+ * canBeSinglePass).  Takes rows of whole 1 KiB strips (k * element size a
+ * multiple of 1024) of 4- or 8-byte elements: fa_vecscan_workspace_bytes is 0
+ * for every other shape and fa_vecscan then returns FA_ENOTSUP (transpose with
+ * fa_map_transpose, scan rows with fa_segscan_rows, transpose back).  The
+ * workspace's contents are irrelevant; xss, out and workspace 16-byte aligned. */
+size_t fa_vecscan_workspace_bytes(fa_dtype t, int64_t n, int64_t k);
+int fa_vecscan(fa_stream_t stream, fa_dtype t, fa_op op, const void *xss, int64_t n, int64_t k,
+               void *out, void *workspace, size_t workspace_bytes);
+
 /* ------------------------------------------------ builtin data movement
  * Batched 2-D transpose: dst[b][j][i] = src[b][i][j], src : [batch][rows][cols].
  * Replaces: map_transpose_{1,2,4,8}b and their low_height / low_width / small /

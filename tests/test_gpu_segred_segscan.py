@@ -448,9 +448,12 @@ def test_segred_reports_segments_that_are_not_segments(segops_lib):
 def test_scan_with_a_vector_operator(ctx, t, op):
     """scan (map2 op) (replicate k ne) xss: column j of the result is the scan of column j.
     Shapes: one column (an ordinary scan), few and many columns, more rows than a tile of the row
-    scan holds, sizes off every tile of the transposes, empty in either dimension."""
+    scan holds, sizes off every tile of the transposes, empty in either dimension; rows of whole
+    strips with fewer rows than chunks, rows that do not divide into chunks, one row."""
     for n, k in [(1, 1), (1000, 1), (7, 3), (1, 300), (1000, 4), (333, 33), (40001, 5), (70, 1000),
-                 (20000, 64), (0, 4), (4, 0)]:
+                 (20000, 64), (0, 4), (4, 0),
+                 # rows of whole 1 KiB strips take the kernels without a transposed copy
+                 (5, 256), (1000, 256), (40001, 512), (17, 1024), (1, 768), (3000, 128), (16385, 256)]:
         xss = _data(t, n * k, 17).reshape(n, k)
         out = ctx.call(f"vecscan_{op}_{t}", [f"{t}_2d"], ctx.new(f"{t}_2d", xss))
         got = out.values()
