@@ -27,6 +27,9 @@
 
 namespace fa {
 
+#ifndef HIST_ASM_MATCH
+#define HIST_ASM_MATCH 1
+#endif
 constexpr int HIST_BLOCK = 1024;
 constexpr int HIST_LDS_BYTES = 128 * 1024;  // bin storage per block
 constexpr int HIST_MAX_RANGES = 4;          // ranges covered by one launch
@@ -426,8 +429,6 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
   auto update = [&](int64_t bin, T v) {
     const bool valid = (uint64_t)bin < (uint64_t)H;
     const uint32_t b = valid ? (uint32_t)bin : 0u;
-    // The match is left to the compiler here: the hand-scheduled one of the
-    // radix scatter (rs_match2) made this kernel slower (345 against 295 us).
     uint32_t differ_lo = 0u, differ_hi = 0u;
     auto match_bit = [&](int bit) {
       const uint32_t me = (uint32_t)(((int32_t)(b << (31 - bit))) >> 31);  // 0 or ~0
@@ -435,7 +436,16 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
       differ_lo |= (uint32_t)m ^ me;
       differ_hi |= (uint32_t)(m >> 32) ^ me;
     };
-    if constexpr (INDEX_BITS > 0) {
+    if constexpr (INDEX_BITS >= 8 && HIST_ASM_MATCH) {
+      // the low eight bits by the hand-scheduled match of the radix scatter
+      // (H = 256 f32: 297 -> 262 us), the others as the compiler writes them
+      uint32_t same_lo, same_hi;
+      rs_match1(b, same_lo, same_hi);
+      differ_lo = ~same_lo;
+      differ_hi = ~same_hi;
+#pragma unroll
+      for (int bit = 8; bit < INDEX_BITS; bit++) match_bit(bit);
+    } else if constexpr (INDEX_BITS > 0) {
 #pragma unroll
       for (int bit = 0; bit < INDEX_BITS; bit++) match_bit(bit);
     } else {
@@ -670,10 +680,8 @@ static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, in
   } while (0)
   if (H > 256)
     FA_WAVE_PRIVATE(11);
-  else if (sizeof(T) == 8)
-    FA_WAVE_PRIVATE(8);
   else
-    FA_WAVE_PRIVATE(0);
+    FA_WAVE_PRIVATE(8);
 #undef FA_WAVE_PRIVATE
   return launch_status();
 }
