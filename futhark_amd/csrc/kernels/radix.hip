@@ -54,7 +54,7 @@ extern "C" int fa_radix_sort(fa_stream_t stream, int key_bytes, int val_bytes, c
                              void *keys_out, void *keys_tmp, const void *vals_in, void *vals_out,
                              void *vals_tmp, int64_t n, int begin_bit, int end_bit, void *scratch,
                              size_t scratch_bytes) {
-  if (n < 0 || n >= ((int64_t)1 << 31)) return FA_EINVAL;
+  if (n < 0 || n >= RS_MAX_N) return FA_EINVAL;
   if (key_bytes != 4 && key_bytes != 8) return FA_ENOTSUP;
   if (val_bytes != 0 && val_bytes != 4 && val_bytes != 8) return FA_ENOTSUP;
   if (begin_bit < 0 || end_bit > key_bytes * 8 || end_bit < begin_bit ||

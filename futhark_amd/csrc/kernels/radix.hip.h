@@ -18,6 +18,9 @@ constexpr int RS_WAVES = RS_BLOCK / WAVE;
 constexpr int RS_KPT = 16;  // keys per thread
 constexpr int RS_TILE = RS_BLOCK * RS_KPT;
 constexpr int RS_RADIX = 256;
+// Positions in the output are unsigned 32-bit numbers (offsets, counts, the
+// scatter's destinations); everything that scales with the tile count is 64-bit.
+constexpr int64_t RS_MAX_N = ((int64_t)1 << 32) - 1;
 constexpr int RS_DIES = 8;  // a block runs on die blockIdx.x % 8
 
 struct RsScratch {
@@ -423,7 +426,7 @@ __device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__
   __syncthreads();
   // The offsets come from this library's own histogram and scan; should they
   // ever be wrong, a store outside the output would fault the GPU, whereas a
-  // dropped key is a wrong result the caller can see.  n < 2^31.
+  // dropped key is a wrong result the caller can see.  n < 2^32 - 1.
   uint32_t dst[RS_KPT];
   const uint32_t limit = (uint32_t)n;
 #pragma unroll
@@ -478,7 +481,7 @@ template <class K, int VB, class DigitFn>
 static int rs_pass(hipStream_t st, const K *kin, K *kout, const void *vin, void *vout, int64_t n,
                    DigitFn fn, int pass, uint32_t epoch, const RsScratch &sc) {
   using V = typename ValType<VB>::T;
-  if (n >= ((int64_t)1 << 31)) return FA_EINVAL;  // positions are 32-bit
+  if (n >= RS_MAX_N) return FA_EINVAL;  // positions are unsigned 32-bit
   const size_t lds =
       RS_LDS_FIXED + (size_t)RS_TILE * (sizeof(K) > sizeof(V) ? sizeof(K) : sizeof(V));
   auto scatter = rs_scatter_kernel<K, VB, DigitFn>;

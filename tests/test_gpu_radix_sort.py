@@ -107,3 +107,41 @@ def test_config5_full_size_pairs(ctx):
     assert np.all(gv[1:][ties] > gv[:-1][ties])              # ties keep input order
     wk, wv = oracle.radix_sort(keys, vals)
     assert np.array_equal(gk, wk) and np.array_equal(gv, wv)
+
+
+def test_more_than_two_to_the_31_keys(ctx):
+    """Positions are unsigned 32-bit numbers, so the sort takes more than 2^31 keys.  The CPU
+    does not sort 8 GiB in the time a test has: the result is checked for order and, against the
+    input, for the same multiset (counts of the high and of the low 16 bits, sum and xor), in
+    pieces that keep the temporaries small."""
+    n = (1 << 31) + 12345
+    rng = np.random.default_rng(7)
+    keys = rng.integers(0, 1 << 32, n, dtype=np.uint32)
+    a = ctx.new("u32_1d", keys)
+    out = ctx.call("radix_sort_u32", ["u32_1d"], a)
+    a.free()
+    got = out.values()
+    out.free()
+    ctx.clear_caches()  # 25 GiB of device buffers go back to the driver
+    assert got.shape == (n,)
+
+    def summary(x):
+        hi = np.zeros(1 << 16, np.int64)
+        lo = np.zeros(1 << 16, np.int64)
+        total, parity = 0, 0
+        step = 1 << 26
+        for i in range(0, n, step):
+            p = x[i:i + step]
+            hi += np.bincount(p >> 16, minlength=1 << 16)
+            lo += np.bincount(p & 0xFFFF, minlength=1 << 16)
+            total = (total + int(p.sum(dtype=np.uint64))) & ((1 << 64) - 1)
+            parity ^= int(np.bitwise_xor.reduce(p))
+        return hi, lo, total, parity
+
+    step = 1 << 26
+    for i in range(0, n - 1, step):
+        p = got[i:i + step + 1]
+        assert np.all(p[:-1] <= p[1:]), i
+    want, have = summary(keys), summary(got)
+    assert np.array_equal(want[0], have[0]) and np.array_equal(want[1], have[1])
+    assert want[2:] == have[2:]
