@@ -136,6 +136,7 @@ class Segops:
         L.futhark_entry_reduce_compose_i32.argtypes = [vp, pp, vp]
         L.futhark_entry_sumsq_f32.argtypes = [vp, vp, vp]
         L.futhark_entry_scan_norm_f32.argtypes = [vp, pp, vp]
+        L.futhark_entry_reduce_summax_f32.argtypes = [vp, pp, vp]
         L.futhark_entry_rows_fraction_f32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u64.argtypes = [vp, pp, vp]

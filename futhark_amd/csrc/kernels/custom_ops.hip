@@ -83,6 +83,31 @@ __global__ void unzip_pairs_kernel(const int32_t *in, int32_t *a, int32_t *b, in
 
 }  // namespace
 
+// Two operators in one SegRed (a reduction with several SegBinOps is one
+// kernel in the reference too, SegRed.hs:157-199: the operators' accumulators
+// sit side by side and every element is read once): sum and maximum of xs.
+namespace {
+struct SumMax {
+  float sum, max;
+};
+struct OpSumMax {
+  static constexpr bool commutative = true;
+  static __host__ __device__ __forceinline__ SumMax identity() { return SumMax{0.0f, -INFINITY}; }
+  static __host__ __device__ __forceinline__ SumMax apply(SumMax a, SumMax b) {
+    return SumMax{a.sum + b.sum, OpMax<float>::apply(a.max, b.max)};
+  }
+};
+struct Twice {
+  static __device__ __forceinline__ SumMax apply(float x, int64_t) { return SumMax{x, x}; }
+};
+}  // namespace
+
+extern "C" int fa_reduce_summax_f32(fa_stream_t stream, const float *xs, int64_t n, float *out2,
+                                    void *scratch, size_t scratch_bytes, uint32_t epoch) {
+  return launch_reduce<float, SumMax, Twice, OpSumMax>((hipStream_t)stream, xs, n, (SumMax *)out2,
+                                                      scratch, scratch_bytes, epoch);
+}
+
 extern "C" int fa_reduce_argmax_i32(fa_stream_t stream, const int32_t *xs, int64_t n, int32_t *out2,
                                     void *scratch, size_t scratch_bytes, uint32_t epoch) {
   return launch_reduce<int32_t, ValIdx, ZipIndex, OpArgmax>((hipStream_t)stream, xs, n, (ValIdx *)out2,

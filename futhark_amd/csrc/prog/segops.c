@@ -831,6 +831,11 @@ static int sumsq_fn(fa_stream_t s, const void *xs, int64_t n, void *out, void *s
 }
 
 /* A reduction whose result is a pair of i32, returned as a [2]i32 array. */
+static int summax_fn(fa_stream_t s, const void *xs, int64_t n, void *out, void *sc, size_t sb,
+                     uint32_t e) {
+  return fa_reduce_summax_f32(s, (const float *)xs, n, (float *)out, sc, sb, e);
+}
+
 static int do_pair_reduce(struct futhark_context *ctx, custom_reduce_fn fn, const char *name,
                           struct fut_array **out, const struct fut_array *in) {
   const int64_t two = 2;
@@ -849,6 +854,14 @@ int futhark_entry_reduce_argmax_i32(struct futhark_context *ctx, struct futhark_
                                     const struct futhark_i32_1d *in0) {
   ENTER(ctx);
   int ret = do_pair_reduce(ctx, reduce_argmax_fn, "segred_argmax", (struct fut_array **)out0, &in0->a);
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_reduce_summax_f32(struct futhark_context *ctx, struct futhark_f32_1d **out0,
+                                    const struct futhark_f32_1d *in0) {
+  ENTER(ctx);
+  int ret = do_pair_reduce(ctx, summax_fn, "segred_summax", (struct fut_array **)out0, &in0->a);
   LEAVE(ctx);
   return ret;
 }

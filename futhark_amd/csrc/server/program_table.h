@@ -257,6 +257,9 @@ static int e_sumsq_f32(struct futhark_context *c, struct value *o, struct value 
 static int e_rows_fraction_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_rows_fraction_f32(c, (struct futhark_f32_2d **)&o->u.arr, ARRP(i[0]));
 }
+static int e_reduce_summax_f32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_reduce_summax_f32(c, (struct futhark_f32_1d **)&o->u.arr, ARRP(i[0]));
+}
 static int e_scan_norm_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_scan_norm_f32(c, (struct futhark_f32_1d **)&o->u.arr, ARRP(i[0]));
 }
@@ -355,6 +358,7 @@ static const struct entry entries[] = {
     {"reduce_compose_i32", e_reduce_compose_i32, "[]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
     {"sumsq_f32", e_sumsq_f32, "f32", 0, 1, {"[]f32"}, {0}, {NULL}},
     {"scan_norm_f32", e_scan_norm_f32, "[]f32", 1, 1, {"[]f32"}, {0}, {NULL}},
+    {"reduce_summax_f32", e_reduce_summax_f32, "[]f32", 1, 1, {"[]f32"}, {0}, {NULL}},
     {"rows_fraction_f32", e_rows_fraction_f32, "[][]f32", 1, 1, {"[][]f32"}, {0}, {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {MATMUL_PARAM, NULL}},
     {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {MATMUL_PARAM, NULL}},

@@ -80,6 +80,7 @@ def entry_points() -> dict:
         _entry("reduce_compose_i32", "[]i32", [("abs", "[][]i32")]),
         _entry("sumsq_f32", "f32", [("xs", "[]f32")]),
         _entry("scan_norm_f32", "[]f32", [("xs", "[]f32")]),
+        _entry("reduce_summax_f32", "[]f32", [("xs", "[]f32")]),
         _entry("rows_fraction_f32", "[][]f32", [("xss", "[][]f32")]),
         _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")], [MATMUL_PARAM]),
         _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")], [MATMUL_PARAM]),

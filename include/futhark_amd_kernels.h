@@ -348,6 +348,8 @@ int fa_iota(fa_stream_t stream, fa_dtype t, void *dst, int64_t n,
  *   fa_reduce_compose_i32: fold of affine maps (FA_COMPOSE, not commutative) in
  *                          element order (SegRed.hs:836-921); out2: 2 x i32
  *   fa_sumsq_f32:         reduce (+) 0 (map (\x -> x*x) xs)
+ *   fa_reduce_summax_f32: (reduce (+) 0 xs, reduce f32.max (-inf) xs) in one kernel, two
+ *                         operators side by side (SegRed.hs:157-199); out2: 2 x f32
  *   fa_scan_norm_f32:     map sqrt (scan (+) 0 (map (\x -> x*x) xs))
  *   fa_hist_argmax_i32:   reduce_by_index with argmax into dest [H][2]i32 (updated
  *                         in place), bins locked while updated because the tuple's
@@ -363,6 +365,8 @@ int fa_reduce_compose_i32(fa_stream_t stream, const int32_t *abs, int64_t n, int
                           void *scratch, size_t scratch_bytes, uint32_t epoch);
 int fa_sumsq_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
                  void *scratch, size_t scratch_bytes, uint32_t epoch);
+int fa_reduce_summax_f32(fa_stream_t stream, const float *xs, int64_t n, float *out2,
+                         void *scratch, size_t scratch_bytes, uint32_t epoch);
 int fa_scan_norm_f32(fa_stream_t stream, const float *xs, int64_t n, float *out,
                      void *scratch, size_t scratch_bytes, uint32_t epoch);
 /* map (\r -> let t = reduce (+) 0 r in map (/ t) (scan (+) 0 r)) xss for

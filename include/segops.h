@@ -341,6 +341,9 @@ int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhar
  *   entry reduce_compose_i32 (abs: [][2]i32) : [2]i32 =    -- compose as above; does not commute
  *     let (a, b) = reduce compose (1, 0) (map (\r -> (r[0], r[1])) abs) in [a, b]
  *   entry sumsq_f32 (xs: []f32) : f32 = reduce (+) 0 (map (\x -> x * x) xs)
+ *   entry reduce_summax_f32 (xs: []f32) : [2]f32 =
+ *     let (s, m) = reduce (\(a,b) (c,d) -> (a + c, f32.max b d)) (0, -f32.inf) (zip xs xs) in [s, m]
+ *                                   -- two operators in one SegRed, SegRed.hs:157-199
  *   entry scan_norm_f32 (xs: []f32) : []f32 = map f32.sqrt (scan (+) 0 (map (\x -> x * x) xs))
  *   entry rows_fraction_f32 (xss: [][]f32) : [][]f32 =
  *     map (\r -> let t = reduce (+) 0 r in map (/ t) (scan (+) 0 r)) xss
@@ -356,6 +359,8 @@ int futhark_entry_reduce_compose_i32(struct futhark_context *ctx, struct futhark
                                      const struct futhark_i32_2d *in0);
 int futhark_entry_sumsq_f32(struct futhark_context *ctx, float *out0,
                             const struct futhark_f32_1d *in0);
+int futhark_entry_reduce_summax_f32(struct futhark_context *ctx, struct futhark_f32_1d **out0,
+                                    const struct futhark_f32_1d *in0);
 int futhark_entry_scan_norm_f32(struct futhark_context *ctx, struct futhark_f32_1d **out0,
                                 const struct futhark_f32_1d *in0);
 int futhark_entry_rows_fraction_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,

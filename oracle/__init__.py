@@ -202,6 +202,13 @@ def sumsq_f32(xs, variant: str = "lit"):
     return reduce("add", "f32", sq, variant)
 
 
+def reduce_summax_f32(xs, variant: str = "lit"):
+    """[reduce (+) 0 xs, reduce f32.max (-inf) xs]: the fold of the pair operator
+    (a,b) (c,d) -> (a + c, max b d) from (0, -inf) over zip xs xs."""
+    xs = _arr(xs, np.float32)
+    return np.array([reduce("add", "f32", xs, variant), reduce("max", "f32", xs)], dtype=np.float64 if variant == "f64acc" else np.float32)
+
+
 def scan_norm_f32(xs, variant: str = "lit"):
     """map f32.sqrt (scan (+) 0 (map (\\x -> x*x) xs))."""
     xs = _arr(xs, np.float32)

@@ -103,3 +103,15 @@ def test_segops_inside_a_block(ctx):
     want = oracle.rows_fraction_f32(z)
     assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isinf(got), np.isinf(want))
     assert np.array_equal(np.sign(got[np.isinf(got)]), np.sign(want[np.isinf(want)]))
+
+
+def test_two_operators_in_one_reduction(ctx):
+    """reduce_summax_f32: sum and maximum side by side, every element read once.  The maximum is
+    exact; the sum within 1e-5 of the f64-accumulated oracle (mixed signs: relative to sum |x|)."""
+    for n in SIZES:
+        xs = (dg.uniform_f32(27, n) * 4 - 2).astype(np.float32)
+        got = ctx.call("reduce_summax_f32", ["f32_1d"], ctx.new("f32_1d", xs)).values()
+        want = oracle.reduce_summax_f32(xs, "f64acc")
+        assert got.shape == (2,)
+        assert abs(float(got[0]) - float(want[0])) <= 1e-5 * float(np.abs(xs).sum(dtype=np.float64)) + 1e-30, n
+        assert float(got[1]) == float(want[1]) or (n == 0 and np.isneginf(got[1])), n

@@ -46,7 +46,7 @@ def make_inputs(name, e, rng):
         return ([(rng.random(N) < 0.2).astype(np.uint8)] if fam == "segscan" else []) + [ab]
     if name == "hist_argmax_i32":
         return [np.array(5, np.int64), rng.integers(-1, 7, N).astype(np.int32), _vals(rng, "i32", N)]
-    if name in ("sumsq_f32", "scan_norm_f32"):
+    if name in ("sumsq_f32", "scan_norm_f32", "reduce_summax_f32"):
         return [_vals(rng, "f32", N)]
     if name == "rows_fraction_f32":
         return [np.abs(_vals(rng, "f32", (6, 7))) + np.float32(1)]

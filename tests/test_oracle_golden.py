@@ -449,3 +449,11 @@ def test_rows_fraction_oracle_is_pinned():
     assert np.array_equal(oracle.rows_fraction_f32(xss * np.float32(4)), oracle.rows_fraction_f32(xss))
     one_row = oracle.rows_fraction_f32(xss[2:3])
     assert np.array_equal(one_row[0], oracle.rows_fraction_f32(xss)[2])
+
+
+def test_two_operator_reduction_oracle_is_pinned():
+    xs = np.array([1.5, -2.0, 8.25, 0.5], np.float32)
+    assert oracle.reduce_summax_f32(xs).tolist() == [8.25, 8.25]
+    assert oracle.reduce_summax_f32(xs[:2]).tolist() == [-0.5, 1.5]
+    e = oracle.reduce_summax_f32(np.zeros(0, np.float32))
+    assert e[0] == 0 and np.isneginf(e[1])
