@@ -255,8 +255,25 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void matmul16_kernel(
       else f.b[nt].z = h.x, f.b[nt].w = h.y;
     }
   };
-  auto k16_step = [&](const unsigned char *stage, int ks, const Frags &cur, Frags &next,
-                      int next_kt, int next_stage, auto fetch) __attribute__((always_inline)) {
+  const int KT = K / MM16_BK;
+  // All of this wave's loads have landed and its LDS reads have returned, then
+  // all waves': the next tile is public and the current one may be overwritten.
+  auto publish = [&]() {
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    __syncthreads();
+  };
+  // With more MFMAs in a step than LDS reads (MM16_EARLY), the barrier that
+  // publishes the next tile is taken inside the last k16 step of the current
+  // one, after MFMA number PUBLISH_AT, and the first fragments of the next tile
+  // are read behind the remaining MFMAs: the next tile starts with an MFMA
+  // instead of a barrier and a dozen LDS round trips.  (The current tile's LDS
+  // bytes are no longer needed by then: the fragments of its last step were
+  // read during the step before.)
+  constexpr bool MM16_EARLY = MFMAS > READS;
+  constexpr int PUBLISH_AT = MFMAS - READS - 1;
+  auto k16_step = [&](const unsigned char *stage, const unsigned char *other, int ks,
+                      const Frags &cur, Frags &next, int next_kt, int next_stage,
+                      auto fetch) __attribute__((always_inline)) {
     static_for<MFMAS>([&](auto ic) __attribute__((always_inline)) {
       constexpr int i = decltype(ic)::value;
       constexpr int nt = i / MM16_MT, mt = i % MM16_MT;
@@ -268,49 +285,51 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void matmul16_kernel(
         acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
             bit_cast<f16x8>(cur.a[mt]), bit_cast<f16x8>(bfrag), acc[mt][nt], 0, 0, 0);
       }
-      if (ks + 1 < KSTEPS && i < READS) issue_read(stage, ks + 1, i, next);
+      if (ks + 1 < KSTEPS) {
+        if (i < READS) issue_read(stage, ks + 1, i, next);
+      } else if constexpr (MM16_EARLY) {
+        if (i == PUBLISH_AT) publish();
+        if (i > PUBLISH_AT) issue_read(other, 0, i - PUBLISH_AT - 1, next);
+      }
       if constexpr (decltype(fetch)::value)
         if (ks < MM16_LOAD_KSTEPS && i % MFMAS_PER_LOAD == MFMAS_PER_LOAD - 1)
         fetch_one(next_kt, next_stage, ks * LOADS_PER_STEP + i / MFMAS_PER_LOAD);
       __builtin_amdgcn_sched_barrier(0);
     });
   };
-  auto multiply = [&](const unsigned char *stage, int next_kt, int next_stage,
-                      auto fetch) __attribute__((always_inline)) {
-    Frags f0, f1;
+  Frags f0, f1;
+  auto first_reads = [&](const unsigned char *stage) __attribute__((always_inline)) {
     static_for<READS>([&](auto ic) __attribute__((always_inline)) { issue_read(stage, 0, decltype(ic)::value, f0); });
     __builtin_amdgcn_sched_barrier(0);
+  };
+  auto multiply = [&](const unsigned char *stage, const unsigned char *other, int next_kt,
+                      int next_stage, auto fetch) __attribute__((always_inline)) {
+    if constexpr (!MM16_EARLY) first_reads(stage);
+    static_assert(KSTEPS % 2 == 0, "the fragment buffers swap an even number of times per tile");
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks += 2) {
-      k16_step(stage, ks, f0, f1, next_kt, next_stage, fetch);
-      k16_step(stage, ks + 1, f1, f0, next_kt, next_stage, fetch);
+      k16_step(stage, other, ks, f0, f1, next_kt, next_stage, fetch);
+      k16_step(stage, other, ks + 1, f1, f0, next_kt, next_stage, fetch);
     }
-  };
-  // All of this wave's loads have landed, then all waves': the tile is public.
-  auto publish = [&]() {
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    __syncthreads();
+    if constexpr (!MM16_EARLY) publish();
   };
 
-  const int KT = K / MM16_BK;
 #pragma unroll
   for (int j = 0; j < LOADS; j++) fetch_one(0, 0, j);
   publish();
+  if constexpr (MM16_EARLY) first_reads(lds);
   // While tile kt is multiplied out of one stage, tile kt+1 streams into the
   // other, which every wave finished reading before the previous barrier.
   // The tile after the last one is the last one again (loaded, never used),
   // which keeps the loop free of special cases.
   constexpr std::true_type with_fetch{};
+  unsigned char *const stage0 = lds, *const stage1 = lds + MM16_STAGE_BYTES;
   for (int kt = 0; kt + 1 < KT; kt += 2) {
-    multiply(lds, kt + 1, 1, with_fetch);
-    publish();
-    multiply(lds + MM16_STAGE_BYTES, kt + 2 < KT ? kt + 2 : KT - 1, 0, with_fetch);
-    publish();
+    multiply(stage0, stage1, kt + 1, 1, with_fetch);
+    multiply(stage1, stage0, kt + 2 < KT ? kt + 2 : KT - 1, 0, with_fetch);
   }
-  if (KT & 1) {
-    multiply(lds, KT - 1, 1, with_fetch);
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // no load outlives the wave
-  }
+  if (KT & 1) multiply(stage0, stage1, KT - 1, 1, with_fetch);
+  __builtin_amdgcn_s_waitcnt(0x0F70);  // no load outlives the wave
 
   // C fragment: element e of lane l is row (e/4)*8 + (l/32)*4 + e%4, column l%32.
 #pragma unroll
