@@ -71,7 +71,8 @@ __device__ __forceinline__ void sri_mark(int64_t *bounds, int which, int64_t t_l
 
 static __global__ __launch_bounds__(256) void segred_bounds_kernel(
     const int64_t *__restrict__ offsets, const int64_t *__restrict__ lens, int64_t m, int64_t n,
-    int64_t tile_elems, int64_t num_tiles, int64_t *__restrict__ bounds) {
+    int64_t tile_elems, int64_t num_tiles, int64_t *__restrict__ bounds, int32_t *failure,
+    int32_t code) {
   const int lane = lane_id();
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
   const bool live = i <= m;  // whole waves stay in the loops of sri_mark
@@ -84,7 +85,15 @@ static __global__ __launch_bounds__(256) void segred_bounds_kernel(
     }
     if (i < m) {
       s_here = offsets[i];
-      e_here = s_here + lens[i];
+      const int64_t l = lens[i];
+      e_here = s_here + l;
+      // What the kernels require of segment i (and of its place after segment
+      // i - 1), checked while its numbers are here anyway.
+      if (failure != nullptr) {
+        const bool ok = s_here >= 0 && l >= 0 && s_here <= n && l <= n - s_here &&
+                        (i == 0 || e_prev <= s_here);
+        if (!ok) *failure = code;
+      }
     }
   }
   // Interior boundaries are t = 0..num_tiles-1 at p_t = t * tile_elems.
@@ -302,7 +311,8 @@ static size_t sri_scratch_bytes(int64_t tiles) {
 template <class T, class Op>
 static int launch_segred_irregular(hipStream_t s, const void *vs, int64_t n,
                                    const int64_t *offsets, const int64_t *lens, int64_t m,
-                                   void *out, void *scratch, size_t scratch_bytes) {
+                                   void *out, void *scratch, size_t scratch_bytes,
+                                   int32_t *failure, int32_t code) {
   if (m == 0) return 0;
   if (n == 0) {  // every segment is empty
     int grid = (int)(ceil_div(m, 256) < 4096 ? ceil_div(m, 256) : 4096);
@@ -320,7 +330,7 @@ static int launch_segred_irregular(hipStream_t s, const void *vs, int64_t n,
   int64_t *bounds = (int64_t *)scratch;
   SriTileRec *recs = (SriTileRec *)((char *)scratch + (size_t)(tiles + 1) * 16);
   hipLaunchKernelGGL(segred_bounds_kernel, dim3((unsigned)ceil_div(m + 1, (int64_t)256)),
-                     dim3(256), 0, s, offsets, lens, m, n, tile_elems, tiles, bounds);
+                     dim3(256), 0, s, offsets, lens, m, n, tile_elems, tiles, bounds, failure, code);
   hipLaunchKernelGGL((segred_tiles_kernel<T, Op>), dim3((unsigned)tiles), dim3(SRI_BLOCK), 0, s,
                      (const T *)vs, n, offsets, lens, (const int64_t *)bounds, (T *)out, recs);
   hipLaunchKernelGGL((segred_fixup_kernel<T, Op>),
@@ -373,5 +383,22 @@ extern "C" int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op, con
     return FA_EINVAL;
   hipStream_t s = (hipStream_t)stream;
   FA_DISPATCH_TYPE_OP(launch_segred_irregular, t, op, s, vs, n, offsets, lens, m, out, scratch,
-                      scratch_bytes);
+                      scratch_bytes, (int32_t *)nullptr, 0);
+}
+
+extern "C" int fa_segred_irregular_checked(fa_stream_t stream, fa_dtype t, fa_op op, const void *vs,
+                                           int64_t n, const int64_t *offsets, const int64_t *lens,
+                                           int64_t m, void *out, void *scratch,
+                                           size_t scratch_bytes, int32_t *failure, int32_t code) {
+  if (failure == nullptr) return FA_EINVAL;
+  if (n < 0 || m < 0 || (m > 0 && (offsets == nullptr || lens == nullptr || out == nullptr)) ||
+      (n > 0 && m > 0 && (vs == nullptr || scratch == nullptr)))
+    return FA_EINVAL;
+  hipStream_t s = (hipStream_t)stream;
+  if (m > 0 && n == 0) {  // no kernel of the reduction looks at the segments then
+    const int rc = fa_segments_check(stream, offsets, lens, m, n, failure, code);
+    if (rc != 0) return rc;
+  }
+  FA_DISPATCH_TYPE_OP(launch_segred_irregular, t, op, s, vs, n, offsets, lens, m, out, scratch,
+                      scratch_bytes, failure, code);
 }

@@ -285,11 +285,7 @@ static int do_segred(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
   /* The kernels are memory-safe whatever the segments are, but their result is
      only defined for ordered, disjoint segments inside the array: anything
      else makes the next synchronisation fail, as an index out of bounds does
-     in a compiled program. */
-  int chk = fa_segments_check(ctx->stream, (const int64_t *)offsets->mem.mem,
-                              (const int64_t *)lens->mem.mem, m, n, RTS_FAILURE_WORD(ctx),
-                              RTS_FAILURE_SEGMENTS);
-  if (chk != 0) return rts_kernel_end(ctx, NULL, "segments_check", chk);
+     in a compiled program.  The reduction's first kernel checks them. */
   struct fut_array *res = out_array(ctx, m * (int64_t)es, 1, &m, "segred.out");
   if (res == NULL) return FUTHARK_OUT_OF_MEMORY;
   /* Plain workspace from the pool; not the look-back scratch of the scans,
@@ -301,10 +297,11 @@ static int do_segred(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
     struct rts_event *ev = rts_kernel_begin(
         ctx, "segred_irregular",
         rts_msgprintf("{\"n\":%lld,\"segments\":%lld}", (long long)n, (long long)m));
-    int code = fa_segred_irregular(ctx->stream, t, op, vs->mem.mem, n,
-                                   (const int64_t *)offsets->mem.mem,
-                                   (const int64_t *)lens->mem.mem, m, res->mem.mem, scratch.mem,
-                                   (size_t)scratch.size);
+    int code = fa_segred_irregular_checked(ctx->stream, t, op, vs->mem.mem, n,
+                                           (const int64_t *)offsets->mem.mem,
+                                           (const int64_t *)lens->mem.mem, m, res->mem.mem,
+                                           scratch.mem, (size_t)scratch.size,
+                                           RTS_FAILURE_WORD(ctx), RTS_FAILURE_SEGMENTS);
     err = rts_kernel_end(ctx, ev, "segred_irregular", code);
   }
   rts_memblock_unref(ctx, &scratch, "segred.scratch");

@@ -201,6 +201,15 @@ int fa_segred_irregular(fa_stream_t stream, fa_dtype t, fa_op op,
                         const int64_t *offsets, const int64_t *lens, int64_t m,
                         void *out, void *scratch, size_t scratch_bytes);
 
+/* fa_segred_irregular with the check of fa_segments_check (below) done by its
+ * first kernel, which reads every offset and length anyway: one launch less
+ * than the check followed by the reduction. */
+int fa_segred_irregular_checked(fa_stream_t stream, fa_dtype t, fa_op op,
+                                const void *vs, int64_t n,
+                                const int64_t *offsets, const int64_t *lens, int64_t m,
+                                void *out, void *scratch, size_t scratch_bytes,
+                                int32_t *failure, int32_t code);
+
 /* Checks what fa_segred_irregular requires of its segments (in order, disjoint,
  * inside [0, n)): stores `code` into *failure (device-visible memory, e.g. a
  * pinned host word) when they are not, and leaves it alone otherwise.  A
