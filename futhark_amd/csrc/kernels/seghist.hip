@@ -27,6 +27,18 @@
 
 namespace fa {
 
+#ifndef HIST_TAG_MATCH
+#define HIST_TAG_MATCH 1
+#endif
+#ifndef HIST_TAG_MARGIN
+#define HIST_TAG_MARGIN 0
+#endif
+#ifndef HIST_VEC_UNROLL
+#define HIST_VEC_UNROLL 8
+#endif
+#ifndef HIST_CONTENDED
+#define HIST_CONTENDED 32
+#endif
 #ifndef HIST_ASM_MATCH
 #define HIST_ASM_MATCH 1
 #endif
@@ -406,7 +418,8 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
 // A wave keeps 2^copies_log2 copies of its histogram where LDS allows, lane l
 // using copy l mod 2^copies_log2, so that fewer lanes share a cell and fewer
 // of them need the atomic.
-template <class T, class I, int INDEX_BITS /* 0: as many as `index_bits` says, not unrolled */>
+template <class T, class I, int INDEX_BITS /* 0: as many as `index_bits` says, not unrolled */,
+          bool TAGS = false>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
     const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t H,
     int index_bits, int copies_log2) {
@@ -419,6 +432,9 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
   const int copies = 1 << copies_log2;
   // volatile: the compiler must not carry a bin across the rounds below in a register
   volatile T *mine = sh + ((size_t)wave * nb << copies_log2);
+  // TAGS: one byte per cell behind the histograms of the block, see update_tagged
+  volatile uint8_t *tags = reinterpret_cast<uint8_t *>(sh + ((size_t)WAVES * nb << copies_log2)) +
+                           ((size_t)wave * nb << copies_log2);
   for (int i = threadIdx.x; i < nb * WAVES * copies; i += HIST_BLOCK) sh[i] = T(0);
   __syncthreads();
   const uint32_t my_copy = (uint32_t)lane_id() & (uint32_t)(copies - 1);
@@ -426,6 +442,8 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
   uint32_t copy_mask = 0u;
   for (int l = (int)my_copy; l < 32; l += copies) copy_mask |= 1u << l;
 
+  // lanes of this wave that had to follow another lane in the current step
+  int followers = 0;
   auto update = [&](int64_t bin, T v) {
     const bool valid = (uint64_t)bin < (uint64_t)H;
     const uint32_t b = valid ? (uint32_t)bin : 0u;
@@ -469,6 +487,26 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
     if (turn > 0)
       AtomicUpdate<T, OpAdd<T>, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(const_cast<T *>(&mine[slot]), v);
     __builtin_amdgcn_wave_barrier();
+    if constexpr (TAGS) followers += __builtin_popcountll(__ballot(turn > 0));
+  };
+
+  // TAGS: which of the lanes that hit a cell in the same step goes first is
+  // settled by the cell's tag instead of ballots: every lane writes its number
+  // into the tag and reads it back; the one whose number stayed adds with an
+  // ordinary read and write, the others follow with the atomic.  Two LDS
+  // operations in place of some forty instructions of matching.
+  auto update_tagged = [&](int64_t bin, T v) {
+    const bool valid = (uint64_t)bin < (uint64_t)H;
+    const uint32_t slot = ((valid ? (uint32_t)bin : 0u) << copies_log2) + my_copy;
+    if (valid) tags[slot] = (uint8_t)lane_id();
+    __builtin_amdgcn_wave_barrier();
+    const bool first = valid && tags[slot] == (uint8_t)lane_id();
+    if (first) mine[slot] = mine[slot] + v;
+    __builtin_amdgcn_wave_barrier();
+    if (valid && !first)
+      AtomicUpdate<T, OpAdd<T>, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(const_cast<T *>(&mine[slot]), v);
+    __builtin_amdgcn_wave_barrier();
+    followers += __builtin_popcountll(__ballot(valid && !first));
   };
 
   const int64_t nvec = n / VEC;
@@ -490,13 +528,30 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
         bv[e] = T(0);
       }
     }
+    if constexpr (TAGS) {
+      // Many lanes on few cells (skewed indices): the tags of a step cost a
+      // write conflict per lane of a cell, the ballots do not, so a wave
+      // whose last step had more than HIST_CONTENDED followers among its
+      // VEC * 64 updates takes the ballots for the next one.
+      const bool contended = followers > HIST_CONTENDED;
+      followers = 0;
+      if (contended) {
 #pragma unroll
-    for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
+        for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) update_tagged((int64_t)bi[e], bv[e]);
+      }
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
+    }
   }
   if (blockIdx.x == 0 && wave == 0) {  // the n % VEC elements at the end
     const int64_t t = nvec * VEC + lane_id();
     const bool in = lane_id() < VEC && t < n;
-    update(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
+    if constexpr (TAGS) update_tagged(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
+    else update(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
   }
   __syncthreads();
   for (int r = threadIdx.x; r < nb; r += HIST_BLOCK) {
@@ -655,6 +710,20 @@ constexpr int HIST_WAVE_PRIVATE_BYTES = HIST_LDS_BYTES / (HIST_BLOCK / WAVE);
 constexpr int HIST_WAVE_COPIES_MAX = 4;
 
 
+template <class T, class I, int BITS, bool TAGS>
+static int launch_wave_private_kernel(hipStream_t st, dim3 grid, size_t lds, const I *is,
+                                      const T *vs, int64_t n, T *dest, int64_t H, int index_bits,
+                                      int copies_log2) {
+  auto kernel = seghist_wave_private_kernel<T, I, BITS, TAGS>;
+  // Initialised once, under the lock C++ gives function-local statics.
+  static const hipError_t raised = hipFuncSetAttribute(
+      (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
+  if (raised != hipSuccess) return (int)raised;
+  hipLaunchKernelGGL(kernel, grid, dim3(HIST_BLOCK), lds, st, is, vs, n, dest, H, index_bits,
+                     copies_log2);
+  return launch_status();
+}
+
 template <class T, class I>
 static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
                                     int64_t H) {
@@ -667,28 +736,166 @@ static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, in
   int index_bits = 1;
   while (((int64_t)1 << index_bits) < H) index_bits++;
   // as many copies per wave (at most HIST_WAVE_COPIES_MAX) as leave room for two blocks on a CU
-  const size_t one = (size_t)H * sizeof(T) * (HIST_BLOCK / WAVE);
+  // a byte of tag per cell where one block with them fits, else the ballots
+  const bool tags = HIST_TAG_MATCH && sizeof(T) == 4 &&
+                    (size_t)H * (sizeof(T) + 1) * (HIST_BLOCK / WAVE) <= HIST_LDS_BYTES;
+  const size_t one = (size_t)H * (sizeof(T) + (tags ? 1 : 0)) * (HIST_BLOCK / WAVE);
+  const size_t margin = tags ? HIST_TAG_MARGIN : 4096;
   int copies_log2 = 0;
-  while ((1 << copies_log2) < HIST_WAVE_COPIES_MAX && (one << (copies_log2 + 1)) * 2 + 4096 <= 160 * 1024)
+  while ((1 << copies_log2) < HIST_WAVE_COPIES_MAX && (one << (copies_log2 + 1)) * 2 + margin <= 160 * 1024)
     copies_log2++;
   const size_t lds = one << copies_log2;
-  const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
+  const int per_cu = lds * 2 + margin <= 160 * 1024 ? 2 : 1;
   const dim3 grid(hist_num_cus() * per_cu);
-#define FA_WAVE_PRIVATE(BITS)                                                                  \
-  do {                                                                                         \
-    auto kernel = seghist_wave_private_kernel<T, I, BITS>;                                     \
-    /* Initialised once, under the lock C++ gives function-local statics. */                   \
-    static const hipError_t raised = hipFuncSetAttribute(                                      \
-        (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);     \
-    if (raised != hipSuccess) return (int)raised;                                              \
-    hipLaunchKernelGGL(kernel, grid, dim3(HIST_BLOCK), lds, st, is, vs, n, dest, H, index_bits, \
-                       copies_log2);                                                           \
-  } while (0)
+  if (tags && H > 256)
+    return launch_wave_private_kernel<T, I, 11, true>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
+  if (tags)
+    return launch_wave_private_kernel<T, I, 8, true>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
   if (H > 256)
-    FA_WAVE_PRIVATE(11);
-  else
-    FA_WAVE_PRIVATE(8);
-#undef FA_WAVE_PRIVATE
+    return launch_wave_private_kernel<T, I, 11, false>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
+  return launch_wave_private_kernel<T, I, 8, false>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
+}
+
+// ------------------------------- float sums into few bins that are vectors
+// `reduce_by_index dest (map2 (+)) (replicate m 0) is vss` with float elements:
+// the same idea as seghist_wave_private_kernel, with a bin of m cells.  A lane
+// takes 16 bytes of a row of vss at a time (m is a multiple of that), so the
+// lanes of a step cover consecutive rows; rows of one step with the same index
+// are told apart by the tag of the bin (the row number's low byte, written by
+// every lane of the row and read back): the row whose tag stayed adds its
+// vector with ordinary 16-byte reads and writes, the other rows follow with
+// the LDS float atomic.  Blocks of four waves, so that a wave's histogram may
+// take up to 40 KiB (H0 * m <= 10 Ki cells of 4 bytes).
+constexpr int HIST_VEC_BLOCK = 256;
+constexpr int HIST_VEC_LDS_MAX = 160 * 1024;
+
+template <class T, class I>
+__global__ __launch_bounds__(HIST_VEC_BLOCK) void seghist_wave_private_vec_kernel(
+    const I *__restrict__ is, const T *__restrict__ vss, int64_t n_groups, T *dest, int64_t H0,
+    int64_t m) {
+  constexpr int G = 16 / (int)sizeof(T);  // elements of a lane per step
+  constexpr int WAVES = HIST_VEC_BLOCK / WAVE;
+  constexpr int U = HIST_VEC_UNROLL;  // steps of a lane whose loads are in flight together
+  using VT = T __attribute__((ext_vector_type(G)));
+  extern __shared__ __align__(16) unsigned char s_raw[];
+  T *sh = reinterpret_cast<T *>(s_raw);
+  const int cells = (int)(H0 * m);
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / WAVE));
+  for (int i = threadIdx.x; i < cells * WAVES; i += HIST_VEC_BLOCK) sh[i] = T(0);
+  __syncthreads();
+  // volatile: the order of the LDS operations below is the algorithm
+  volatile T *mine = sh + (size_t)wave * cells;
+  volatile uint8_t *tags =
+      reinterpret_cast<uint8_t *>(sh + (size_t)WAVES * cells) + (size_t)wave * H0;
+
+  auto add_row_part = [&](bool in, I index, int64_t row, int col, const VT &v) {
+    const bool valid = in && (uint64_t)(int64_t)index < (uint64_t)H0;
+    const uint32_t bin = valid ? (uint32_t)index : 0u;
+    // rows of one step are consecutive and at most 64: the low byte tells them apart
+    const uint8_t tag = (uint8_t)row;
+    if (valid) tags[bin] = tag;
+    __builtin_amdgcn_wave_barrier();
+    const bool first = valid && tags[bin] == tag;
+    const uint32_t cell = bin * (uint32_t)m + (uint32_t)col;
+    if (first) {
+      volatile VT *p = reinterpret_cast<volatile VT *>(mine + cell);
+      const VT old = *p;
+      *p = old + v;
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (valid && !first) {
+#pragma unroll
+      for (int e = 0; e < G; e++)
+        AtomicUpdate<T, OpAdd<T>, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(
+            const_cast<T *>(&mine[cell + e]), v[e]);
+    }
+    __builtin_amdgcn_wave_barrier();
+  };
+
+  // group g = elements [g * G, g * G + G) of vss, inside row g * G / m.  A lane
+  // takes groups g0, g0 + stride, ... in batches of U whose loads are issued a
+  // batch ahead, without a condition (a group past the end reads the last one
+  // again and is dropped): loads under a condition would make every batch wait
+  // for all that are in flight.
+  struct Batch {
+    VT v[U];
+    I index[U];
+    int64_t row[U];
+    int col[U];
+  };
+  const int64_t stride = (int64_t)gridDim.x * HIST_VEC_BLOCK;
+  const int64_t last_group = n_groups - 1, last_row = last_group * G / m;
+  int64_t next = (int64_t)blockIdx.x * HIST_VEC_BLOCK + threadIdx.x;  // first group not fetched yet
+  int64_t row = next * G / m;
+  int col = (int)(next * G % m);
+  const int64_t row_step = stride * G / m;
+  const int col_step = (int)(stride * G % m);
+  auto fetch = [&](Batch &b) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int64_t g = next < last_group ? next : last_group;
+      b.v[u] = bit_cast<VT>(hist_load_nt(reinterpret_cast<const uint4 *>(vss) + g));
+      b.index[u] = is[row < last_row ? row : last_row];
+      b.row[u] = row;
+      b.col[u] = col;
+      next += stride;
+      row += row_step;
+      col += col_step;
+      if (col >= (int)m) {
+        col -= (int)m;
+        row++;
+      }
+    }
+  };
+  int64_t g = next;  // first group of the batch in `cur`
+  Batch cur;
+  fetch(cur);
+  while (g < n_groups) {
+    Batch ahead;
+    fetch(ahead);
+    __builtin_amdgcn_sched_barrier(0);  // keep the loads above what follows
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      add_row_part(g + u * stride < n_groups, cur.index[u], cur.row[u], cur.col[u], cur.v[u]);
+    cur = ahead;
+    g += U * stride;
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < cells; c += HIST_VEC_BLOCK) {
+    T acc = T(0);
+#pragma unroll
+    for (int w = 0; w < WAVES; w++) acc += sh[(size_t)w * cells + c];
+    if (!bits_equal(acc, T(0))) global_update<T, OpAdd<T>>(dest + c, acc);
+  }
+}
+
+// Bytes of LDS a block of seghist_wave_private_vec_kernel needs for [H0][m]
+// bins, or 0 when the kernel does not take them.
+template <class T> static size_t hist_vec_lds_bytes(int64_t H0, int64_t m) {
+  constexpr int64_t G = 16 / (int64_t)sizeof(T);
+  if (m % G != 0 || H0 > HIST_VEC_LDS_MAX || m > HIST_VEC_LDS_MAX) return 0;
+  const size_t bytes =
+      (size_t)(HIST_VEC_BLOCK / WAVE) * ((size_t)H0 * (size_t)m * sizeof(T) + (size_t)H0);
+  return bytes <= (size_t)HIST_VEC_LDS_MAX ? (bytes + 15) & ~(size_t)15 : 0;
+}
+
+template <class T, class I>
+static int launch_wave_private_vec_hist(hipStream_t st, const I *is, const T *vss,
+                                        int64_t n_updates, T *dest, int64_t H0, int64_t m) {
+  const size_t lds = hist_vec_lds_bytes<T>(H0, m);
+  if (lds == 0) return FA_EINVAL;
+  const int64_t n_groups = n_updates * m / (16 / (int64_t)sizeof(T));
+  int per_cu = (int)((size_t)HIST_VEC_LDS_MAX / lds);
+  if (per_cu > 8) per_cu = 8;
+  const int64_t grid = std::min<int64_t>((int64_t)hist_num_cus() * per_cu,
+                                         ceil_div(n_groups, (int64_t)HIST_VEC_BLOCK));
+  auto kernel = seghist_wave_private_vec_kernel<T, I>;
+  // Initialised once, under the lock C++ gives function-local statics.
+  static const hipError_t raised = hipFuncSetAttribute(
+      (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_VEC_LDS_MAX);
+  if (raised != hipSuccess) return (int)raised;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(HIST_VEC_BLOCK), lds, st, is, vss, n_groups,
+                     dest, H0, m);
   return launch_status();
 }
 
@@ -839,6 +1046,16 @@ static int launch_hist_shaped(hipStream_t st, const void *is, const void *js, in
     return FA_EALIGN;
   const int64_t lds_limit =
       (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
+  if constexpr (std::is_same<Op, OpAdd<T>>::value && std::is_floating_point<T>::value) {
+    // sums of float vectors into few bins: a histogram per wave, no float atomic per element
+    if (js == nullptr && m > 1 && hist_vec_lds_bytes<T>(H0, m) != 0) {
+      if (is64)
+        return launch_wave_private_vec_hist<T, int64_t>(st, (const int64_t *)is, (const T *)vss,
+                                                        n_updates, (T *)dest, H0, m);
+      return launch_wave_private_vec_hist<T, int32_t>(st, (const int32_t *)is, (const T *)vss,
+                                                      n_updates, (T *)dest, H0, m);
+    }
+  }
   if (js == nullptr && m > 1 && H <= lds_limit) {  // one index per vector: no flat indices needed
     if (is64)
       return launch_lds_hist<T, Op, int64_t, HIST_VECTOR>(st, (const int64_t *)is, (const T *)vss,

@@ -265,6 +265,65 @@ def test_hist_with_vector_operator_goldens_and_shapes(ctx, goldens):
         h.free()
 
 
+def test_float_sums_into_vector_bins(ctx):
+    """reduce_by_index dest (map2 (+)) (replicate m 0) is vss with float elements: bins that a
+    wave can keep for itself (16-byte pieces of a row per lane, so m a multiple of 4 f32 or 2 f64)
+    and the shapes next to them that take the other kernels; indices out of range, every row on
+    one bin, rows longer than a wave's step, enough rows for the unrolled loop and its ragged end,
+    i32 indices through the kernel library.  Values are small whole numbers: sums are exact in any
+    order, so the comparison with the oracle is bit for bit."""
+    import ctypes as C
+    from futhark_amd import lib_path
+    rng = np.random.default_rng(41)
+    cases = [("f32", 256, 16, 700001, "uniform"), ("f32", 256, 16, 5000, "one"),
+             ("f32", 7, 4, 1, "uniform"), ("f32", 1, 4, 100000, "uniform"),
+             ("f32", 3, 1024, 2001, "uniform"), ("f32", 630, 16, 30011, "skewed"),
+             ("f32", 631, 16, 30011, "uniform"),          # one bin too many for a wave: LDS kernel
+             ("f32", 100, 6, 30011, "uniform"),           # rows are not whole 16-byte pieces
+             ("f64", 256, 8, 300007, "uniform"), ("f64", 50, 2, 99999, "skewed"),
+             ("f64", 9, 3, 5000, "uniform")]
+    for t, H, m, n, how in cases:
+        dt = {"f32": np.float32, "f64": np.float64}[t]
+        if how == "one":
+            is_ = np.full(n, H // 2, np.int64)
+        elif how == "skewed":
+            is_ = np.minimum(rng.geometric(0.3, n) - 1, H + 2).astype(np.int64)
+        else:
+            is_ = rng.integers(-3, H + 3, n).astype(np.int64)
+        vss = rng.integers(-8, 9, (n, m)).astype(dt)
+        dest = rng.integers(-5, 5, (H, m)).astype(dt)
+        d, i, v = ctx.new(f"{t}_2d", dest), ctx.new("i64_1d", is_), ctx.new(f"{t}_2d", vss)
+        print(f"rbi_vec_add_{t} H={H} m={m} n={n} {how}", flush=True)
+        out = ctx.call(f"rbi_vec_add_{t}", [f"{t}_2d"], d, i, v)
+        want = oracle.rbi_vec("add", t, dest, is_, vss)
+        assert np.array_equal(out.values(), want), (t, H, m, n, how)
+        for h in (out, d, i, v):
+            h.free()
+    # i32 indices: the kernel library directly
+    k = C.CDLL(str(lib_path("libfuthark_amd_kernels.so")))
+    k.fa_seghist_shaped.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int,
+                                    C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_int64,
+                                    C.c_int64, C.c_void_p, C.c_size_t]
+    k.fa_seghist_shaped_scratch_bytes.restype = C.c_size_t
+    k.fa_seghist_shaped_scratch_bytes.argtypes = [C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64,
+                                                  C.c_int64]
+    FA_F32, FA_ADD = 2, 0
+    H, m, n = 100, 8, 123457
+    is32 = rng.integers(-3, H + 3, n).astype(np.int32)
+    vss = rng.integers(-8, 9, (n, m)).astype(np.float32)
+    dest0 = rng.integers(-5, 5, (H, m)).astype(np.float32)
+    d_is, d_vs, dest = ctx.new("i32_1d", is32), ctx.new("f32_2d", vss), ctx.new("f32_2d", dest0)
+    sb = k.fa_seghist_shaped_scratch_bytes(FA_F32, 0, n, H, 1, m)
+    scratch = ctx.new("u8_1d", np.zeros(max(sb, 256), np.uint8))
+    print("fa_seghist_shaped f32 with i32 indices", flush=True)
+    rc = k.fa_seghist_shaped(ctx.stream, FA_F32, FA_ADD, d_is.device_ptr, None, 0, d_vs.device_ptr,
+                             n, dest.device_ptr, H, 1, m, scratch.device_ptr, sb)
+    assert rc == 0
+    assert np.array_equal(dest.values(), oracle.rbi_vec("add", "f32", dest0, is32.astype(np.int64), vss))
+    for h in (d_is, d_vs, dest, scratch):
+        h.free()
+
+
 def test_hist_with_2d_indices_goldens_and_shapes(ctx, goldens):
     """reduce_by_index_2d: tests/hist/hist2d.fut (an update is dropped when either coordinate is
     outside), then random cases of both sizes of bin space."""
