@@ -419,14 +419,14 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
 // using copy l mod 2^copies_log2, so that fewer lanes share a cell and fewer
 // of them need the atomic.
 template <class T, class I, int INDEX_BITS /* 0: as many as `index_bits` says, not unrolled */,
-          bool TAGS = false>
-__global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
+          bool TAGS = false, int BLOCK = HIST_BLOCK>
+__global__ __launch_bounds__(BLOCK) void seghist_wave_private_kernel(
     const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t H,
     int index_bits, int copies_log2) {
   extern __shared__ __align__(16) unsigned char s_raw[];
   T *sh = reinterpret_cast<T *>(s_raw);
   constexpr int VEC = 4;
-  constexpr int WAVES = HIST_BLOCK / WAVE;
+  constexpr int WAVES = BLOCK / WAVE;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / WAVE));
   const int nb = (int)H;
   const int copies = 1 << copies_log2;
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
   // TAGS: one byte per cell behind the histograms of the block, see update_tagged
   volatile uint8_t *tags = reinterpret_cast<uint8_t *>(sh + ((size_t)WAVES * nb << copies_log2)) +
                            ((size_t)wave * nb << copies_log2);
-  for (int i = threadIdx.x; i < nb * WAVES * copies; i += HIST_BLOCK) sh[i] = T(0);
+  for (int i = threadIdx.x; i < nb * WAVES * copies; i += BLOCK) sh[i] = T(0);
   __syncthreads();
   const uint32_t my_copy = (uint32_t)lane_id() & (uint32_t)(copies - 1);
   // the lanes of my copy: every copies-th bit, starting at my_copy
@@ -510,8 +510,8 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
   };
 
   const int64_t nvec = n / VEC;
-  const int64_t stride = (int64_t)gridDim.x * HIST_BLOCK;
-  for (int64_t i = (int64_t)blockIdx.x * HIST_BLOCK + threadIdx.x; i < nvec + (HIST_BLOCK - 1);
+  const int64_t stride = (int64_t)gridDim.x * BLOCK;
+  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < nvec + (BLOCK - 1);
        i += stride) {
     // whole waves take part in every step, also the one with the ragged end
     const int64_t first_of_wave = i - lane_id();
@@ -554,7 +554,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
     else update(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
   }
   __syncthreads();
-  for (int r = threadIdx.x; r < nb; r += HIST_BLOCK) {
+  for (int r = threadIdx.x; r < nb; r += BLOCK) {
     T acc = T(0);
     for (int w = 0; w < WAVES; w++)
       for (int c = 0; c < copies; c++) acc += sh[(((size_t)w * nb + r) << copies_log2) + c];
@@ -710,16 +710,16 @@ constexpr int HIST_WAVE_PRIVATE_BYTES = HIST_LDS_BYTES / (HIST_BLOCK / WAVE);
 constexpr int HIST_WAVE_COPIES_MAX = 4;
 
 
-template <class T, class I, int BITS, bool TAGS>
+template <class T, class I, int BITS, bool TAGS, int BLOCK = HIST_BLOCK>
 static int launch_wave_private_kernel(hipStream_t st, dim3 grid, size_t lds, const I *is,
                                       const T *vs, int64_t n, T *dest, int64_t H, int index_bits,
                                       int copies_log2) {
-  auto kernel = seghist_wave_private_kernel<T, I, BITS, TAGS>;
+  auto kernel = seghist_wave_private_kernel<T, I, BITS, TAGS, BLOCK>;
   // Initialised once, under the lock C++ gives function-local statics.
   static const hipError_t raised = hipFuncSetAttribute(
       (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
   if (raised != hipSuccess) return (int)raised;
-  hipLaunchKernelGGL(kernel, grid, dim3(HIST_BLOCK), lds, st, is, vs, n, dest, H, index_bits,
+  hipLaunchKernelGGL(kernel, grid, dim3(BLOCK), lds, st, is, vs, n, dest, H, index_bits,
                      copies_log2);
   return launch_status();
 }
@@ -735,18 +735,32 @@ static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, in
   static_assert(HIST_WAVE_PRIVATE_BYTES / 4 <= (1 << 11), "eleven index bits cover every bin");
   int index_bits = 1;
   while (((int64_t)1 << index_bits) < H) index_bits++;
-  // as many copies per wave (at most HIST_WAVE_COPIES_MAX) as leave room for two blocks on a CU
-  // a byte of tag per cell where one block with them fits, else the ballots
+  // 4-byte sums: a byte of tag per cell where one block with them fits (8-byte
+  // sums were no faster with tags: H = 256 f64, 292 against 282 us)
   const bool tags = HIST_TAG_MATCH && sizeof(T) == 4 &&
                     (size_t)H * (sizeof(T) + 1) * (HIST_BLOCK / WAVE) <= HIST_LDS_BYTES;
   const size_t one = (size_t)H * (sizeof(T) + (tags ? 1 : 0)) * (HIST_BLOCK / WAVE);
+  // two blocks with tags may take the 160 KiB of a CU to the byte
   const size_t margin = tags ? HIST_TAG_MARGIN : 4096;
+  // as many copies per wave (at most HIST_WAVE_COPIES_MAX) as leave room for two blocks on a CU
   int copies_log2 = 0;
   while ((1 << copies_log2) < HIST_WAVE_COPIES_MAX && (one << (copies_log2 + 1)) * 2 + margin <= 160 * 1024)
     copies_log2++;
   const size_t lds = one << copies_log2;
   const int per_cu = lds * 2 + margin <= 160 * 1024 ? 2 : 1;
   const dim3 grid(hist_num_cus() * per_cu);
+  if constexpr (sizeof(T) == 4 && HIST_TAG_MATCH) {
+    // More 4-byte bins than let two blocks of 16 histograms with tags share
+    // a CU: blocks of eight waves, as many as fit (1024 < H <= 2048: 3 or 2,
+    // that is 24 or 16 waves on the CU).
+    if (per_cu == 1) {
+      constexpr int HALF = HIST_BLOCK / 2;
+      const size_t lds_half = (size_t)H * (sizeof(T) + 1) * (HALF / WAVE);
+      const int blocks = std::min(4, (int)((size_t)160 * 1024 / lds_half));
+      return launch_wave_private_kernel<T, I, 11, true, HALF>(
+          st, dim3(hist_num_cus() * blocks), lds_half, is, vs, n, dest, H, index_bits, 0);
+    }
+  }
   if (tags && H > 256)
     return launch_wave_private_kernel<T, I, 11, true>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
   if (tags)

@@ -44,6 +44,34 @@ def test_hist_small_and_ragged(ctx, t, op):
             h.free()
 
 
+@pytest.mark.parametrize("t", ["f32", "f64"])
+def test_float_sums_every_size_class_exactly(ctx, t):
+    """Sums of floats into up to 2048 (f64: 1024) bins keep a histogram per wave; which lane of a
+    cell goes first is settled by tags or by ballots, in blocks of 16 or 8 waves, depending on the
+    number of bins and on how many lanes meet (a wave changes over when indices are skewed).  Bin
+    counts on both sides of every limit, uniform and skewed indices, one bin for everything; the
+    values are small whole numbers, so the sums are exact in any order and must match bit for bit."""
+    dt = {"f32": np.float32, "f64": np.float64}[t]
+    rng = np.random.default_rng(77)
+    n = 600011
+    for H in (1, 2, 255, 256, 257, 1024, 1025, 1200, 1638, 1639, 2047, 2048, 2049):
+        for how in ("uniform", "skewed", "one"):
+            if how == "uniform":
+                is_ = rng.integers(-2, H + 2, n).astype(np.int32)
+            elif how == "skewed":     # runs of skew between runs without: waves change over and back
+                is_ = rng.integers(0, H, n).astype(np.int32)
+                hot = (np.arange(n) // 50000) % 2 == 1
+                is_[hot] = np.minimum(rng.geometric(0.4, int(hot.sum())) - 1, H - 1).astype(np.int32)
+            else:
+                is_ = np.full(n, H - 1, np.int32)
+            vs = rng.integers(-8, 9, n).astype(dt)
+            i, v = ctx.new("i32_1d", is_), ctx.new(f"{t}_1d", vs)
+            out = ctx.call(f"hist_add_{t}", [f"{t}_1d"], H, i, v)
+            assert np.array_equal(out.values(), oracle.hist("add", t, H, is_, vs)), (t, H, how)
+            for h in (i, v, out):
+                h.free()
+
+
 def test_reference_goldens(ctx, goldens):
     for c in goldens["hist_simple"]["cases"]:
         img = np.array(c["image"], np.int32)
