@@ -23,24 +23,32 @@
 // stable ranked scatter, radix.hip.h), then runs LDS histograms over the
 // partitions; out-of-range indices land in a partition that is never read.
 // Only H beyond 255 ranges falls back to one device atomic per element.
+//
+// Sums of floats are the exception: the LDS float atomic runs at a quarter of
+// the integer rate, so up to 2048 f32 (1024 f64) bins, or [H0][m] bins of
+// float vectors up to 40 KiB, are kept once per wave and updated with ordinary
+// LDS reads and writes (seghist_wave_private_kernel and
+// seghist_wave_private_vec_kernel below).
 #include "radix.hip.h"
 
 namespace fa {
 
+// Choices of the float-sum kernels, overridable at compile time to measure the
+// alternative (the figures stand where each is used):
 #ifndef HIST_TAG_MATCH
-#define HIST_TAG_MATCH 1
+#define HIST_TAG_MATCH 1  // 4-byte sums: a tag per cell picks the first lane (0: ballots only)
 #endif
 #ifndef HIST_TAG_MARGIN
-#define HIST_TAG_MARGIN 0
-#endif
-#ifndef HIST_VEC_UNROLL
-#define HIST_VEC_UNROLL 8
+#define HIST_TAG_MARGIN 0  // bytes of a CU's 160 KiB of LDS left unused by two blocks with tags
 #endif
 #ifndef HIST_CONTENDED
-#define HIST_CONTENDED 32
+#define HIST_CONTENDED 32  // followers among a wave's 256 updates beyond which it takes the ballots
 #endif
 #ifndef HIST_ASM_MATCH
-#define HIST_ASM_MATCH 1
+#define HIST_ASM_MATCH 1  // low eight index bits matched by rs_match1 (0: as the compiler writes it)
+#endif
+#ifndef HIST_VEC_UNROLL
+#define HIST_VEC_UNROLL 8  // 16-byte loads a lane of the vector-bin kernel keeps in flight
 #endif
 constexpr int HIST_BLOCK = 1024;
 constexpr int HIST_LDS_BYTES = 128 * 1024;  // bin storage per block
