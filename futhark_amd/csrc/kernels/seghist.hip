@@ -24,28 +24,35 @@
 // partitions; out-of-range indices land in a partition that is never read.
 // Only H beyond 255 ranges falls back to one device atomic per element.
 //
-// Sums of floats are the exception: the LDS float atomic runs at a quarter of
-// the integer rate, so up to 2048 f32 (1024 f64) bins, or [H0][m] bins of
-// float vectors up to 40 KiB, are kept once per wave and updated with ordinary
-// LDS reads and writes (seghist_wave_private_kernel and
-// seghist_wave_private_vec_kernel below).
+// Sums of floats are the exception: the LDS float atomic runs at a third to a
+// quarter of the integer rate.  f32 sums read the cell, add in a register and
+// put the sum back with an integer compare-and-swap (lds_update); up to 1024
+// f64 bins, and [H0][m] bins of float vectors up to 40 KiB, are kept once per
+// wave and updated with ordinary LDS reads and writes
+// (seghist_wave_private_kernel, seghist_wave_private_vec_kernel).
 #include "radix.hip.h"
 
 namespace fa {
 
-// Choices of the float-sum kernels, overridable at compile time to measure the
+// Choices of the float-sum paths, overridable at compile time to measure the
 // alternative (the figures stand where each is used):
-#ifndef HIST_TAG_MATCH
-#define HIST_TAG_MATCH 1  // 4-byte sums: a tag per cell picks the first lane (0: ballots only)
+#ifndef HIST_CAS_FEW
+#define HIST_CAS_FEW 1  // compare-and-swap attempts of an f32 sum before the float atomic ...
 #endif
-#ifndef HIST_TAG_MARGIN
-#define HIST_TAG_MARGIN 0  // bytes of a CU's 160 KiB of LDS left unused by two blocks with tags
+#ifndef HIST_CAS_MANY
+#define HIST_CAS_MANY 4  // ... and where a bin has at least 2^HIST_CAS_MANY_COPIES_LOG2 copies
 #endif
-#ifndef HIST_CONTENDED
-#define HIST_CONTENDED 32  // followers among a wave's 256 updates beyond which it takes the ballots
+#ifndef HIST_CAS_MANY_COPIES_LOG2
+#define HIST_CAS_MANY_COPIES_LOG2 2
+#endif
+#ifndef HIST_COPY_BYTES
+#define HIST_COPY_BYTES (32 * 1024)  // a bin range is replicated while its copies fit in this
 #endif
 #ifndef HIST_ASM_MATCH
 #define HIST_ASM_MATCH 1  // low eight index bits matched by rs_match1 (0: as the compiler writes it)
+#endif
+#ifndef HIST_VEC_KERNEL
+#define HIST_VEC_KERNEL 1  // float vector bins: a histogram per wave (0: the LDS kernel)
 #endif
 #ifndef HIST_VEC_UNROLL
 #define HIST_VEC_UNROLL 8  // 16-byte loads a lane of the vector-bin kernel keeps in flight
@@ -152,10 +159,29 @@ template <class T, int Scope> struct AtomicUpdate<T, OpMin<T>, Scope> {
 // elements of a bin almost no update changes it (LDS atomics run at about a
 // quarter of the rate of LDS reads).  NaN values never change a bin (fmax/fmin
 // ignore them), and bins start from the identity, so they never hold NaN.
-template <class T, class Op>
+template <class T, class Op, int CAS = 0>
 __device__ __forceinline__ void lds_update(T *p, T v) {
   constexpr bool minmax = std::is_same<Op, OpMax<T>>::value || std::is_same<Op, OpMin<T>>::value;
-  if constexpr (!minmax) {
+  if constexpr (CAS > 0) {
+    // Sums of f32: the cell is read, the sum formed in a register and put back
+    // with an integer compare-and-swap, which LDS runs at the rate of its
+    // integer atomics; the float atomic, at a third of that rate, takes what
+    // is left after CAS attempts (lanes of one wave on one cell: one of them
+    // succeeds per attempt).
+    static_assert(std::is_same<T, float>::value && std::is_same<Op, OpAdd<T>>::value, "f32 sums");
+    uint32_t *q = reinterpret_cast<uint32_t *>(p);
+    uint32_t seen = *reinterpret_cast<volatile uint32_t *>(q);
+    bool done = false;
+#pragma unroll
+    for (int attempt = 0; attempt < CAS; attempt++) {
+      if (!done) {
+        const uint32_t want = bit_cast<uint32_t>(bit_cast<float>(seen) + v);
+        done = __hip_atomic_compare_exchange_strong(q, &seen, want, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
+    }
+    if (!done) AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(p, v);
+  } else if constexpr (!minmax) {
     AtomicUpdate<T, Op, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(p, v);
   } else {
     const T cur = *reinterpret_cast<volatile T *>(p);
@@ -282,7 +308,7 @@ template <class E> __device__ __forceinline__ void load_elems4(E (&dst)[4], cons
 // is[p] * seg_len + js[p] when is[p] lies in [0, H_seg) and js[p] in [0, seg_len).
 enum { HIST_PLAIN = 0, HIST_ROWS = 1, HIST_VECTOR = 2, HIST_PAIRS = 3 };
 
-template <class T, class Op, class I, int MODE>
+template <class T, class Op, class I, int MODE, int CAS = 0>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
     const I *__restrict__ is, const I *__restrict__ js, const T *__restrict__ vs, int64_t n, T *dest,
     int64_t bin_base, int64_t H, int range_bins, int P, int log2_copies, int64_t seg_len,
@@ -314,7 +340,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
   auto update = [&](int64_t bin, T v) {
     const int64_t r = bin - lo;
     if ((uint64_t)r < (uint64_t)nb)
-      lds_update<A, OpA>(&sh[((int)r << log2_copies) + copy], (A)v);
+      lds_update<A, OpA, CAS>(&sh[((int)r << log2_copies) + copy], (A)v);
   };
   // (row, column) of every element is tracked
   constexpr bool SEGMENTED = MODE == HIST_ROWS || MODE == HIST_VECTOR;
@@ -411,10 +437,14 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
   }
 }
 
-// ------------------------------------------- float sums into few bins
+// ------------------------------------------- f64 sums into few bins
 // LDS atomics on floats run at about a quarter of the integer rate on MI355X
-// (2^27 updates: 670 us), so sums of f32 / f64 into few bins take another
-// route: every wave keeps a histogram of its own in LDS and updates it with
+// (2^27 updates: 670 us), and for 8-byte sums compare-and-swap is no faster
+// (H = 2048 f64: 260 against 247 us), so sums of f64 into few bins take another
+// route (the kernel also takes f32, which is how it was measured against
+// compare-and-swap: H = 256 uniform / Zipf 211 / 243 us against 170 / 174 us,
+// H = 2048 310 / 346 against 166 / 405 us): every wave keeps a histogram of its
+// own in LDS and updates it with
 // ordinary reads and writes.  Lanes of a wave that hit the same bin in the same
 // step find each other with one ballot per index bit (as the radix scatter
 // does): the first lane of a group adds its value with an ordinary read and
@@ -426,32 +456,26 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
 // A wave keeps 2^copies_log2 copies of its histogram where LDS allows, lane l
 // using copy l mod 2^copies_log2, so that fewer lanes share a cell and fewer
 // of them need the atomic.
-template <class T, class I, int INDEX_BITS /* 0: as many as `index_bits` says, not unrolled */,
-          bool TAGS = false, int BLOCK = HIST_BLOCK>
-__global__ __launch_bounds__(BLOCK) void seghist_wave_private_kernel(
+template <class T, class I, int INDEX_BITS /* 0: as many as `index_bits` says, not unrolled */>
+__global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
     const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t H,
     int index_bits, int copies_log2) {
   extern __shared__ __align__(16) unsigned char s_raw[];
   T *sh = reinterpret_cast<T *>(s_raw);
   constexpr int VEC = 4;
-  constexpr int WAVES = BLOCK / WAVE;
+  constexpr int WAVES = HIST_BLOCK / WAVE;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / WAVE));
   const int nb = (int)H;
   const int copies = 1 << copies_log2;
   // volatile: the compiler must not carry a bin across the rounds below in a register
   volatile T *mine = sh + ((size_t)wave * nb << copies_log2);
-  // TAGS: one byte per cell behind the histograms of the block, see update_tagged
-  volatile uint8_t *tags = reinterpret_cast<uint8_t *>(sh + ((size_t)WAVES * nb << copies_log2)) +
-                           ((size_t)wave * nb << copies_log2);
-  for (int i = threadIdx.x; i < nb * WAVES * copies; i += BLOCK) sh[i] = T(0);
+  for (int i = threadIdx.x; i < nb * WAVES * copies; i += HIST_BLOCK) sh[i] = T(0);
   __syncthreads();
   const uint32_t my_copy = (uint32_t)lane_id() & (uint32_t)(copies - 1);
   // the lanes of my copy: every copies-th bit, starting at my_copy
   uint32_t copy_mask = 0u;
   for (int l = (int)my_copy; l < 32; l += copies) copy_mask |= 1u << l;
 
-  // lanes of this wave that had to follow another lane in the current step
-  int followers = 0;
   auto update = [&](int64_t bin, T v) {
     const bool valid = (uint64_t)bin < (uint64_t)H;
     const uint32_t b = valid ? (uint32_t)bin : 0u;
@@ -495,31 +519,11 @@ __global__ __launch_bounds__(BLOCK) void seghist_wave_private_kernel(
     if (turn > 0)
       AtomicUpdate<T, OpAdd<T>, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(const_cast<T *>(&mine[slot]), v);
     __builtin_amdgcn_wave_barrier();
-    if constexpr (TAGS) followers += __builtin_popcountll(__ballot(turn > 0));
-  };
-
-  // TAGS: which of the lanes that hit a cell in the same step goes first is
-  // settled by the cell's tag instead of ballots: every lane writes its number
-  // into the tag and reads it back; the one whose number stayed adds with an
-  // ordinary read and write, the others follow with the atomic.  Two LDS
-  // operations in place of some forty instructions of matching.
-  auto update_tagged = [&](int64_t bin, T v) {
-    const bool valid = (uint64_t)bin < (uint64_t)H;
-    const uint32_t slot = ((valid ? (uint32_t)bin : 0u) << copies_log2) + my_copy;
-    if (valid) tags[slot] = (uint8_t)lane_id();
-    __builtin_amdgcn_wave_barrier();
-    const bool first = valid && tags[slot] == (uint8_t)lane_id();
-    if (first) mine[slot] = mine[slot] + v;
-    __builtin_amdgcn_wave_barrier();
-    if (valid && !first)
-      AtomicUpdate<T, OpAdd<T>, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(const_cast<T *>(&mine[slot]), v);
-    __builtin_amdgcn_wave_barrier();
-    followers += __builtin_popcountll(__ballot(valid && !first));
   };
 
   const int64_t nvec = n / VEC;
-  const int64_t stride = (int64_t)gridDim.x * BLOCK;
-  for (int64_t i = (int64_t)blockIdx.x * BLOCK + threadIdx.x; i < nvec + (BLOCK - 1);
+  const int64_t stride = (int64_t)gridDim.x * HIST_BLOCK;
+  for (int64_t i = (int64_t)blockIdx.x * HIST_BLOCK + threadIdx.x; i < nvec + (HIST_BLOCK - 1);
        i += stride) {
     // whole waves take part in every step, also the one with the ragged end
     const int64_t first_of_wave = i - lane_id();
@@ -536,33 +540,16 @@ __global__ __launch_bounds__(BLOCK) void seghist_wave_private_kernel(
         bv[e] = T(0);
       }
     }
-    if constexpr (TAGS) {
-      // Many lanes on few cells (skewed indices): the tags of a step cost a
-      // write conflict per lane of a cell, the ballots do not, so a wave
-      // whose last step had more than HIST_CONTENDED followers among its
-      // VEC * 64 updates takes the ballots for the next one.
-      const bool contended = followers > HIST_CONTENDED;
-      followers = 0;
-      if (contended) {
 #pragma unroll
-        for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
-      } else {
-#pragma unroll
-        for (int e = 0; e < VEC; e++) update_tagged((int64_t)bi[e], bv[e]);
-      }
-    } else {
-#pragma unroll
-      for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
-    }
+    for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
   }
   if (blockIdx.x == 0 && wave == 0) {  // the n % VEC elements at the end
     const int64_t t = nvec * VEC + lane_id();
     const bool in = lane_id() < VEC && t < n;
-    if constexpr (TAGS) update_tagged(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
-    else update(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
+    update(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
   }
   __syncthreads();
-  for (int r = threadIdx.x; r < nb; r += BLOCK) {
+  for (int r = threadIdx.x; r < nb; r += HIST_BLOCK) {
     T acc = T(0);
     for (int w = 0; w < WAVES; w++)
       for (int c = 0; c < copies; c++) acc += sh[(((size_t)w * nb + r) << copies_log2) + c];
@@ -610,7 +597,9 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
     const int nb = (int)((H - bin0) < range_bins ? (H - bin0) : range_bins);
     for (int i = threadIdx.x; i < nb; i += HIST_BLOCK) sh[i] = OpA::identity();
     __syncthreads();
-    auto update = [&](U b, T v) { lds_update<A, OpA>(&sh[(int)((int64_t)b - bin0)], (A)v); };
+    // f32 sums: one compare-and-swap attempt before the float atomic (no copies here)
+    constexpr int CAS = std::is_same<A, float>::value && std::is_same<OpA, OpAdd<A>>::value ? HIST_CAS_FEW : 0;
+    auto update = [&](U b, T v) { lds_update<A, OpA, CAS>(&sh[(int)((int64_t)b - bin0)], (A)v); };
     // [lo, hi) = loose elements up to a multiple of four, groups of four read
     // with 16-byte non-temporal loads (two groups of a thread in flight),
     // loose elements at the end.
@@ -684,25 +673,11 @@ static int hist_num_cus() {
   return cus;
 }
 
-// Launches the LDS kernel over bins [0,H) of `dest` (H <= max ranges * range size).
-template <class T, class Op, class I, int MODE = HIST_PLAIN>
-static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
-                           int64_t H, int64_t seg_len = 0, int64_t H_seg = 0,
-                           const I *js = nullptr) {
-  using A = typename HistAcc<T>::A;
-  const int max_range = hist_range_bins_max(sizeof(A));
-  const int P = (int)ceil_div(H, max_range);
-  const int range_bins = (int)ceil_div(H, P);
-  int log2_copies = 0;
-  while (log2_copies < 5 && (int64_t)range_bins * (2 << log2_copies) * (int64_t)sizeof(A) <= 32 * 1024)
-    log2_copies++;
-  const size_t lds = (size_t)range_bins * sizeof(A) << log2_copies;
-  // One block per CU when the range fills LDS, two when two fit.
-  const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
-  int grid = hist_num_cus() * per_cu;
-  grid -= grid % (NUM_XCDS * P);
-  if (grid < NUM_XCDS * P) grid = NUM_XCDS * P;
-  auto kernel = seghist_lds_kernel<T, Op, I, MODE>;
+template <class T, class Op, class I, int MODE, int CAS>
+static int launch_lds_kernel(hipStream_t st, int grid, size_t lds, const I *is, const I *js,
+                             const T *vs, int64_t n, T *dest, int64_t H, int range_bins, int P,
+                             int log2_copies, int64_t seg_len, int64_t H_seg) {
+  auto kernel = seghist_lds_kernel<T, Op, I, MODE, CAS>;
   // Initialised once, under the lock C++ gives function-local statics.
   static const hipError_t raised = hipFuncSetAttribute(
       (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
@@ -712,25 +687,49 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
   return launch_status();
 }
 
+// Launches the LDS kernel over bins [0,H) of `dest` (H <= max ranges * range size).
+template <class T, class Op, class I, int MODE = HIST_PLAIN>
+static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
+                           int64_t H, int64_t seg_len = 0, int64_t H_seg = 0,
+                           const I *js = nullptr) {
+  using A = typename HistAcc<T>::A;
+  const int max_range = hist_range_bins_max(sizeof(A));
+  const int P = (int)ceil_div(H, max_range);
+  const int range_bins = (int)ceil_div(H, P);
+  // A small range is replicated while its copies fit in 32 KiB; f32 sums, where
+  // every lane that meets another on a cell costs a failed compare-and-swap,
+  // take 64 KiB, the most that leaves two blocks on a CU (Zipf indices,
+  // H = 1024 / 2048 / 4096: 314 / 407 / 471 -> 218 / 301 / 390 us; integer sums
+  // gain nothing from it).
+  constexpr bool f32_sum = std::is_same<A, float>::value && std::is_same<Op, OpAdd<T>>::value;
+  const int64_t copy_bytes = f32_sum ? 2 * HIST_COPY_BYTES : HIST_COPY_BYTES;
+  int log2_copies = 0;
+  while (log2_copies < 5 && (int64_t)range_bins * (2 << log2_copies) * (int64_t)sizeof(A) <= copy_bytes)
+    log2_copies++;
+  const size_t lds = (size_t)range_bins * sizeof(A) << log2_copies;
+  // One block per CU when the range fills LDS, two when two fit.
+  const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
+  int grid = hist_num_cus() * per_cu;
+  grid -= grid % (NUM_XCDS * P);
+  if (grid < NUM_XCDS * P) grid = NUM_XCDS * P;
+  if constexpr (f32_sum) {
+    // f32 sums go through compare-and-swap: several attempts where a bin has
+    // many copies (lanes that meet on a cell are few), one where it has not
+    if (log2_copies >= HIST_CAS_MANY_COPIES_LOG2)
+      return launch_lds_kernel<T, Op, I, MODE, HIST_CAS_MANY>(st, grid, lds, is, js, vs, n, dest, H,
+                                                             range_bins, P, log2_copies, seg_len, H_seg);
+    return launch_lds_kernel<T, Op, I, MODE, HIST_CAS_FEW>(st, grid, lds, is, js, vs, n, dest, H,
+                                                          range_bins, P, log2_copies, seg_len, H_seg);
+  }
+  return launch_lds_kernel<T, Op, I, MODE, 0>(st, grid, lds, is, js, vs, n, dest, H, range_bins, P,
+                                              log2_copies, seg_len, H_seg);
+}
+
 // Sums of floats into at most this many bytes of bins per wave go through
 // seghist_wave_private_kernel.
 constexpr int HIST_WAVE_PRIVATE_BYTES = HIST_LDS_BYTES / (HIST_BLOCK / WAVE);
 constexpr int HIST_WAVE_COPIES_MAX = 4;
 
-
-template <class T, class I, int BITS, bool TAGS, int BLOCK = HIST_BLOCK>
-static int launch_wave_private_kernel(hipStream_t st, dim3 grid, size_t lds, const I *is,
-                                      const T *vs, int64_t n, T *dest, int64_t H, int index_bits,
-                                      int copies_log2) {
-  auto kernel = seghist_wave_private_kernel<T, I, BITS, TAGS, BLOCK>;
-  // Initialised once, under the lock C++ gives function-local statics.
-  static const hipError_t raised = hipFuncSetAttribute(
-      (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
-  if (raised != hipSuccess) return (int)raised;
-  hipLaunchKernelGGL(kernel, grid, dim3(BLOCK), lds, st, is, vs, n, dest, H, index_bits,
-                     copies_log2);
-  return launch_status();
-}
 
 template <class T, class I>
 static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
@@ -743,39 +742,30 @@ static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, in
   static_assert(HIST_WAVE_PRIVATE_BYTES / 4 <= (1 << 11), "eleven index bits cover every bin");
   int index_bits = 1;
   while (((int64_t)1 << index_bits) < H) index_bits++;
-  // 4-byte sums: a byte of tag per cell where one block with them fits (8-byte
-  // sums were no faster with tags: H = 256 f64, 292 against 282 us)
-  const bool tags = HIST_TAG_MATCH && sizeof(T) == 4 &&
-                    (size_t)H * (sizeof(T) + 1) * (HIST_BLOCK / WAVE) <= HIST_LDS_BYTES;
-  const size_t one = (size_t)H * (sizeof(T) + (tags ? 1 : 0)) * (HIST_BLOCK / WAVE);
-  // two blocks with tags may take the 160 KiB of a CU to the byte
-  const size_t margin = tags ? HIST_TAG_MARGIN : 4096;
   // as many copies per wave (at most HIST_WAVE_COPIES_MAX) as leave room for two blocks on a CU
+  const size_t one = (size_t)H * sizeof(T) * (HIST_BLOCK / WAVE);
   int copies_log2 = 0;
-  while ((1 << copies_log2) < HIST_WAVE_COPIES_MAX && (one << (copies_log2 + 1)) * 2 + margin <= 160 * 1024)
+  while ((1 << copies_log2) < HIST_WAVE_COPIES_MAX && (one << (copies_log2 + 1)) * 2 + 4096 <= 160 * 1024)
     copies_log2++;
   const size_t lds = one << copies_log2;
-  const int per_cu = lds * 2 + margin <= 160 * 1024 ? 2 : 1;
+  const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
   const dim3 grid(hist_num_cus() * per_cu);
-  if constexpr (sizeof(T) == 4 && HIST_TAG_MATCH) {
-    // More 4-byte bins than let two blocks of 16 histograms with tags share
-    // a CU: blocks of eight waves, as many as fit (1024 < H <= 2048: 3 or 2,
-    // that is 24 or 16 waves on the CU).
-    if (per_cu == 1) {
-      constexpr int HALF = HIST_BLOCK / 2;
-      const size_t lds_half = (size_t)H * (sizeof(T) + 1) * (HALF / WAVE);
-      const int blocks = std::min(4, (int)((size_t)160 * 1024 / lds_half));
-      return launch_wave_private_kernel<T, I, 11, true, HALF>(
-          st, dim3(hist_num_cus() * blocks), lds_half, is, vs, n, dest, H, index_bits, 0);
-    }
-  }
-  if (tags && H > 256)
-    return launch_wave_private_kernel<T, I, 11, true>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
-  if (tags)
-    return launch_wave_private_kernel<T, I, 8, true>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
+#define FA_WAVE_PRIVATE(BITS)                                                                  \
+  do {                                                                                         \
+    auto kernel = seghist_wave_private_kernel<T, I, BITS>;                                     \
+    /* Initialised once, under the lock C++ gives function-local statics. */                   \
+    static const hipError_t raised = hipFuncSetAttribute(                                      \
+        (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);     \
+    if (raised != hipSuccess) return (int)raised;                                              \
+    hipLaunchKernelGGL(kernel, grid, dim3(HIST_BLOCK), lds, st, is, vs, n, dest, H, index_bits, \
+                       copies_log2);                                                           \
+  } while (0)
   if (H > 256)
-    return launch_wave_private_kernel<T, I, 11, false>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
-  return launch_wave_private_kernel<T, I, 8, false>(st, grid, lds, is, vs, n, dest, H, index_bits, copies_log2);
+    FA_WAVE_PRIVATE(11);
+  else
+    FA_WAVE_PRIVATE(8);
+#undef FA_WAVE_PRIVATE
+  return launch_status();
 }
 
 // ------------------------------- float sums into few bins that are vectors
@@ -962,7 +952,8 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
   const int64_t lds_limit =
       (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
   if constexpr (std::is_same<Op, OpAdd<T>>::value && std::is_floating_point<T>::value) {
-    if (H * (int64_t)sizeof(T) <= HIST_WAVE_PRIVATE_BYTES) {
+    // f64 only: f32 sums are faster through compare-and-swap in the LDS kernel
+    if (sizeof(T) == 8 && H * (int64_t)sizeof(T) <= HIST_WAVE_PRIVATE_BYTES) {
       if (is64)
         return launch_wave_private_hist<T, int64_t>(st, (const int64_t *)is, (const T *)vs, n,
                                                     (T *)dest, H);
@@ -1070,7 +1061,7 @@ static int launch_hist_shaped(hipStream_t st, const void *is, const void *js, in
       (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
   if constexpr (std::is_same<Op, OpAdd<T>>::value && std::is_floating_point<T>::value) {
     // sums of float vectors into few bins: a histogram per wave, no float atomic per element
-    if (js == nullptr && m > 1 && hist_vec_lds_bytes<T>(H0, m) != 0) {
+    if (HIST_VEC_KERNEL && js == nullptr && m > 1 && hist_vec_lds_bytes<T>(H0, m) != 0) {
       if (is64)
         return launch_wave_private_vec_hist<T, int64_t>(st, (const int64_t *)is, (const T *)vss,
                                                         n_updates, (T *)dest, H0, m);
