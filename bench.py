@@ -378,7 +378,8 @@ SUITE = [
     "segred_add_f32_2p26", "segscan_add_i64_2p26",
     "hist_add_i32_H256_uniform_2p27", "hist_add_i32_H65536_uniform_2p27",
     "hist_add_i32_H4194304_uniform_2p27", "hist_add_i32_H4194304_zipf_2p27",
-    "hist_add_f32_H256_uniform_2p27", "hist_add_f32_H256_zipf_2p27", "hist_max_f32_H65536_uniform_2p27",
+    "hist_add_f32_H256_uniform_2p27", "hist_add_f32_H256_zipf_2p27", "hist_add_f32_H65536_uniform_2p27",
+    "hist_max_f32_H65536_uniform_2p27",
     "sort_u32_2p26", "sort_u64i32_2p26",
     "bmm_f16_1x4096", "bmm_bf16_1x4096", "bmm_f32_1x4096", "bmm_f16_64x512", "bmm_f32_64x512",
     "mfma_peak_f16", "mfma_peak_bf16",
