@@ -954,9 +954,9 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
   if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
   const int64_t lds_limit =
       (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
-  if constexpr (std::is_same<Op, OpAdd<T>>::value && std::is_floating_point<T>::value) {
+  if constexpr (std::is_same<Op, OpAdd<T>>::value && std::is_same<T, double>::value) {
     // f64 only: f32 sums are faster through compare-and-swap in the LDS kernel
-    if (sizeof(T) == 8 && H * (int64_t)sizeof(T) <= HIST_WAVE_PRIVATE_BYTES) {
+    if (H * (int64_t)sizeof(T) <= HIST_WAVE_PRIVATE_BYTES) {
       if (is64)
         return launch_wave_private_hist<T, int64_t>(st, (const int64_t *)is, (const T *)vs, n,
                                                     (T *)dest, H);
