@@ -24,12 +24,12 @@
 // partitions; out-of-range indices land in a partition that is never read.
 // Only H beyond 255 ranges falls back to one device atomic per element.
 //
-// Sums of floats are the exception: the LDS float atomic runs at a third to a
+// Sums of floats are the exception: the LDS f32 atomic runs at a third to a
 // quarter of the integer rate.  f32 sums read the cell, add in a register and
-// put the sum back with an integer compare-and-swap (lds_update); up to 1024
-// f64 bins, and [H0][m] bins of float vectors up to 40 KiB, are kept once per
-// wave and updated with ordinary LDS reads and writes
-// (seghist_wave_private_kernel, seghist_wave_private_vec_kernel).
+// put the sum back with an integer compare-and-swap (lds_update); float sums
+// keep twice the copies of a small range; [H0][m] bins of float vectors
+// between 8 and 40 KiB are kept once per wave and updated with ordinary LDS
+// reads and writes (seghist_wave_private_vec_kernel).
 #include "radix.hip.h"
 
 namespace fa {
@@ -47,9 +47,6 @@ namespace fa {
 #endif
 #ifndef HIST_COPY_BYTES
 #define HIST_COPY_BYTES (32 * 1024)  // a bin range is replicated while its copies fit in this
-#endif
-#ifndef HIST_ASM_MATCH
-#define HIST_ASM_MATCH 1  // low eight index bits matched by rs_match1 (0: as the compiler writes it)
 #endif
 #ifndef HIST_VEC_KERNEL
 #define HIST_VEC_KERNEL 1  // float vector bins: a histogram per wave (0: the LDS kernel)
@@ -440,129 +437,6 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
   }
 }
 
-// ------------------------------------------- f64 sums into few bins
-// LDS atomics on floats run at about a quarter of the integer rate on MI355X
-// (2^27 updates: 670 us), and for 8-byte sums compare-and-swap is no faster
-// (H = 2048 f64: 260 against 247 us), so sums of f64 into few bins take another
-// route (the kernel also takes f32, which is how it was measured against
-// compare-and-swap: H = 256 uniform / Zipf 211 / 243 us against 170 / 174 us,
-// H = 2048 310 / 346 against 166 / 405 us): every wave keeps a histogram of its
-// own in LDS and updates it with
-// ordinary reads and writes.  Lanes of a wave that hit the same bin in the same
-// step find each other with one ballot per index bit (as the radix scatter
-// does): the first lane of a group adds its value with an ordinary read and
-// write, the other lanes of the group follow with the LDS float atomic (few
-// lanes, one instruction).  LDS operations of one wave complete in order, so
-// the atomics see the writes before them.  The 16 histograms of a block are
-// combined at the end and flushed with one device atomic per non-zero bin.
-//
-// A wave keeps 2^copies_log2 copies of its histogram where LDS allows, lane l
-// using copy l mod 2^copies_log2, so that fewer lanes share a cell and fewer
-// of them need the atomic.
-template <class T, class I, int INDEX_BITS /* 0: as many as `index_bits` says, not unrolled */>
-__global__ __launch_bounds__(HIST_BLOCK) void seghist_wave_private_kernel(
-    const I *__restrict__ is, const T *__restrict__ vs, int64_t n, T *dest, int64_t H,
-    int index_bits, int copies_log2) {
-  extern __shared__ __align__(16) unsigned char s_raw[];
-  T *sh = reinterpret_cast<T *>(s_raw);
-  constexpr int VEC = 4;
-  constexpr int WAVES = HIST_BLOCK / WAVE;
-  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / WAVE));
-  const int nb = (int)H;
-  const int copies = 1 << copies_log2;
-  // volatile: the compiler must not carry a bin across the rounds below in a register
-  volatile T *mine = sh + ((size_t)wave * nb << copies_log2);
-  for (int i = threadIdx.x; i < nb * WAVES * copies; i += HIST_BLOCK) sh[i] = T(0);
-  __syncthreads();
-  const uint32_t my_copy = (uint32_t)lane_id() & (uint32_t)(copies - 1);
-  // the lanes of my copy: every copies-th bit, starting at my_copy
-  uint32_t copy_mask = 0u;
-  for (int l = (int)my_copy; l < 32; l += copies) copy_mask |= 1u << l;
-
-  auto update = [&](int64_t bin, T v) {
-    const bool valid = (uint64_t)bin < (uint64_t)H;
-    const uint32_t b = valid ? (uint32_t)bin : 0u;
-    uint32_t differ_lo = 0u, differ_hi = 0u;
-    auto match_bit = [&](int bit) {
-      const uint32_t me = (uint32_t)(((int32_t)(b << (31 - bit))) >> 31);  // 0 or ~0
-      const uint64_t m = __ballot(me != 0u);
-      differ_lo |= (uint32_t)m ^ me;
-      differ_hi |= (uint32_t)(m >> 32) ^ me;
-    };
-    if constexpr (INDEX_BITS >= 8 && HIST_ASM_MATCH) {
-      // the low eight bits by the hand-scheduled match of the radix scatter
-      // (H = 256 f32: 297 -> 262 us), the others as the compiler writes them
-      uint32_t same_lo, same_hi;
-      rs_match1(b, same_lo, same_hi);
-      differ_lo = ~same_lo;
-      differ_hi = ~same_hi;
-#pragma unroll
-      for (int bit = 8; bit < INDEX_BITS; bit++) match_bit(bit);
-    } else if constexpr (INDEX_BITS > 0) {
-#pragma unroll
-      for (int bit = 0; bit < INDEX_BITS; bit++) match_bit(bit);
-    } else {
-      for (int bit = 0; bit < index_bits; bit++) match_bit(bit);
-    }
-    const uint32_t peers_lo = ~differ_lo, peers_hi = ~differ_hi;
-    const uint64_t vm = __ballot(valid);
-    const uint32_t lo = peers_lo & (uint32_t)vm & copy_mask;
-    const uint32_t hi = peers_hi & (uint32_t)(vm >> 32) & copy_mask;
-    // this lane's turn among the lanes with its bin and copy; lanes without a bin never get one
-    const int turn = valid ? (int)__builtin_amdgcn_mbcnt_hi(hi, __builtin_amdgcn_mbcnt_lo(lo, 0u)) : -1;
-    const uint32_t slot = (b << copies_log2) + my_copy;
-    // The first lane of every group adds with an ordinary read and write; the
-    // others follow with the LDS float atomic, which is slow per lane but
-    // issued once for all of them (LDS operations of a wave complete in order,
-    // so the atomics land on what the first lanes wrote).  Taking turns instead,
-    // one read and write per lane of the largest group, took 262 against 211 us
-    // (H = 256 f32, uniform indices) and 358 against 243 us (Zipf).
-    if (turn == 0) mine[slot] = mine[slot] + v;
-    __builtin_amdgcn_wave_barrier();
-    if (turn > 0)
-      AtomicUpdate<T, OpAdd<T>, __HIP_MEMORY_SCOPE_WORKGROUP>::apply(const_cast<T *>(&mine[slot]), v);
-    __builtin_amdgcn_wave_barrier();
-  };
-
-  const int64_t nvec = n / VEC;
-  const int64_t stride = (int64_t)gridDim.x * HIST_BLOCK;
-  for (int64_t i = (int64_t)blockIdx.x * HIST_BLOCK + threadIdx.x; i < nvec + (HIST_BLOCK - 1);
-       i += stride) {
-    // whole waves take part in every step, also the one with the ragged end
-    const int64_t first_of_wave = i - lane_id();
-    if (first_of_wave >= nvec) break;
-    I bi[VEC];
-    T bv[VEC];
-    if (i < nvec) {
-      load_elems4(bi, is + i * VEC);
-      load_elems4(bv, vs + i * VEC);
-    } else {
-#pragma unroll
-      for (int e = 0; e < VEC; e++) {
-        bi[e] = (I)-1;
-        bv[e] = T(0);
-      }
-    }
-#pragma unroll
-    for (int e = 0; e < VEC; e++) update((int64_t)bi[e], bv[e]);
-  }
-  if (blockIdx.x == 0 && wave == 0) {  // the n % VEC elements at the end
-    const int64_t t = nvec * VEC + lane_id();
-    const bool in = lane_id() < VEC && t < n;
-    update(in ? (int64_t)is[t] : (int64_t)-1, in ? vs[t] : T(0));
-  }
-  __syncthreads();
-  for (int r = threadIdx.x; r < nb; r += HIST_BLOCK) {
-    T acc = T(0);
-    for (int w = 0; w < WAVES; w++)
-      for (int c = 0; c < copies; c++) acc += sh[(((size_t)w * nb + r) << copies_log2) + c];
-    if (!bits_equal(acc, T(0))) global_update<T, OpAdd<T>>(dest + r, acc);
-  }
-}
-
-// ------------------------------------------------- partitioned large histograms
-// Digit of a pair = index of the LDS-sized bin range its bin falls in; 255 for
-// bins outside [0,H).
 template <class U> struct DigitBinRange {
   uint64_t H;
   int shift;
@@ -699,13 +573,16 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
   const int max_range = hist_range_bins_max(sizeof(A));
   const int P = (int)ceil_div(H, max_range);
   const int range_bins = (int)ceil_div(H, P);
-  // A small range is replicated while its copies fit in 32 KiB; f32 sums, where
-  // every lane that meets another on a cell costs a failed compare-and-swap,
-  // take 64 KiB, the most that leaves two blocks on a CU (Zipf indices,
-  // H = 1024 / 2048 / 4096: 314 / 407 / 471 -> 218 / 301 / 390 us; integer sums
-  // gain nothing from it).
+  // A small range is replicated while its copies fit in 32 KiB; float sums,
+  // where every lane that meets another on a cell costs a failed
+  // compare-and-swap (f32) or a slow atomic (f64), take 64 KiB, the most that
+  // leaves two blocks on a CU (f32, Zipf indices, H = 1024 / 2048 / 4096: 314 /
+  // 407 / 471 -> 218 / 301 / 390 us; f64 H = 256: 392 -> 250 us, which is also
+  // less than the 282 us of a kernel that kept a histogram per wave and is
+  // gone; integer sums gain nothing from it).
   constexpr bool f32_sum = std::is_same<A, float>::value && std::is_same<Op, OpAdd<T>>::value;
-  const int64_t copy_bytes = f32_sum ? 2 * HIST_COPY_BYTES : HIST_COPY_BYTES;
+  constexpr bool f64_sum = std::is_same<A, double>::value && std::is_same<Op, OpAdd<T>>::value;
+  const int64_t copy_bytes = f32_sum || f64_sum ? 2 * HIST_COPY_BYTES : HIST_COPY_BYTES;
   int log2_copies = 0;
   while (log2_copies < 5 && (int64_t)range_bins * (2 << log2_copies) * (int64_t)sizeof(A) <= copy_bytes)
     log2_copies++;
@@ -728,53 +605,12 @@ static int launch_lds_hist(hipStream_t st, const I *is, const T *vs, int64_t n, 
                                               log2_copies, seg_len, H_seg);
 }
 
-// Sums of floats into at most this many bytes of bins per wave go through
-// seghist_wave_private_kernel.
-constexpr int HIST_WAVE_PRIVATE_BYTES = HIST_LDS_BYTES / (HIST_BLOCK / WAVE);
-constexpr int HIST_WAVE_COPIES_MAX = 4;
-
-
-template <class T, class I>
-static int launch_wave_private_hist(hipStream_t st, const I *is, const T *vs, int64_t n, T *dest,
-                                    int64_t H) {
-  // The match loop over the index bits is unrolled (8 bits for up to 256 bins,
-  // else 11: HIST_WAVE_PRIVATE_BYTES / 4 = 2048 bins at most) except for 4-byte
-  // sums into up to 256 bins, where the unrolled loop costs registers and with
-  // them time (H = 256 f32: 309 against 297 us; H = 2048 f32: 428 against
-  // 465 us, H = 256 f64: 372 against 392 us in favour of unrolling).
-  static_assert(HIST_WAVE_PRIVATE_BYTES / 4 <= (1 << 11), "eleven index bits cover every bin");
-  int index_bits = 1;
-  while (((int64_t)1 << index_bits) < H) index_bits++;
-  // as many copies per wave (at most HIST_WAVE_COPIES_MAX) as leave room for two blocks on a CU
-  const size_t one = (size_t)H * sizeof(T) * (HIST_BLOCK / WAVE);
-  int copies_log2 = 0;
-  while ((1 << copies_log2) < HIST_WAVE_COPIES_MAX && (one << (copies_log2 + 1)) * 2 + 4096 <= 160 * 1024)
-    copies_log2++;
-  const size_t lds = one << copies_log2;
-  const int per_cu = lds * 2 + 4096 <= 160 * 1024 ? 2 : 1;
-  const dim3 grid(hist_num_cus() * per_cu);
-#define FA_WAVE_PRIVATE(BITS)                                                                  \
-  do {                                                                                         \
-    auto kernel = seghist_wave_private_kernel<T, I, BITS>;                                     \
-    /* Initialised once, under the lock C++ gives function-local statics. */                   \
-    static const hipError_t raised = hipFuncSetAttribute(                                      \
-        (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);     \
-    if (raised != hipSuccess) return (int)raised;                                              \
-    hipLaunchKernelGGL(kernel, grid, dim3(HIST_BLOCK), lds, st, is, vs, n, dest, H, index_bits, \
-                       copies_log2);                                                           \
-  } while (0)
-  if (H > 256)
-    FA_WAVE_PRIVATE(11);
-  else
-    FA_WAVE_PRIVATE(8);
-#undef FA_WAVE_PRIVATE
-  return launch_status();
-}
-
 // ------------------------------- float sums into few bins that are vectors
 // `reduce_by_index dest (map2 (+)) (replicate m 0) is vss` with float elements:
-// the same idea as seghist_wave_private_kernel, with a bin of m cells.  A lane
-// takes 16 bytes of a row of vss at a time (m is a multiple of that), so the
+// every wave keeps a histogram of its own in LDS and updates it with ordinary
+// reads and writes (LDS operations of one wave complete in order); the four
+// histograms of a block are combined at the end and flushed with one device
+// atomic per non-zero cell.  A lane takes 16 bytes of a row of vss at a time (m is a multiple of that), so the
 // lanes of a step cover consecutive rows; rows of one step with the same index
 // are told apart by the tag of the bin (the row number's low byte, written by
 // every lane of the row and read back): the row whose tag stayed adds its
@@ -954,16 +790,6 @@ static int launch_hist(hipStream_t st, const void *is, int is64, const void *vs,
   if (!is_aligned(is, 16) || !is_aligned(vs, 16) || !is_aligned(dest, sizeof(T))) return FA_EALIGN;
   const int64_t lds_limit =
       (int64_t)HIST_MAX_RANGES * hist_range_bins_max(sizeof(typename HistAcc<T>::A));
-  if constexpr (std::is_same<Op, OpAdd<T>>::value && std::is_same<T, double>::value) {
-    // f64 only: f32 sums are faster through compare-and-swap in the LDS kernel
-    if (H * (int64_t)sizeof(T) <= HIST_WAVE_PRIVATE_BYTES) {
-      if (is64)
-        return launch_wave_private_hist<T, int64_t>(st, (const int64_t *)is, (const T *)vs, n,
-                                                    (T *)dest, H);
-      return launch_wave_private_hist<T, int32_t>(st, (const int32_t *)is, (const T *)vs, n,
-                                                  (T *)dest, H);
-    }
-  }
   if (H <= lds_limit) {
     if (is64) return launch_lds_hist<T, Op, int64_t>(st, (const int64_t *)is, (const T *)vs, n, (T *)dest, H);
     return launch_lds_hist<T, Op, int32_t>(st, (const int32_t *)is, (const T *)vs, n, (T *)dest, H);

@@ -46,11 +46,12 @@ def test_hist_small_and_ragged(ctx, t, op):
 
 @pytest.mark.parametrize("t", ["f32", "f64"])
 def test_float_sums_every_size_class_exactly(ctx, t):
-    """Sums of floats do not use the LDS float atomic where it can be avoided: f32 reads the cell
-    and puts the sum back with compare-and-swap (one to four attempts, by the number of copies a
-    bin has), f64 into up to 1024 bins keeps a histogram per wave.  Bin counts on both sides of
-    every limit (copies, wave-private), uniform and skewed indices, one bin for everything; the
-    values are small whole numbers, so the sums are exact in any order and must match bit for bit."""
+    """Sums of floats: f32 reads the cell and puts the sum back with compare-and-swap (one to
+    four attempts, by the number of copies a bin has, then the float atomic), f64 uses the atomic;
+    both keep more copies of a small range than the integer operators.  Bin counts on both sides
+    of every change in the number of copies and ranges, uniform and skewed indices, one bin for
+    everything; the values are small whole numbers, so the sums are exact in any order and must
+    match bit for bit."""
     dt = {"f32": np.float32, "f64": np.float64}[t]
     rng = np.random.default_rng(77)
     n = 600011
