@@ -254,50 +254,6 @@ __device__ __forceinline__ void rs_match2(uint32_t da, uint32_t db, uint32_t &a_
       : "s84", "s85", "s86", "s87", "s88", "s89", "s90", "s91", "s92", "s93", "s94", "s95", "s96", "s97", "s98", "s99");
 }
 
-// The same for one digit per lane, with half the vector registers and scalar
-// registers below s72: a kernel that wants eight waves per SIMD may use at most
-// 96 scalar registers, which rs_match2's pairs (up to s99) would exceed.
-__device__ __forceinline__ void rs_match1(uint32_t d, uint32_t &lo, uint32_t &hi) {
-  uint32_t t0, t1, t2, t3;
-  asm(
-      "v_bfe_i32 %2, %6, 0, 1\n"
-      "v_bfe_i32 %3, %6, 1, 1\n"
-      "v_cmp_ne_u32_e64 s[64:65], 0, %2\n"
-      "v_cmp_ne_u32_e64 s[66:67], 0, %3\n"
-      "v_bfe_i32 %4, %6, 2, 1\n"
-      "v_bfe_i32 %5, %6, 3, 1\n"
-      "v_cmp_ne_u32_e64 s[68:69], 0, %4\n"
-      "v_cmp_ne_u32_e64 s[70:71], 0, %5\n"
-      "v_xnor_b32 %0, s64, %2\n"
-      "v_xnor_b32 %1, s65, %2\n"
-      "v_bitop3_b32 %0, %0, s66, %3 bitop3:0x90\n"
-      "v_bitop3_b32 %1, %1, s67, %3 bitop3:0x90\n"
-      "v_bfe_i32 %2, %6, 4, 1\n"
-      "v_bfe_i32 %3, %6, 5, 1\n"
-      "v_cmp_ne_u32_e64 s[64:65], 0, %2\n"
-      "v_cmp_ne_u32_e64 s[66:67], 0, %3\n"
-      "v_bitop3_b32 %0, %0, s68, %4 bitop3:0x90\n"
-      "v_bitop3_b32 %1, %1, s69, %4 bitop3:0x90\n"
-      "v_bitop3_b32 %0, %0, s70, %5 bitop3:0x90\n"
-      "v_bitop3_b32 %1, %1, s71, %5 bitop3:0x90\n"
-      "v_bfe_i32 %4, %6, 6, 1\n"
-      "v_bfe_i32 %5, %6, 7, 1\n"
-      "v_cmp_ne_u32_e64 s[68:69], 0, %4\n"
-      "v_cmp_ne_u32_e64 s[70:71], 0, %5\n"
-      "v_bitop3_b32 %0, %0, s64, %2 bitop3:0x90\n"
-      "v_bitop3_b32 %1, %1, s65, %2 bitop3:0x90\n"
-      "v_bitop3_b32 %0, %0, s66, %3 bitop3:0x90\n"
-      "v_bitop3_b32 %1, %1, s67, %3 bitop3:0x90\n"
-      "s_nop 0\n"
-      "v_bitop3_b32 %0, %0, s68, %4 bitop3:0x90\n"
-      "v_bitop3_b32 %1, %1, s69, %4 bitop3:0x90\n"
-      "v_bitop3_b32 %0, %0, s70, %5 bitop3:0x90\n"
-      "v_bitop3_b32 %1, %1, s71, %5 bitop3:0x90\n"
-      : "=&v"(lo), "=&v"(hi), "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
-      : "v"(d)
-      : "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71");
-}
-
 constexpr size_t RS_LDS_FIXED = RS_WAVES * RS_RADIX * 4 + 2 * RS_RADIX * 4 + 64;
 
 // Ranked scatter.  Inside a wave, lanes with equal digits find each other with
