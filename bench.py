@@ -64,6 +64,11 @@ def make_workload(name: str, ctx):
                 ctx.call(f"segred_{op}_{t}", [f"{t}_1d"], o, l, v).free()
             w["bytes"] = n * es + len(offsets) * (8 + es)
             w["kernel"] = "segred_irregular"
+            if t == "f32" and op == "add":
+                tmp = (np.empty(n, np.uint8), np.empty(n, np.float32))
+                w["cpu"] = lambda: oracle.mc_segred_add_f32(offsets, lens, xs, tmp=tmp)
+                w["cpu_how"] = ("segmented scan with flags written from the offsets, then one read "
+                                "per segment (what flattening makes of it)")
         w.update(step=step, dtype=t, bound="hbm", keep=[v],
                  describe=f"{kind} ({op}) over 2^{sz[2:]} {t}, {len(offsets)} irregular segments "
                           f"(geometric, mean 1024), u8 flags / i64 offsets")
@@ -77,8 +82,16 @@ def make_workload(name: str, ctx):
         if kind == "reduce":
             nt = np.float32 if t == "f32" else np.int32
 
+            import ctypes as C
+            entry = getattr(ctx.L, f"futhark_entry_reduce_{op}_{t}")
+            result = np.zeros(1, nt)
+            result_p = result.ctypes.data_as(C.c_void_p)
+
             def step():
-                ctx.call(f"reduce_{op}_{t}", [nt], a)
+                # The scalar arrives at the synchronisation that ends the timed loop
+                # (docs/c-api.rst:578-581), like the arrays of the other workloads.
+                ctx.check(entry(ctx.ptr, result_p, a.ptr))
+            w["result"] = result
             w["bytes"] = n * es
             w["kernel"] = "segred_nonseg"
             w["cpu"] = lambda: oracle.mc_reduce_add(t, xs)
@@ -115,6 +128,10 @@ def make_workload(name: str, ctx):
                                        f"indices, 1% out of range")
         if t == "i32" and op == "add":
             w["cpu"] = lambda: oracle.mc_rbi_add_i32(np.zeros(H, np.int32), is_, vs)
+        elif t == "f32" and op in ("add", "max"):
+            ne = np.float32(0.0 if op == "add" else -np.inf)
+            w["cpu"] = lambda: oracle.mc_rbi_f32(op, np.full(H, ne, np.float32), is_, vs)
+        w["cpu_how"] = "a private sub-histogram per task, then a reduce over the tasks per bin"
     elif name.startswith("rbivec_"):
         # rbivec_add_i32_H256x16_2p23: 2^23 updates of 16-element vectors into [256][16] bins
         _, op, t, hs, sz = name.split("_")
@@ -160,18 +177,24 @@ def make_workload(name: str, ctx):
         n = 1 << int(sz[2:])
         w["elements"] = n
         if kt == "u32":
-            k = ctx.new("u32_1d", dg.uniform_u32(80, n))
+            keys = dg.uniform_u32(80, n)
+            k = ctx.new("u32_1d", keys)
+            w["cpu"] = lambda: oracle.mc_radix_sort(keys)
 
             def step():
                 ctx.call("radix_sort_u32", ["u32_1d"], k).free()
             w.update(bytes=4 * 12 * n, keep=[k])
         else:
-            k = ctx.new("u64_1d", dg.uniform_u64(81, n))
-            vv = ctx.new("i32_1d", np.arange(n, dtype=np.int32))
+            keys, idx = dg.uniform_u64(81, n), np.arange(n, dtype=np.int32)
+            k = ctx.new("u64_1d", keys)
+            vv = ctx.new("i32_1d", idx)
+            w["cpu"] = lambda: oracle.mc_radix_sort(keys, idx)
 
             def step():
                 ctx.call("radix_sort_pairs_u64_i32", ["tup2_arr1d_u64_arr1d_i32"], k, vv).free()
             w.update(bytes=8 * 32 * n, keep=[k, vv])
+        w["cpu_how"] = ("per 8-bit digit a histogram per task, an exclusive scan of the [digit][task] "
+                        "counts and a stable scatter; each pass includes a copy of the unsorted input")
         w.update(step=step, kernel="radix_sort", dtype=kt, bound="hbm",
                  describe=f"stable LSD radix sort, 8-bit digits, 2^{sz[2:]} {kt}")
     elif name.startswith("bmm_"):
@@ -183,6 +206,14 @@ def make_workload(name: str, ctx):
         B = dg.normal_f32(65, b * m * m, sc).reshape(b, m, m)
         if t == "f32":
             a, bb = ctx.new("f32_3d", A), ctx.new("f32_3d", B)
+            # CPU: a bounded sample of the rows of C (all of B is needed for any row)
+            rows = min(b * m, max(16, (1 << 31) // (m * m)))
+            Bt = oracle.mc_transpose_f32(B)
+            Cs = np.empty((b, m, m), np.float32)
+            w["cpu"] = lambda: oracle.mc_bmm_rows_f32(A, Bt, Cs, 0, rows)
+            w["cpu_work"] = 2 * rows * m * m
+            w["cpu_how"] = (f"rows 0..{rows - 1} of the {b * m} rows of C: parallel over rows, sequential "
+                            f"loops over columns and k, B transposed once beforehand (not timed)")
         elif t == "f16":
             a, bb = ctx.new("f16_3d", dg.to_f16_bits(A)), ctx.new("f16_3d", dg.to_f16_bits(B))
         else:
@@ -449,6 +480,40 @@ def measure(ctx, w, steps: int, warmup: int, prewarm_seconds: float):
     }
 
 
+def cpu_baseline(w, seconds: float):
+    """Times the futhark-multicore-style restatement of the workload (oracle/multicore.c) on the
+    host cores for about `seconds`; None for a workload that has none."""
+    if "cpu" not in w:
+        return None
+    import oracle
+    hbm = w["bound"] == "hbm"
+    work = w.get("cpu_work", w["bytes"] if hbm else w["flops"])
+    w["cpu"]()  # warm-up
+    reps, t_cpu = 0, 0.0
+    start = time.perf_counter()
+    while t_cpu < seconds and reps < 100000:
+        w["cpu"]()
+        reps += 1
+        t_cpu = time.perf_counter() - start
+    scale, unit = (1e9, "GB/s") if hbm else (1e12, "TFLOP/s")
+    how = w.get("cpu_how")
+    whole = "cpu_work" not in w
+    cpu = {"value": round(work * reps / t_cpu / scale, 6 if not hbm else 3), "unit": unit,
+           "cores": oracle.mc_threads(), "kind": "port",
+           "sample": f"{reps} passes of " + ("the full workload" if whole else "a bounded part of the workload")
+                     + " with the futhark-multicore-style restatement in oracle/multicore.c"
+                     + (f" ({how})" if how else "") + f", {t_cpu:.1f} s"}
+    if "cpu_seq" in w:
+        fn, nbytes = w["cpu_seq"]
+        fn()
+        t_s = time.perf_counter()
+        fn()
+        cpu["single_thread"] = {"value": round(nbytes / (time.perf_counter() - t_s) / 1e9, 3),
+                                "unit": "GB/s", "sample": "one pass of oracle/oracle.c (the "
+                                "sequential futhark c fold) over the first 2^24 elements"}
+    return cpu
+
+
 def release(ctx, w) -> None:
     """Frees a workload's resident inputs and what the pool kept for it."""
     for a in w.get("keep", []):
@@ -480,6 +545,9 @@ def main() -> None:
                          "other BASELINE configurations are measured after it and reported "
                          "under `suite` in the same JSON line")
     ap.add_argument("--suite-steps", type=int, default=20)
+    ap.add_argument("--suite-cpu-seconds", type=float, default=1.5,
+                    help="CPU baseline time per workload of the suite (the headline workload "
+                         "gets --cpu-seconds)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run the plain copy kernel (fa_copy, 256 MiB) a few times, so "
                          "that a rocprofv3 --pmc run of this command holds a dispatch of known "
@@ -497,28 +565,7 @@ def main() -> None:
     w["name"] = args.workload
     m = measure(ctx, w, args.steps, args.warmup, args.prewarm_seconds)
 
-    cpu = None
-    if not args.no_cpu_baseline and "cpu" in w:
-        import oracle
-        w["cpu"]()  # warm-up
-        reps, t_cpu = 0, 0.0
-        start = time.perf_counter()
-        while t_cpu < args.cpu_seconds and reps < 100000:
-            w["cpu"]()
-            reps += 1
-            t_cpu = time.perf_counter() - start
-        cpu = {"value": round(w["bytes"] * reps / t_cpu / 1e9, 3), "unit": "GB/s",
-               "cores": oracle.mc_threads(), "kind": "port",
-               "sample": f"{reps} passes of the full workload with the futhark-multicore-style "
-                         f"restatement in oracle/multicore.c ({t_cpu:.1f} s)"}
-        if "cpu_seq" in w:
-            fn, nbytes = w["cpu_seq"]
-            fn()
-            t_s = time.perf_counter()
-            fn()
-            cpu["single_thread"] = {"value": round(nbytes / (time.perf_counter() - t_s) / 1e9, 3),
-                                    "unit": "GB/s", "sample": "one pass of oracle/oracle.c (the "
-                                    "sequential futhark c fold) over the first 2^24 elements"}
+    cpu = None if args.no_cpu_baseline else cpu_baseline(w, args.cpu_seconds)
 
     server = None
     if args.via_server:
@@ -573,6 +620,9 @@ def main() -> None:
                      "roofline": sm["roofline"]}
             if "elements" in sw:
                 entry["elements_per_s"] = round(sw["elements"] / (sm["ms_per_step"] * 1e-3), 1)
+            if not args.no_cpu_baseline:
+                sw.pop("cpu_seq", None)
+                entry["cpu_baseline"] = cpu_baseline(sw, args.suite_cpu_seconds)
             suite[name] = entry
             release(ctx, sw)
             print(f"[bench] {name}: {sm['value']} {sm['unit']}, kernel {sm['roofline']['kernel_us']} us, "

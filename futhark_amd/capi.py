@@ -117,14 +117,16 @@ class Segops:
                 getattr(L, f"futhark_entry_seghist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
                 getattr(L, f"futhark_entry_scanrows_{op}_{t}").argtypes = [vp, pp, vp]
                 getattr(L, f"futhark_entry_vecscan_{op}_{t}").argtypes = [vp, pp, vp]
-                getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
-                getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
+                for ix in ("", "_i64"):
+                    getattr(L, f"futhark_entry_hist_{op}_{t}{ix}").argtypes = [vp, pp, i64, vp, vp]
+                    getattr(L, f"futhark_entry_rbi_{op}_{t}{ix}").argtypes = [vp, pp, vp, vp, vp]
                 getattr(L, f"futhark_entry_rbi_vec_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
                 getattr(L, f"futhark_entry_rbi_2d_{op}_{t}").argtypes = [vp, pp, vp, vp, vp, vp]
         for t in HIST_ONLY_TYPES:
             for op in ops_for(t):
-                getattr(L, f"futhark_entry_hist_{op}_{t}").argtypes = [vp, pp, i64, vp, vp]
-                getattr(L, f"futhark_entry_rbi_{op}_{t}").argtypes = [vp, pp, vp, vp, vp]
+                for ix in ("", "_i64"):
+                    getattr(L, f"futhark_entry_hist_{op}_{t}{ix}").argtypes = [vp, pp, i64, vp, vp]
+                    getattr(L, f"futhark_entry_rbi_{op}_{t}{ix}").argtypes = [vp, pp, vp, vp, vp]
         for e in ("bmm_f32", "bmm_f16", "bmm_bf16", "matmul_f32"):
             getattr(L, f"futhark_entry_{e}").argtypes = [vp, pp, vp, vp]
         L.futhark_entry_scan_compose_i32.argtypes = [vp, pp, vp]

@@ -150,12 +150,14 @@ extern "C" size_t fa_hist_argmax_workspace_bytes(int64_t H) {
   return (size_t)(3 * H) * 4 + 256;  // two component arrays and the lock words
 }
 
-extern "C" int64_t fa_hist_argmax_max_bins(void) { return HL_MAX_BINS; }
+// Bins beyond what a block's LDS holds are updated in place under locks in
+// global memory; what bounds H is the 32-bit grid of the helper kernels.
+extern "C" int64_t fa_hist_argmax_max_bins(void) { return (int64_t)1 << 31; }
 
 // dest: [H][2]i32 (value, index) pairs, updated in place.
 extern "C" int fa_hist_argmax_i32(fa_stream_t stream, const int32_t *is, const int32_t *xs, int64_t n,
                                   int32_t *dest, int64_t H, void *workspace, size_t workspace_bytes) {
-  if (n < 0 || H < 0 || H > HL_MAX_BINS) return FA_EINVAL;
+  if (n < 0 || H < 0 || H > fa_hist_argmax_max_bins()) return FA_EINVAL;
   if (H == 0) return 0;
   if (dest == nullptr || workspace == nullptr || (n > 0 && (is == nullptr || xs == nullptr)))
     return FA_EINVAL;

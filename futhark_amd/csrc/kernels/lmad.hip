@@ -59,7 +59,8 @@ template <class T> constexpr int skinny_width() { return sizeof(T) == 8 ? 128 : 
 template <class T, bool SHORT_ROWS>
 __global__ __launch_bounds__(256) void transpose_skinny_kernel(T *__restrict__ dst,
                                                                const T *__restrict__ src,
-                                                               int64_t rows, int64_t cols) {
+                                                               int64_t rows, int64_t cols,
+                                                               int64_t first_block) {
   constexpr int W = skinny_width<T>();
   constexpr int LD = W + 1;  // padded: the strided side of each phase walks distinct banks
   __shared__ T tile[32 * LD];
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(256) void transpose_skinny_kernel(T *__restrict__ d
   const T *s = src + b * rows * cols;
   T *d = dst + b * rows * cols;
   const int tid = threadIdx.x;
-  const int64_t x0 = (int64_t)blockIdx.x * W;  // first long-axis index of the strip
+  const int64_t x0 = (first_block + blockIdx.x) * W;  // first long-axis index of the strip
   if (SHORT_ROWS) {
     const int S = (int)rows;
     const int w = (int)(cols - x0 < W ? cols - x0 : W);
@@ -92,14 +93,17 @@ __global__ __launch_bounds__(256) void transpose_skinny_kernel(T *__restrict__ d
 template <class T>
 __global__ __launch_bounds__(256) void transpose_tile_kernel(T *__restrict__ dst,
                                                              const T *__restrict__ src,
-                                                             int64_t rows, int64_t cols) {
+                                                             int64_t rows, int64_t cols,
+                                                             int64_t first_block) {
   constexpr int TS = 64;
   __shared__ T tile[TS][TS + 1];
-  // grid.x enumerates the tiles of one matrix row by row (the second and third
-  // grid dimensions hold 65535 at most), grid.y the matrices of the batch.
+  // grid.x enumerates the tiles of one matrix row by row, from `first_block` on
+  // (the second and third grid dimensions hold 65535 at most), grid.y the
+  // matrices of the batch.
   const int64_t b = blockIdx.y;
   const int64_t tiles_x = (cols + TS - 1) / TS;
-  const int64_t r0 = ((int64_t)blockIdx.x / tiles_x) * TS, c0 = ((int64_t)blockIdx.x % tiles_x) * TS;
+  const int64_t tile_id = first_block + blockIdx.x;
+  const int64_t r0 = (tile_id / tiles_x) * TS, c0 = (tile_id % tiles_x) * TS;
   const T *s = src + b * rows * cols;
   T *d = dst + b * rows * cols;
   const int tx = threadIdx.x % TS, ty = threadIdx.x / TS;  // 64 x 4
@@ -127,17 +131,20 @@ __global__ __launch_bounds__(256) void transpose_tile_kernel(T *__restrict__ dst
 template <class T>
 __global__ __launch_bounds__(256) void transpose_tile_vec_kernel(T *__restrict__ dst,
                                                                  const T *__restrict__ src,
-                                                                 int64_t rows, int64_t cols) {
+                                                                 int64_t rows, int64_t cols,
+                                                                 int64_t first_block) {
   constexpr int TS = 64;
   constexpr int V = 16 / sizeof(T);
   constexpr int LANES = TS / V;         // lanes across one tile row
   constexpr int STEP = 256 / LANES;     // tile rows covered per pass
   __shared__ T tile[TS][TS + 1];
-  // grid.x enumerates the tiles of one matrix row by row (the second and third
-  // grid dimensions hold 65535 at most), grid.y the matrices of the batch.
+  // grid.x enumerates the tiles of one matrix row by row, from `first_block` on
+  // (the second and third grid dimensions hold 65535 at most), grid.y the
+  // matrices of the batch.
   const int64_t b = blockIdx.y;
   const int64_t tiles_x = (cols + TS - 1) / TS;
-  const int64_t r0 = ((int64_t)blockIdx.x / tiles_x) * TS, c0 = ((int64_t)blockIdx.x % tiles_x) * TS;
+  const int64_t tile_id = first_block + blockIdx.x;
+  const int64_t r0 = (tile_id / tiles_x) * TS, c0 = (tile_id % tiles_x) * TS;
   const T *s = src + b * rows * cols;
   T *d = dst + b * rows * cols;
   const int tx = threadIdx.x % LANES, ty = threadIdx.x / LANES;
@@ -175,31 +182,43 @@ static int launch_map_transpose(hipStream_t st, T *dst, const T *src, int64_t ba
     }
     return 0;
   }
+  // A launch holds fewer than 2^32 threads along x: with 256 per block that is
+  // 16777215 blocks; longer grids go out in pieces.
+  constexpr int64_t MAX_BLOCKS_X = ((int64_t(1) << 32) - 1) / 256;
   if (rows <= 32 || cols <= 32) {
     const bool short_rows = rows <= cols;
     const int64_t longest = short_rows ? cols : rows;
     const int64_t gx = ceil_div(longest, (int64_t)skinny_width<T>());
-    if (gx > INT32_MAX) return FA_EINVAL;
-    const dim3 grid((unsigned)gx, (unsigned)batch);
-    if (short_rows)
-      hipLaunchKernelGGL((transpose_skinny_kernel<T, true>), grid, dim3(256), 0, st, dst, src,
-                         rows, cols);
-    else
-      hipLaunchKernelGGL((transpose_skinny_kernel<T, false>), grid, dim3(256), 0, st, dst, src,
-                         rows, cols);
-    return launch_status();
+    for (int64_t b0 = 0; b0 < gx; b0 += MAX_BLOCKS_X) {
+      const dim3 grid((unsigned)(gx - b0 < MAX_BLOCKS_X ? gx - b0 : MAX_BLOCKS_X), (unsigned)batch);
+      if (short_rows)
+        hipLaunchKernelGGL((transpose_skinny_kernel<T, true>), grid, dim3(256), 0, st, dst, src,
+                           rows, cols, b0);
+      else
+        hipLaunchKernelGGL((transpose_skinny_kernel<T, false>), grid, dim3(256), 0, st, dst, src,
+                           rows, cols, b0);
+      const int rc = launch_status();
+      if (rc != 0) return rc;
+    }
+    return 0;
   }
   const int64_t gx = ceil_div(cols, (int64_t)64), gy = ceil_div(rows, (int64_t)64);
-  if (gx * gy > INT32_MAX) return FA_EINVAL;  // more than 2^43 elements in one matrix
-  const dim3 grid((unsigned)(gx * gy), (unsigned)batch);
+  if (gx > INT64_MAX / gy) return FA_EINVAL;
+  const int64_t tiles = gx * gy;
   constexpr int V = 16 / (int)sizeof(T);
-  if (sizeof(T) >= 4 && rows % V == 0 && cols % V == 0 && is_aligned(dst, 16) &&
-      is_aligned(src, 16))
-    hipLaunchKernelGGL((transpose_tile_vec_kernel<T>), grid, dim3(256), 0, st, dst, src, rows,
-                       cols);
-  else
-    hipLaunchKernelGGL((transpose_tile_kernel<T>), grid, dim3(256), 0, st, dst, src, rows, cols);
-  return launch_status();
+  const bool vec = sizeof(T) >= 4 && rows % V == 0 && cols % V == 0 && is_aligned(dst, 16) &&
+                   is_aligned(src, 16);
+  for (int64_t b0 = 0; b0 < tiles; b0 += MAX_BLOCKS_X) {
+    const dim3 grid((unsigned)(tiles - b0 < MAX_BLOCKS_X ? tiles - b0 : MAX_BLOCKS_X), (unsigned)batch);
+    if (vec)
+      hipLaunchKernelGGL((transpose_tile_vec_kernel<T>), grid, dim3(256), 0, st, dst, src, rows,
+                         cols, b0);
+    else
+      hipLaunchKernelGGL((transpose_tile_kernel<T>), grid, dim3(256), 0, st, dst, src, rows, cols, b0);
+    const int rc = launch_status();
+    if (rc != 0) return rc;
+  }
+  return 0;
 }
 
 // ------------------------------------------------------------ classification

@@ -114,7 +114,7 @@ __device__ __forceinline__ void load_to_lds_16(const char *uniform_base, uint32_
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(
                    __builtin_amdgcn_readfirstlane(lds_addr)),
                "v"(lane_offset), "s"(sbase)
-               : "memory");
+               : "memory", "m0");
 }
 
 // BM x BN: the block's tile of C; WAVES_M x WAVES_N: how its waves share it.
@@ -620,11 +620,20 @@ static int launch_mm16(hipStream_t st, const uint16_t *A, const uint16_t *B, flo
   auto kernel = matmul16_kernel<BF16, BM, BN, WAVES_M, WAVES_N>;
   static const int raised = raise_lds(kernel, lds);
   if (raised) return raised;
-  if (M / BM > 65535) return FA_EINVAL;
-  const dim3 grid((unsigned)(N / BN), (unsigned)(M / BM), (unsigned)batch);
-  hipLaunchKernelGGL(kernel, grid, dim3(64 * WAVES_M * WAVES_N), lds, st, A, B, C, (int)M, (int)N,
-                     (int)K);
-  return launch_status();
+  // The grid's second dimension holds 65535 tile rows: a single matrix with more
+  // goes out in bands of rows (A and C advance, B stays); with a batch the
+  // matrices of a band would no longer be M rows apart, so that case is refused.
+  constexpr int64_t BAND = (int64_t)65535 * BM;
+  if (M > BAND && batch > 1) return FA_EINVAL;
+  for (int64_t r0 = 0; r0 < M; r0 += BAND) {
+    const int64_t rows = M - r0 < BAND ? M - r0 : BAND;
+    const dim3 grid((unsigned)(N / BN), (unsigned)(rows / BM), (unsigned)batch);
+    hipLaunchKernelGGL(kernel, grid, dim3(64 * WAVES_M * WAVES_N), lds, st, A + r0 * K, B, C + r0 * N,
+                       (int)rows, (int)N, (int)K);
+    const int rc = launch_status();
+    if (rc != 0) return rc;
+  }
+  return 0;
 }
 
 // 128 x 128 tiles serve shapes that are multiples of 128 but not of 256 without

@@ -34,29 +34,13 @@
 
 namespace fa {
 
-// Choices of the float-sum paths, overridable at compile time to measure the
-// alternative (the figures stand where each is used):
-#ifndef HIST_CAS_FEW
-#define HIST_CAS_FEW 1  // compare-and-swap attempts of an f32 sum before the float atomic ...
-#endif
-#ifndef HIST_CAS_MANY
-#define HIST_CAS_MANY 4  // ... and where a bin has at least 2^HIST_CAS_MANY_COPIES_LOG2 copies
-#endif
-#ifndef HIST_CAS_MANY_COPIES_LOG2
-#define HIST_CAS_MANY_COPIES_LOG2 2
-#endif
-#ifndef HIST_COPY_BYTES
-#define HIST_COPY_BYTES (32 * 1024)  // a bin range is replicated while its copies fit in this
-#endif
-#ifndef HIST_VEC_KERNEL
-#define HIST_VEC_KERNEL 1  // float vector bins: a histogram per wave (0: the LDS kernel)
-#endif
-#ifndef HIST_VEC_MIN_BYTES
-#define HIST_VEC_MIN_BYTES 8192  // bytes of cells up to which float vector bins stay with the LDS kernel
-#endif
-#ifndef HIST_VEC_UNROLL
-#define HIST_VEC_UNROLL 8  // 16-byte loads a lane of the vector-bin kernel keeps in flight
-#endif
+// Choices of the float-sum paths (the measurements stand where each is used).
+constexpr int HIST_CAS_FEW = 1;   // compare-and-swap attempts of an f32 sum before the float atomic ...
+constexpr int HIST_CAS_MANY = 4;  // ... and where a bin has at least 2^HIST_CAS_MANY_COPIES_LOG2 copies
+constexpr int HIST_CAS_MANY_COPIES_LOG2 = 2;
+constexpr int HIST_COPY_BYTES = 32 * 1024;  // a bin range is replicated while its copies fit in this
+constexpr int HIST_VEC_MIN_BYTES = 8192;    // bytes of cells up to which float vector bins stay with the LDS kernel
+constexpr int HIST_VEC_UNROLL = 8;          // 16-byte loads a lane of the vector-bin kernel keeps in flight
 constexpr int HIST_BLOCK = 1024;
 constexpr int HIST_LDS_BYTES = 128 * 1024;  // bin storage per block
 constexpr int HIST_MAX_RANGES = 4;          // ranges covered by one launch
@@ -897,7 +881,7 @@ static int launch_hist_shaped(hipStream_t st, const void *is, const void *js, in
     // above: f32 [192][16] 150 against 116 us, [256][16] 148 against 122,
     // [512][16] 236 against 194 in favour of this kernel).
     const bool many_cells = H * (int64_t)sizeof(T) > HIST_VEC_MIN_BYTES;
-    if (HIST_VEC_KERNEL && many_cells && js == nullptr && m > 1 && hist_vec_lds_bytes<T>(H0, m) != 0) {
+    if (many_cells && js == nullptr && m > 1 && hist_vec_lds_bytes<T>(H0, m) != 0) {
       if (is64)
         return launch_wave_private_vec_hist<T, int64_t>(st, (const int64_t *)is, (const T *)vss,
                                                         n_updates, (T *)dest, H0, m);

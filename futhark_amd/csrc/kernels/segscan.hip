@@ -31,7 +31,8 @@
 namespace fa {
 
 // ---- scratch for the entry point that allocates nothing
-constexpr size_t SCAN_STATIC_BYTES = 256 * 1024;
+// The header and 256 KiB of tile descriptors (16384 tiles).
+constexpr size_t SCAN_STATIC_BYTES = SCAN_HEADER_BYTES + 256 * 1024;
 constexpr int SCAN_STATIC_EPOCH_WORD = 16;  // 32-bit word of the header that holds the epoch
 
 }  // namespace fa
@@ -119,6 +120,12 @@ extern "C" int fa_segscan_static(fa_stream_t stream, fa_dtype t, fa_op op, const
                ? launch_scan_static<AffineI32, OpCompose>(s, xs, flags, n, exclusive, out, base)
                : FA_ENOTSUP;
   FA_DISPATCH_TYPE_OP(launch_scan_static, t, op, s, xs, flags, n, exclusive, out, base);
+}
+
+extern "C" int64_t fa_segscan_tile_elems(fa_dtype t) {
+  const size_t es = dtype_size(t);
+  if (es != 4 && es != 8) return 0;
+  return (es == 4) ? ss_tile_elems<int32_t>() : ss_tile_elems<int64_t>();
 }
 
 extern "C" size_t fa_segscan_scratch_bytes(fa_dtype t, int64_t n) {

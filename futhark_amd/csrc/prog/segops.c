@@ -237,14 +237,17 @@ static int do_reduce(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t e
   uint32_t epoch = 0;
   void *scratch = rts_scan_scratch(ctx, fa_segred_scratch_bytes(t), &epoch);
   if (scratch == NULL) return ctx->error ? FUTHARK_OUT_OF_MEMORY : 1;
-  /* The kernel stores the one result into the context's pinned host slot. */
+  /* The kernel stores the one result into a pinned host slot of the context;
+   * the caller gets it at the next futhark_context_sync. */
+  void *slot = rts_scalar_slot(ctx);
+  if (slot == NULL) return 1;
   struct rts_event *ev = rts_kernel_begin(
       ctx, "segred_nonseg", rts_msgprintf("{\"n\":%lld,\"bytes\":%lld}", (long long)n,
                                           (long long)(n * (int64_t)es)));
-  int code = fa_segred_nonseg(ctx->stream, t, op, in->mem.mem, n, ctx->scalar_stage, scratch,
+  int code = fa_segred_nonseg(ctx->stream, t, op, in->mem.mem, n, slot, scratch,
                               ctx->scan_scratch_bytes, epoch);
   int err = rts_kernel_end(ctx, ev, "segred_nonseg", code);
-  if (err == 0) err = rts_take_scalar(ctx, out, es);
+  if (err == 0) err = rts_take_scalar(ctx, slot, out, es);
   return err;
 }
 
@@ -491,7 +494,8 @@ static uint64_t neutral_bits(fa_dtype t, fa_op op) {
 /* dest_in == NULL: histogram into a fresh array of k neutral elements. */
 static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
                    struct fut_array **out, int64_t k, const struct fut_array *dest_in,
-                   const struct fut_array *is, const struct fut_array *vs, const char *entry) {
+                   const struct fut_array *is, int is64, const struct fut_array *vs,
+                   const char *entry) {
   const int64_t n = is->shape[0];
   if (vs->shape[0] != n) return bad_sizes(ctx, entry);
   if (dest_in != NULL) k = dest_in->shape[0];
@@ -514,13 +518,13 @@ static int do_hist(struct futhark_context *ctx, fa_dtype t, fa_op op, size_t es,
   }
   struct memblock_device scratch = {0};
   if (err == 0) {
-    err = rts_memblock_alloc(ctx, &scratch, (int64_t)fa_seghist_scratch_bytes(t, 0, n, k),
+    err = rts_memblock_alloc(ctx, &scratch, (int64_t)fa_seghist_scratch_bytes(t, is64, n, k),
                              "hist.scratch");
   }
   if (err == 0) {
     struct rts_event *ev = rts_kernel_begin(
         ctx, "seghist", rts_msgprintf("{\"n\":%lld,\"bins\":%lld}", (long long)n, (long long)k));
-    int code = fa_seghist(ctx->stream, t, op, is->mem.mem, 0, vs->mem.mem, n, res->mem.mem, k,
+    int code = fa_seghist(ctx->stream, t, op, is->mem.mem, is64, vs->mem.mem, n, res->mem.mem, k,
                           scratch.mem, (size_t)scratch.size);
     err = rts_kernel_end(ctx, ev, "seghist", code);
   }
@@ -751,24 +755,29 @@ static int do_rbi_shaped(struct futhark_context *ctx, fa_dtype t, fa_op op, size
   DEFINE_HIST_ENTRIES(OP, T, CT)
 
 #define DEFINE_HIST_ENTRIES(OP, T, CT)                                                        \
-  int futhark_entry_hist_##OP##_##T(struct futhark_context *ctx,                              \
-                                    struct futhark_##T##_1d **out0, const int64_t in0,        \
-                                    const struct futhark_i32_1d *in1,                         \
-                                    const struct futhark_##T##_1d *in2) {                     \
+  DEFINE_HIST_ENTRIES_IX(OP, T, CT, , i32, 0)                                                 \
+  DEFINE_HIST_ENTRIES_IX(OP, T, CT, _i64, i64, 1)
+/* SUFFIX: nothing for []i32 indices (widened in the fused map), _i64 for the []i64
+ * indices `hist` and `reduce_by_index` are defined over (prelude/soacs.fut:132-146). */
+#define DEFINE_HIST_ENTRIES_IX(OP, T, CT, SUFFIX, IT, IS64)                                   \
+  int futhark_entry_hist_##OP##_##T##SUFFIX(struct futhark_context *ctx,                      \
+                                            struct futhark_##T##_1d **out0, const int64_t in0, \
+                                            const struct futhark_##IT##_1d *in1,              \
+                                            const struct futhark_##T##_1d *in2) {             \
     ENTER(ctx);                                                                               \
     int ret = do_hist(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, in0, NULL, \
-                      &in1->a, &in2->a, "hist_" #OP "_" #T);                                  \
+                      &in1->a, IS64, &in2->a, "hist_" #OP "_" #T #SUFFIX);                    \
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }                                                                                           \
-  int futhark_entry_rbi_##OP##_##T(struct futhark_context *ctx,                               \
-                                   struct futhark_##T##_1d **out0,                            \
-                                   const struct futhark_##T##_1d *in0,                        \
-                                   const struct futhark_i32_1d *in1,                          \
-                                   const struct futhark_##T##_1d *in2) {                      \
+  int futhark_entry_rbi_##OP##_##T##SUFFIX(struct futhark_context *ctx,                       \
+                                           struct futhark_##T##_1d **out0,                    \
+                                           const struct futhark_##T##_1d *in0,                \
+                                           const struct futhark_##IT##_1d *in1,               \
+                                           const struct futhark_##T##_1d *in2) {              \
     ENTER(ctx);                                                                               \
     int ret = do_hist(ctx, DT_##T, OP_##OP, sizeof(CT), (struct fut_array **)out0, 0,         \
-                      &in0->a, &in1->a, &in2->a, "rbi_" #OP "_" #T);                          \
+                      &in0->a, &in1->a, IS64, &in2->a, "rbi_" #OP "_" #T #SUFFIX);            \
     LEAVE(ctx);                                                                               \
     return ret;                                                                               \
   }
@@ -876,8 +885,9 @@ int futhark_entry_reduce_compose_i32(struct futhark_context *ctx, struct futhark
 
 int futhark_entry_sumsq_f32(struct futhark_context *ctx, float *out0, const struct futhark_f32_1d *in0) {
   ENTER(ctx);
-  int ret = do_custom_reduce(ctx, sumsq_fn, "segred_sumsq", &in0->a, in0->a.shape[0], ctx->scalar_stage);
-  if (ret == 0) ret = rts_take_scalar(ctx, out0, 4);
+  void *slot = rts_scalar_slot(ctx);
+  int ret = slot == NULL ? 1 : do_custom_reduce(ctx, sumsq_fn, "segred_sumsq", &in0->a, in0->a.shape[0], slot);
+  if (ret == 0) ret = rts_take_scalar(ctx, slot, out0, 4);
   LEAVE(ctx);
   return ret;
 }

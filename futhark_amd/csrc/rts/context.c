@@ -244,10 +244,14 @@ static int backend_setup(struct futhark_context *ctx) {
   hipStream_t s;
   if (hip_check(ctx, hipStreamCreate(&s), "hipStreamCreate") != 0) return 1;
   ctx->stream = (void *)s;
-  if (hip_check(ctx, hipHostMalloc(&ctx->scalar_stage, 256, hipHostMallocDefault),
-                "hipHostMalloc (scalar slot)") != 0)
+  if (hip_check(ctx, hipHostMalloc(&ctx->scalar_stage, RTS_SCALAR_STAGE_BYTES, hipHostMallocDefault),
+                "hipHostMalloc (scalar slots)") != 0) {
+    ctx->scalar_stage = NULL;
+    (void)hipStreamDestroy(s);
+    ctx->stream = NULL;
     return 1;
-  memset(ctx->scalar_stage, 0, 256);
+  }
+  memset(ctx->scalar_stage, 0, RTS_SCALAR_STAGE_BYTES);
   if (ctx->logging) {
     fprintf(ctx->log, "Device: %s, %d CUs, %zu B LDS per block, %zu B L2, %s memory\n",
             ctx->device_name, ctx->num_cus, ctx->max_shared_memory, ctx->l2_cache_bytes,
@@ -392,12 +396,50 @@ int rts_copy_d2h(struct futhark_context *ctx, void *dst, const void *src, size_t
   return hip_check(ctx, hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost,
                                        (hipStream_t)ctx->stream), "hipMemcpyAsync (D2H)");
 }
-int rts_take_scalar(struct futhark_context *ctx, void *dst, size_t bytes) {
-  if (bytes > 256) return 1;
-  int err = hip_check(ctx, hipStreamSynchronize((hipStream_t)ctx->stream), "hipStreamSynchronize");
-  if (err != 0) return err;
-  memcpy(dst, ctx->scalar_stage, bytes);
-  return 0;
+/* Hands over the scalars of slots [head, upto): the caller has drained the
+ * stream after `upto` was read, so their kernels have finished. */
+static void deliver_scalars(struct futhark_context *ctx, uint64_t upto) {
+  pthread_mutex_lock(&ctx->scalar_lock);
+  while (ctx->scalar_head < upto) {
+    const size_t i = (size_t)(ctx->scalar_head % RTS_SCALAR_SLOTS);
+    memcpy(ctx->scalar_pending[i].dst, (char *)ctx->scalar_stage + 256 + i * RTS_SCALAR_SLOT_BYTES,
+           ctx->scalar_pending[i].bytes);
+    ctx->scalar_head++;
+  }
+  pthread_mutex_unlock(&ctx->scalar_lock);
+}
+static uint64_t scalars_queued(struct futhark_context *ctx) {
+  pthread_mutex_lock(&ctx->scalar_lock);
+  const uint64_t tail = ctx->scalar_tail;
+  pthread_mutex_unlock(&ctx->scalar_lock);
+  return tail;
+}
+void *rts_scalar_slot(struct futhark_context *ctx) {
+  /* Entry points run one at a time (the context's lock), so the tail does not
+   * move between this call and rts_take_scalar. */
+  pthread_mutex_lock(&ctx->scalar_lock);
+  const uint64_t tail = ctx->scalar_tail;
+  const int full = tail - ctx->scalar_head >= RTS_SCALAR_SLOTS;
+  pthread_mutex_unlock(&ctx->scalar_lock);
+  if (full) {
+    if (hip_check(ctx, hipStreamSynchronize((hipStream_t)ctx->stream), "hipStreamSynchronize") != 0)
+      return NULL;
+    deliver_scalars(ctx, tail);
+  }
+  return (char *)ctx->scalar_stage + 256 + (size_t)(tail % RTS_SCALAR_SLOTS) * RTS_SCALAR_SLOT_BYTES;
+}
+int rts_take_scalar(struct futhark_context *ctx, void *slot, void *dst, size_t bytes) {
+  if (bytes > RTS_SCALAR_SLOT_BYTES || dst == NULL) return 1;
+  pthread_mutex_lock(&ctx->scalar_lock);
+  const size_t i = (size_t)(ctx->scalar_tail % RTS_SCALAR_SLOTS);
+  const int ok = slot == (char *)ctx->scalar_stage + 256 + i * RTS_SCALAR_SLOT_BYTES;
+  if (ok) {
+    ctx->scalar_pending[i].dst = dst;
+    ctx->scalar_pending[i].bytes = bytes;
+    ctx->scalar_tail++;
+  }
+  pthread_mutex_unlock(&ctx->scalar_lock);
+  return ok ? 0 : 1;
 }
 int rts_copy_d2d(struct futhark_context *ctx, void *dst, const void *src, size_t bytes) {
   if (bytes == 0) return 0;
@@ -538,25 +580,30 @@ void futhark_context_set_logging_file(struct futhark_context *ctx, FILE *f) { ct
 
 int futhark_context_sync(struct futhark_context *ctx) {
   if (ctx->stream == NULL) return 1;
+  /* Scalars queued up to here belong to work this synchronisation waits for. */
+  const uint64_t queued = scalars_queued(ctx);
   hipError_t e = hipStreamSynchronize((hipStream_t)ctx->stream);
   if (e != hipSuccess) return hip_check(ctx, e, "hipStreamSynchronize");
+  deliver_scalars(ctx, queued);
+  /* The device's failure word is read and cleared whatever else is pending, so
+   * that a failure of this interval cannot surface at a later, unrelated
+   * synchronisation; an error deferred by the host goes first (it was raised
+   * first: the first error wins, rts/c/context.h:5-13). */
+  volatile int32_t *failure = ctx->scalar_stage != NULL ? RTS_FAILURE_WORD(ctx) : NULL;
+  const int32_t code = failure != NULL ? *failure : 0;
+  if (code != 0) *failure = 0;
   if (ctx->pending_error != 0) {
     int p = ctx->pending_error;
     ctx->pending_error = 0;
     return p;
   }
-  if (ctx->scalar_stage != NULL) {
-    volatile int32_t *failure = RTS_FAILURE_WORD(ctx);
-    const int32_t code = *failure;
-    if (code != 0) {
-      *failure = 0;
-      rts_set_error(ctx, rts_msgprintf(
-          code == RTS_FAILURE_SEGMENTS
-              ? "Error: segments are not in order, overlap or leave the array (offsets[i] + lens[i] "
-                "<= offsets[i+1] <= n required).\n"
-              : "Error: a kernel reported failure %d.\n", (int)code));
-      return FUTHARK_PROGRAM_ERROR;
-    }
+  if (code != 0) {
+    rts_set_error(ctx, rts_msgprintf(
+        code == RTS_FAILURE_SEGMENTS
+            ? "Error: segments are not in order, overlap or leave the array (offsets[i] + lens[i] "
+              "<= offsets[i+1] <= n required).\n"
+            : "Error: a kernel reported failure %d.\n", (int)code));
+    return FUTHARK_PROGRAM_ERROR;
   }
   return FUTHARK_SUCCESS;
 }
@@ -582,6 +629,7 @@ struct futhark_context *futhark_context_new(struct futhark_context_config *cfg) 
   cfg->in_use = 1;
   pthread_mutex_init(&ctx->lock, NULL);
   pthread_mutex_init(&ctx->error_lock, NULL);
+  pthread_mutex_init(&ctx->scalar_lock, NULL);
   free_list_init(&ctx->gpu_free_list);
   ctx->debugging = cfg->debugging;
   ctx->logging = cfg->logging;
@@ -610,6 +658,7 @@ void futhark_context_free(struct futhark_context *ctx) {
   free(ctx->error);
   pthread_mutex_destroy(&ctx->lock);
   pthread_mutex_destroy(&ctx->error_lock);
+  pthread_mutex_destroy(&ctx->scalar_lock);
   ctx->cfg->in_use = 0;
   free(ctx);
 }

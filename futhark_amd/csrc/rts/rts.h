@@ -163,11 +163,24 @@ struct futhark_context {
   size_t scan_scratch_bytes;
   uint32_t scan_epoch;
 
-  /* a pinned host slot (hipHostMalloc, 256 bytes) the device can write: a kernel
-   * that produces one scalar stores it here, and the entry point hands it to
-   * the caller after the stream has drained, without a copy operation
-   * (a copy into pageable memory costs about 20 us per call). */
+  /* pinned host memory (hipHostMalloc) the device can write: 256 bytes of
+   * header, then a ring of RTS_SCALAR_SLOTS slots of 16 bytes.  A kernel that
+   * produces one scalar stores it into a slot; the entry point records where
+   * the caller wants it, and futhark_context_sync hands it over once the
+   * stream has drained (docs/c-api.rst:578-581: a scalar result may be used
+   * after the synchronisation).  No copy operation and no wait inside the
+   * entry point (a copy into pageable memory costs about 20 us per call, a
+   * wait per call about 10). */
   void *scalar_stage;
+#define RTS_SCALAR_SLOTS 64
+#define RTS_SCALAR_SLOT_BYTES 16
+#define RTS_SCALAR_STAGE_BYTES (256 + RTS_SCALAR_SLOTS * RTS_SCALAR_SLOT_BYTES)
+  struct {
+    void *dst;     /* where the caller wants the value */
+    size_t bytes;
+  } scalar_pending[RTS_SCALAR_SLOTS];
+  uint64_t scalar_head, scalar_tail; /* slots [head, tail) await delivery; slot = index mod RTS_SCALAR_SLOTS */
+  pthread_mutex_t scalar_lock;
   /* a word of that slot (byte 128) kernels raise when the program must fail, as
    * the reference's global_failure (rts/c/gpu.h): checked and cleared at every
    * synchronisation, which then returns FUTHARK_PROGRAM_ERROR */
@@ -199,8 +212,13 @@ int rts_memblock_set(struct futhark_context *ctx, struct memblock_device *lhs,
 /* copies on the context's stream; asynchronous (hip.h:790-862) */
 int rts_copy_h2d(struct futhark_context *ctx, void *dst, const void *src, size_t bytes);
 int rts_copy_d2h(struct futhark_context *ctx, void *dst, const void *src, size_t bytes);
-/* waits for the stream, then copies `bytes` (at most 256) from the pinned scalar slot to dst */
-int rts_take_scalar(struct futhark_context *ctx, void *dst, size_t bytes);
+/* A pinned slot for one scalar result of the launch about to be queued (NULL on
+ * failure, error set); when every slot awaits delivery the stream is drained
+ * and the values are handed over first. */
+void *rts_scalar_slot(struct futhark_context *ctx);
+/* After the launch: `bytes` (at most RTS_SCALAR_SLOT_BYTES) of `slot` go to
+ * `dst` at the next futhark_context_sync.  dst must stay valid until then. */
+int rts_take_scalar(struct futhark_context *ctx, void *slot, void *dst, size_t bytes);
 int rts_copy_d2d(struct futhark_context *ctx, void *dst, const void *src, size_t bytes);
 int rts_memset0(struct futhark_context *ctx, void *dst, size_t bytes);
 

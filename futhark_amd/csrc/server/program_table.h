@@ -208,14 +208,17 @@ struct entry {
                                            ARRP(i[0]), ARRP(i[1]), ARRP(i[2]), ARRP(i[3]));    \
   }                                                                                            \
   HIST_ENTRY_FNS(OP, T, CT)
-#define HIST_ENTRY_FNS(OP, T, CT)                                                              \
-  static int e_hist_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) { \
-    return futhark_entry_hist_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr,             \
-                                         i[0]->u.i64, ARRP(i[1]), ARRP(i[2]));                 \
+#define HIST_ENTRY_FNS(OP, T, CT) HIST_ENTRY_FNS_IX(OP, T, CT, ) HIST_ENTRY_FNS_IX(OP, T, CT, _i64)
+#define HIST_ENTRY_FNS_IX(OP, T, CT, SUFFIX)                                                   \
+  static int e_hist_##OP##_##T##SUFFIX(struct futhark_context *c, struct value *o,             \
+                                       struct value **i) {                                     \
+    return futhark_entry_hist_##OP##_##T##SUFFIX(c, (struct futhark_##T##_1d **)&o->u.arr,     \
+                                                 i[0]->u.i64, ARRP(i[1]), ARRP(i[2]));         \
   }                                                                                            \
-  static int e_rbi_##OP##_##T(struct futhark_context *c, struct value *o, struct value **i) {  \
-    return futhark_entry_rbi_##OP##_##T(c, (struct futhark_##T##_1d **)&o->u.arr, ARRP(i[0]),  \
-                                        ARRP(i[1]), ARRP(i[2]));                               \
+  static int e_rbi_##OP##_##T##SUFFIX(struct futhark_context *c, struct value *o,              \
+                                      struct value **i) {                                      \
+    return futhark_entry_rbi_##OP##_##T##SUFFIX(c, (struct futhark_##T##_1d **)&o->u.arr,      \
+                                                ARRP(i[0]), ARRP(i[1]), ARRP(i[2]));           \
   }
 #define SEGOP_ENTRY_FNS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(SEGOP_ENTRY_FNS, T, CT)
 FUTHARK_FOR_EACH_NUM_TYPE(SEGOP_ENTRY_FNS_FOR_TYPE)
@@ -331,11 +334,13 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
   {"rbi_2d_" #OP "_" #T, e_rbi_2d_##OP##_##T, "[][]" #T, 1, 4,                                  \
    {"[][]" #T, "[]i64", "[]i64", "[]" #T}, {1, 0, 0, 0}, {HIST_PARAM, NULL}},                   \
   HIST_ENTRY_ROWS(OP, T, CT)
-#define HIST_ENTRY_ROWS(OP, T, CT)                                                              \
-  {"hist_" #OP "_" #T, e_hist_##OP##_##T, "[]" #T, 1, 3, {"i64", "[]i32", "[]" #T}, {0},        \
-   {HIST_PARAM, NULL}},                                                                         \
-  {"rbi_" #OP "_" #T, e_rbi_##OP##_##T, "[]" #T, 1, 3, {"[]" #T, "[]i32", "[]" #T}, {1, 0, 0},  \
-   {HIST_PARAM, NULL}},
+#define HIST_ENTRY_ROWS(OP, T, CT) \
+  HIST_ENTRY_ROWS_IX(OP, T, CT, , "[]i32") HIST_ENTRY_ROWS_IX(OP, T, CT, _i64, "[]i64")
+#define HIST_ENTRY_ROWS_IX(OP, T, CT, SUFFIX, IXT)                                              \
+  {"hist_" #OP "_" #T #SUFFIX, e_hist_##OP##_##T##SUFFIX, "[]" #T, 1, 3,                        \
+   {"i64", IXT, "[]" #T}, {0}, {HIST_PARAM, NULL}},                                             \
+  {"rbi_" #OP "_" #T #SUFFIX, e_rbi_##OP##_##T##SUFFIX, "[]" #T, 1, 3,                          \
+   {"[]" #T, IXT, "[]" #T}, {1, 0, 0}, {HIST_PARAM, NULL}},
 #define SEGOP_ENTRY_ROWS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(SEGOP_ENTRY_ROWS, T, CT)
 #define SEGOP_BITOP_ROWS_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_BITOP(SEGOP_ENTRY_ROWS, T, CT)
 #define HIST_ONLY_INT_ROWS(T, CT) \

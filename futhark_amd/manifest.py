@@ -64,10 +64,11 @@ def entry_points() -> dict:
     for t in list(NUM_TYPES) + list(HIST_ONLY_TYPES):
         for op in ops_for(t):
             a = f"[]{t}"
-            eps += [
-                _entry(f"hist_{op}_{t}", a, [("k", "i64"), ("is", "[]i32"), ("vs", a)], [HIST_PARAM]),
-                _entry(f"rbi_{op}_{t}", a, [("dest", "*" + a), ("is", "[]i32"), ("vs", a)], [HIST_PARAM]),
-            ]
+            for ix, it in (("", "[]i32"), ("_i64", "[]i64")):
+                eps += [
+                    _entry(f"hist_{op}_{t}{ix}", a, [("k", "i64"), ("is", it), ("vs", a)], [HIST_PARAM]),
+                    _entry(f"rbi_{op}_{t}{ix}", a, [("dest", "*" + a), ("is", it), ("vs", a)], [HIST_PARAM]),
+                ]
     eps += [
         _entry("bmm_f32", "[][][]f32", [("A", "[][][]f32"), ("B", "[][][]f32")], [MATMUL_PARAM]),
         _entry("bmm_f16", "[][][]f32", [("A", "[][][]f16"), ("B", "[][][]f16")], [MATMUL_PARAM]),

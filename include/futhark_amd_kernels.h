@@ -160,6 +160,10 @@ int fa_segred_columns(fa_stream_t stream, fa_dtype t, fa_op op,
  * (1 <= epoch < 2^28; zero-fill again before wrapping).  Tile descriptors
  * carry the epoch, so no per-call clearing kernel is needed. */
 size_t fa_segscan_scratch_bytes(fa_dtype t, int64_t n);
+/* Elements of type t per tile (the unit of the look-back: one descriptor per
+ * tile; the reference's B * chunk elements of a virtual block,
+ * SinglePass.hs:32-48).  0 for types the scan does not take. */
+int64_t fa_segscan_tile_elems(fa_dtype t);
 int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op,
                const void *xs, const uint8_t *flags, int64_t n, int exclusive,
                void *out, void *scratch, size_t scratch_bytes, uint32_t epoch);
@@ -175,7 +179,9 @@ int fa_segscan_rows(fa_stream_t stream, fa_dtype t, fa_op op,
 /* fa_segscan for callers that cannot allocate or pass a workspace: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It
  * has no counterpart in the reference.  The look-back scratch is a fixed
- * 256 KiB array inside the library (one copy per GPU, held until the process
+ * array inside the library (a header and 256 KiB of tile descriptors, 16384
+ * tiles: 234 881 024 four-byte or 117 440 512 eight-byte elements; one copy per
+ * GPU, held until the process
  * ends), its epoch lives in that array and is advanced on the device, so
  * identical launches may be repeated.  No device memory is allocated or
  * freed.  n beyond fa_segscan_static_max_n(t) returns FA_ESCRATCH.  All calls
@@ -362,7 +368,9 @@ int fa_iota(fa_stream_t stream, fa_dtype t, void *dst, int64_t n,
  *   fa_scan_norm_f32:     map sqrt (scan (+) 0 (map (\x -> x*x) xs))
  *   fa_hist_argmax_i32:   reduce_by_index with argmax into dest [H][2]i32 (updated
  *                         in place), bins locked while updated because the tuple's
- *                         components live in two arrays (ImpGen/GPU/Base.hs:769-842);
+ *                         components live in two arrays (ImpGen/GPU/Base.hs:769-842):
+ *                         up to 8192 bins in sub-histograms in LDS, more in place
+ *                         in global memory (SegHist.hs:377-467);
  *                         H <= fa_hist_argmax_max_bins(); workspace of
  *                         fa_hist_argmax_workspace_bytes(H) bytes, contents irrelevant. */
 int fa_reduce_argmax_i32(fa_stream_t stream, const int32_t *xs, int64_t n, int32_t *out2,

@@ -50,17 +50,22 @@ constexpr uint32_t ST_P = 2;  // inclusive prefix up to the end of the tile
 
 // Scratch: a header, then one descriptor per tile.  Header: 32-bit word 1
 // counts the blocks that have left, word 16 is the epoch word of
-// fa_segscan_static, and every 64th word (256 bytes apart, so that they sit in
-// different memory channels) is a ticket counter: same-address atomics are
-// performed one at a time, about 12 ns each on MI355X, and a channel that does
-// little else slows every stream that crosses it.  Counter c hands out the
-// tiles congruent to c modulo the number of counters in use; a block draws
-// from counter (block index mod that number).  Every tile is handed out as
-// long as at least that many blocks get to run at the same time, which the
-// number (8) is small enough for: a block occupies one CU.
+// fa_segscan_static, word 512 counts the blocks that have arrived, and every
+// 64th word up to there (256 bytes apart, so that they sit in different memory
+// channels) is a ticket counter: same-address atomics are performed one at a
+// time, about 12 ns each on MI355X, and a channel that does little else slows
+// every stream that crosses it.  Counter c hands out the tiles congruent to c
+// modulo the number of counters in use.  A block draws from the counter its
+// arrival number selects (arrival number mod the number of counters), not
+// from one its block index selects: whichever blocks the hardware starts
+// first, the first eight of them cover all eight counters, so every tile is
+// handed out as long as eight blocks (or the whole grid, if it is smaller)
+// can be resident at the same time -- on any CUs, of any die.  Blocks that
+// start later join the counters in turn.
 constexpr size_t SCAN_HEADER_BYTES = 8192;
 constexpr int SCAN_MAX_COUNTERS = 8;
 constexpr int SCAN_COUNTER_STRIDE = 64;  // in 32-bit words
+constexpr int SCAN_ARRIVAL_WORD = SCAN_MAX_COUNTERS * SCAN_COUNTER_STRIDE;
 constexpr size_t SCAN_DESC_BYTES = 16;
 
 __device__ __forceinline__ uint32_t desc_meta(uint32_t epoch, uint32_t flag, uint32_t status) {
@@ -186,12 +191,12 @@ __device__ __forceinline__ void ss_load_to_lds(const void *gaddr, uint32_t lds_a
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(
                      __builtin_amdgcn_readfirstlane(lds_addr)),
                  "v"(gaddr)
-                 : "memory");
+                 : "memory", "m0");
   else
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(
                      __builtin_amdgcn_readfirstlane(lds_addr)),
                  "v"(gaddr)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // Waits until at most `younger` vector memory operations of this wave are
@@ -279,13 +284,15 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
 
   // Ticket v of counter c is tile v * counters + c.
   const uint32_t counters = gridDim.x < (unsigned)SCAN_MAX_COUNTERS ? gridDim.x : (unsigned)SCAN_MAX_COUNTERS;
-  const uint32_t my_counter = blockIdx.x % counters;
-  uint32_t *ticket = header + my_counter * SCAN_COUNTER_STRIDE;
   const int tid = threadIdx.x;
   const int lane = lane_id();
   const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)ss_lds;
 
+  // The protocol wave takes the block's arrival number first of all: its round
+  // trip runs while the rest of the block sets up.
+  uint32_t arrival = 0u;
+  if (tid == SS_DATA_THREADS) arrival = atomicAdd(header + SCAN_ARRIVAL_WORD, 1u);
   if (tid < SS_WAVES) s_scanned[tid] = 0u;
   if (tid == 0) {
     s_tiles_known = 0u;
@@ -302,6 +309,8 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
 
   if (wave == SS_WAVES) {
     // ------------------------------------------------------------ protocol wave
+    const uint32_t my_counter = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrival) % counters;
+    uint32_t *ticket = header + my_counter * SCAN_COUNTER_STRIDE;
     // Exclusive prefix of `tile` (> 0): folds the descriptors of the tiles
     // before it, newest window first, back to one that has published its prefix
     // (or, in a segmented scan, contains a segment start).
@@ -447,6 +456,7 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
       const uint32_t left = atomicAdd(header + 1, 1u);
       if (left == gridDim.x - 1) {
         st_relaxed_u32(header + 1, 0u);
+        st_relaxed_u32(header + SCAN_ARRIVAL_WORD, 0u);
         for (uint32_t c = 0; c < counters; c++) st_relaxed_u32(header + c * SCAN_COUNTER_STRIDE, 0u);
       }
     }
@@ -1001,20 +1011,53 @@ __global__ __launch_bounds__(HL_BLOCK) void hist_locked_kernel(const I *__restri
   }
 }
 
+// More bins than a block's LDS holds: every update locks its bin in the
+// destination itself (the reference's pass over global memory with locks,
+// SegHist.hs:377-467 with Base.hs:769-842; one sub-histogram, hist_M = 1).
+template <class Tin, class A, class B, class P, class Pre, class Op, class I>
+__global__ __launch_bounds__(HL_BLOCK) void hist_locked_global_kernel(const I *__restrict__ is,
+                                                                      const Tin *__restrict__ xs,
+                                                                      int64_t n, A *dest_a, B *dest_b,
+                                                                      uint32_t *locks, int64_t H) {
+  const int64_t stride = (int64_t)gridDim.x * HL_BLOCK;
+  for (int64_t i = (int64_t)blockIdx.x * HL_BLOCK + threadIdx.x; i < n; i += stride) {
+    const int64_t bin = (int64_t)is[i];
+    if ((uint64_t)bin >= (uint64_t)H) continue;  // out of range: ignored
+    const P mine = Pre::apply(xs[i], i);
+    hl_with_lock<P, Op>(&locks[bin], [&] {
+      P cur;
+      cur.a = __hip_atomic_load(dest_a + bin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      cur.b = __hip_atomic_load(dest_b + bin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const P r = Op::apply(cur, mine);
+      __hip_atomic_store(dest_a + bin, r.a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dest_b + bin, r.b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    });
+  }
+}
+
 // dest_a, dest_b: H bins each, holding the values to combine with (as
 // reduce_by_index takes them); locks: H 32-bit words, all zero, zero again
-// afterwards.  H <= HL_MAX_BINS.
+// afterwards.  Up to HL_MAX_BINS bins are accumulated per block in LDS; more
+// are updated in place under the locks.
 template <class Tin, class A, class B, class P, class Pre, class Op, class I>
 static int launch_hist_locked(hipStream_t s, const I *is, const Tin *xs, int64_t n, A *dest_a,
                               B *dest_b, uint32_t *locks, int64_t H) {
   static_assert(Op::commutative, "reduce_by_index needs a commutative operator");
-  if (n < 0 || H < 0 || H > HL_MAX_BINS) return FA_EINVAL;
+  if (n < 0 || H < 0) return FA_EINVAL;
   if (H == 0 || n == 0) return 0;
   if (is == nullptr || xs == nullptr || dest_a == nullptr || dest_b == nullptr || locks == nullptr)
     return FA_EINVAL;
   int dev = 0, cus = NUM_CUS_HINT;
   if (hipGetDevice(&dev) == hipSuccess)
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (H > HL_MAX_BINS) {
+    const int64_t want = ceil_div(n, (int64_t)HL_BLOCK * 4);
+    const int64_t most = (int64_t)cus * 8;
+    const int grid = (int)(want < 1 ? 1 : (want > most ? most : want));
+    hipLaunchKernelGGL((hist_locked_global_kernel<Tin, A, B, P, Pre, Op, I>), dim3(grid), dim3(HL_BLOCK),
+                       0, s, is, xs, n, dest_a, dest_b, locks, H);
+    return launch_status();
+  }
   const size_t lds = (size_t)H * (sizeof(A) + sizeof(B) + 4);
   const int64_t want = ceil_div(n, (int64_t)HL_BLOCK * 8);
   const int grid = (int)(want < 1 ? 1 : (want > cus ? cus : want));

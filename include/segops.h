@@ -31,6 +31,9 @@
  *                                   -- tests/hist/segmented.fut
  *   entry rbi_OP_T (dest: *[]T) (is: []i32) (vs: []T) : []T =
  *     reduce_by_index dest OP NE (map i64.i32 is) vs
+ *   entry hist_OP_T_i64 (k: i64) (is: []i64) (vs: []T) : [k]T = hist OP NE k is vs
+ *   entry rbi_OP_T_i64 (dest: *[]T) (is: []i64) (vs: []T) : []T =
+ *     reduce_by_index dest OP NE is vs           -- the index type of the prelude
  *   entry rbi_vec_OP_T [m] (dest: *[][m]T) (is: []i64) (vss: [][m]T) : [][m]T =
  *     reduce_by_index dest (map2 OP) (replicate m NE) is vss
  *   entry rbi_2d_OP_T (dest: *[][]T) (is: []i64) (js: []i64) (vs: []T) : [][]T =
@@ -49,7 +52,7 @@
  * OP in {add, max, min}; NE = 0, T.lowest, T.highest; T in {i32, i64, f32, f64};
  * for T in {i32, i64} also OP in {and, or, xor} with NE = -1, 0, 0
  * (tests/hist/{and,or,xor}.fut).
- * hist_OP_T and rbi_OP_T exist in addition for T in {i8, u8, i16, u16, u32,
+ * hist_OP_T, rbi_OP_T and their _i64 forms exist in addition for T in {i8, u8, i16, u16, u32,
  * u64} with all six operators and for f16 with add, max, min: the element types
  * whose updates the reference emulates with compare-and-swap, and the unsigned
  * comparisons (tests/hist/{i8,i16,and8,and16,max8,max16,max,f16}.fut ...).
@@ -280,15 +283,18 @@ FUTHARK_DECLARE_ARRAY_3D(u16, uint16_t)
   FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)
 
 #define FUTHARK_DECLARE_HIST_ENTRIES(OP, T, CT)                                               \
-  int futhark_entry_hist_##OP##_##T(struct futhark_context *ctx,                              \
-                                    struct futhark_##T##_1d **out0, const int64_t in0,        \
-                                    const struct futhark_i32_1d *in1,                         \
-                                    const struct futhark_##T##_1d *in2);                      \
-  int futhark_entry_rbi_##OP##_##T(struct futhark_context *ctx,                               \
-                                   struct futhark_##T##_1d **out0,                            \
-                                   const struct futhark_##T##_1d *in0,                        \
-                                   const struct futhark_i32_1d *in1,                          \
-                                   const struct futhark_##T##_1d *in2);
+  FUTHARK_DECLARE_HIST_ENTRIES_IX(OP, T, CT, , i32)                                           \
+  FUTHARK_DECLARE_HIST_ENTRIES_IX(OP, T, CT, _i64, i64)
+#define FUTHARK_DECLARE_HIST_ENTRIES_IX(OP, T, CT, SUFFIX, IT)                                \
+  int futhark_entry_hist_##OP##_##T##SUFFIX(struct futhark_context *ctx,                      \
+                                            struct futhark_##T##_1d **out0, const int64_t in0, \
+                                            const struct futhark_##IT##_1d *in1,              \
+                                            const struct futhark_##T##_1d *in2);              \
+  int futhark_entry_rbi_##OP##_##T##SUFFIX(struct futhark_context *ctx,                       \
+                                           struct futhark_##T##_1d **out0,                    \
+                                           const struct futhark_##T##_1d *in0,                \
+                                           const struct futhark_##IT##_1d *in1,               \
+                                           const struct futhark_##T##_1d *in2);
 
 #define FUTHARK_DECLARE_FOR_TYPE(T, CT) FUTHARK_FOR_EACH_OP(FUTHARK_DECLARE_SEGOP_ENTRIES, T, CT)
 FUTHARK_FOR_EACH_NUM_TYPE(FUTHARK_DECLARE_FOR_TYPE)

@@ -407,3 +407,66 @@ def mc_rbi_add_i32(dest, is_, vs, threads: int | None = None):
     fn.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
     fn(_p(dest), dest.size, _p(is_), _p(vs), is_.size, threads or mc_threads())
     return dest
+
+
+def mc_rbi_f32(op: str, dest, is_, vs, threads: int | None = None):
+    dest = _arr(dest, np.float32).copy()
+    is_, vs = _arr(is_, np.int32), _arr(vs, np.float32)
+    fn = getattr(lib(), f"mc_rbi_{op}_f32")
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+    fn(_p(dest), dest.size, _p(is_), _p(vs), is_.size, threads or mc_threads())
+    return dest
+
+
+def mc_segred_add_f32(offsets, lens, xs, threads: int | None = None, tmp=None):
+    """tmp: (u8[n], f32[n]) scratch a caller that times this may keep between calls."""
+    xs, offsets, lens = _arr(xs, np.float32), _arr(offsets, np.int64), _arr(lens, np.int64)
+    out = np.empty(offsets.size, np.float32)
+    ft, st = tmp if tmp is not None else (np.empty(xs.size, np.uint8), np.empty(xs.size, np.float32))
+    fn = lib().mc_segred_add_f32
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p,
+                   C.c_void_p, C.c_int]
+    fn(_p(offsets), _p(lens), offsets.size, _p(xs), xs.size, _p(out), _p(ft), _p(st),
+       threads or mc_threads())
+    return out
+
+
+def mc_transpose_f32(B, threads: int | None = None):
+    B = _arr(B, np.float32)
+    b, K, N = B.shape
+    Bt = np.empty((b, N, K), np.float32)
+    fn = lib().mc_transpose_f32
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int]
+    fn(_p(B), _p(Bt), b, K, N, threads or mc_threads())
+    return Bt
+
+
+def mc_bmm_rows_f32(A, Bt, C_out, row_lo: int, row_hi: int, threads: int | None = None):
+    """Rows [row_lo, row_hi) of the flattened [b*M] rows of C = A x B, with Bt = mc_transpose_f32(B)."""
+    A, Bt = _arr(A, np.float32), _arr(Bt, np.float32)
+    b, M, K = A.shape
+    N = Bt.shape[1]
+    assert C_out.shape == (b, M, N) and C_out.dtype == np.float32 and C_out.flags.c_contiguous
+    fn = lib().mc_bmm_rows_f32
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                   C.c_int64, C.c_int]
+    fn(_p(A), _p(Bt), _p(C_out), M, N, K, row_lo, row_hi, threads or mc_threads())
+    return C_out
+
+
+def mc_radix_sort(keys, vals=None, threads: int | None = None):
+    keys = np.array(keys, copy=True)
+    assert keys.dtype in (np.uint32, np.uint64)
+    vals = None if vals is None else np.array(vals, dtype=np.int32, copy=True)
+    kt = np.empty_like(keys)
+    vt = None if vals is None else np.empty_like(vals)
+    fn = lib().mc_radix_sort
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int, C.c_void_p, C.c_void_p, C.c_int]
+    fn(_p(keys), None if vals is None else _p(vals), keys.size, keys.itemsize, _p(kt),
+       None if vt is None else _p(vt), threads or mc_threads())
+    return keys if vals is None else (keys, vals)

@@ -14,6 +14,8 @@
  *   hist    one private sub-histogram per task plus a column reduce when
  *           tasks*H <= n, otherwise atomic updates of the shared histogram
  *           (Multicore/SegHist.hs:50-71,103-151,180-320)
+ *   segmented reduce over irregular segments, matmul and radix sort: the
+ *           compositions stated at each function below
  * Work is split statically into one task per thread, as the scheduler does for
  * a parallel loop without nested parallelism (rts/c/scheduler.h:788-968).
  */
@@ -233,4 +235,164 @@ void mc_rbi_add_i32(int32_t *dest, int64_t H, const int32_t *is, const int32_t *
     par_loop(threads, col_task_i32, &c);
     free(a.subs);
   }
+}
+
+/* f32 histograms: the same schedule with the float operator (sub-histograms
+ * start at the neutral element; the column reduce folds them into dest). */
+#define MC_HIST_F32(NAME, NE, OPF)                                                               \
+  struct histf_##NAME { const int32_t *is; const float *vs; int64_t n, H; float *subs; float *dest; }; \
+  static void histf_task_##NAME(int tid, int nt, void *p) {                                      \
+    struct histf_##NAME *a = (struct histf_##NAME *)p;                                           \
+    int64_t lo, hi;                                                                              \
+    split(a->n, tid, nt, &lo, &hi);                                                              \
+    float *sub = a->subs + (int64_t)tid * a->H;                                                  \
+    for (int64_t b = 0; b < a->H; b++) sub[b] = (NE);                                            \
+    for (int64_t i = lo; i < hi; i++) {                                                          \
+      const int64_t b = a->is[i];                                                                \
+      if (b >= 0 && b < a->H) sub[b] = OPF(sub[b], a->vs[i]);                                    \
+    }                                                                                            \
+  }                                                                                              \
+  static void colf_task_##NAME(int tid, int nt, void *p) {                                       \
+    struct histf_##NAME *a = (struct histf_##NAME *)p;                                           \
+    int64_t lo, hi;                                                                              \
+    split(a->H, tid, nt, &lo, &hi);                                                              \
+    for (int64_t b = lo; b < hi; b++) {                                                          \
+      float acc = a->dest[b];                                                                    \
+      for (int t = 0; t < nt; t++) acc = OPF(acc, a->subs[(int64_t)t * a->H + b]);               \
+      a->dest[b] = acc;                                                                          \
+    }                                                                                            \
+  }                                                                                              \
+  void mc_rbi_##NAME##_f32(float *dest, int64_t H, const int32_t *is, const float *vs,           \
+                           int64_t n, int threads) {                                             \
+    struct histf_##NAME a = {is, vs, n, H, NULL, dest};                                          \
+    a.subs = (float *)malloc((size_t)threads * (size_t)(H > 0 ? H : 1) * sizeof(float));         \
+    par_loop(threads, histf_task_##NAME, &a);                                                    \
+    par_loop(threads, colf_task_##NAME, &a);                                                     \
+    free(a.subs);                                                                                \
+  }
+MC_HIST_F32(add, 0.0f, ADD_F)
+MC_HIST_F32(max, -INFINITY, fmaxf)
+
+/* ------------------------------------------------- irregular segmented reduce
+ * What flattening makes of it (Pass/Flatten/Builtins.hs:582-602): a segmented
+ * scan with flags written from the offsets, then one read per segment of the
+ * scanned value at its last element (the neutral element for an empty one). */
+struct gather_f32 { const int64_t *offsets, *lens; int64_t m; const float *scanned; float *out; };
+static void gather_task_f32(int tid, int nt, void *p) {
+  struct gather_f32 *a = (struct gather_f32 *)p;
+  int64_t lo, hi;
+  split(a->m, tid, nt, &lo, &hi);
+  for (int64_t i = lo; i < hi; i++)
+    a->out[i] = a->lens[i] == 0 ? 0.0f : a->scanned[a->offsets[i] + a->lens[i] - 1];
+}
+void mc_segred_add_f32(const int64_t *offsets, const int64_t *lens, int64_t m, const float *xs,
+                       int64_t n, float *out, uint8_t *flags_tmp, float *scan_tmp, int threads) {
+  memset(flags_tmp, 0, (size_t)n);
+  for (int64_t i = 0; i < m; i++)
+    if (lens[i] > 0) flags_tmp[offsets[i]] = 1;
+  mc_segscan_f32(flags_tmp, xs, n, scan_tmp, 0, threads);
+  struct gather_f32 g = {offsets, lens, m, scan_tmp, out};
+  par_loop(threads, gather_task_f32, &g);
+}
+
+/* ------------------------------------------------------------------ matmul
+ * C[b][i][j] = sum_k A[b][i][k] * B[b][k][j] as the nested map-reduce of
+ * tests/reg-tiling/mmm.fut:17-21 comes out of the multicore backend: the outer
+ * map over rows is the parallel loop (rows [row_lo, row_hi) of the flattened
+ * b*M rows, so that a bounded sample can be timed), the inner map and the
+ * reduction are sequential loops; `transpose B` is materialised once so that a
+ * column is a contiguous row of the copy (Bt, b*N*K floats, caller's memory). */
+struct mm_f32 { const float *A, *Bt; float *C; int64_t M, N, K, row_lo, row_hi; };
+static void mm_task_f32(int tid, int nt, void *p) {
+  struct mm_f32 *a = (struct mm_f32 *)p;
+  int64_t lo, hi;
+  split(a->row_hi - a->row_lo, tid, nt, &lo, &hi);
+  for (int64_t r = a->row_lo + lo; r < a->row_lo + hi; r++) {
+    const int64_t b = r / a->M;
+    const float *arow = a->A + r * a->K;
+    const float *bt = a->Bt + b * a->N * a->K;
+    float *crow = a->C + r * a->N;
+    for (int64_t j = 0; j < a->N; j++) {
+      const float *bcol = bt + j * a->K;
+      float acc = 0.0f;
+      for (int64_t k = 0; k < a->K; k++) acc += arow[k] * bcol[k];
+      crow[j] = acc;
+    }
+  }
+}
+struct tr_f32 { const float *B; float *Bt; int64_t batch, K, N; };
+static void tr_task_f32(int tid, int nt, void *p) {
+  struct tr_f32 *a = (struct tr_f32 *)p;
+  int64_t lo, hi;
+  split(a->batch * a->N, tid, nt, &lo, &hi);
+  for (int64_t r = lo; r < hi; r++) {
+    const int64_t b = r / a->N, j = r % a->N;
+    for (int64_t k = 0; k < a->K; k++) a->Bt[r * a->K + k] = a->B[(b * a->K + k) * a->N + j];
+  }
+}
+void mc_transpose_f32(const float *B, float *Bt, int64_t batch, int64_t K, int64_t N, int threads) {
+  struct tr_f32 t = {B, Bt, batch, K, N};
+  par_loop(threads, tr_task_f32, &t);
+}
+void mc_bmm_rows_f32(const float *A, const float *Bt, float *C, int64_t M, int64_t N, int64_t K,
+                     int64_t row_lo, int64_t row_hi, int threads) {
+  struct mm_f32 a = {A, Bt, C, M, N, K, row_lo, row_hi};
+  par_loop(threads, mm_task_f32, &a);
+}
+
+/* -------------------------------------------------------------- radix sort
+ * The composition the sort is made of, per 8-bit digit from the least
+ * significant one: a histogram of the digit per task, an exclusive scan of the
+ * [digit][task] counts, and a scatter in which every task moves its stretch in
+ * order (stable).  Keys of `kb` bytes (4 or 8) as 64-bit values; vals may be
+ * NULL.  tmp buffers are the caller's (n keys, n vals). */
+struct rs_arg {
+  const uint64_t *k8; const uint32_t *k4; const int32_t *v;
+  uint64_t *ok8; uint32_t *ok4; int32_t *ov;
+  int64_t n; int shift; int64_t *counts; /* [tasks][256] */
+};
+static inline unsigned rs_digit(const struct rs_arg *a, int64_t i) {
+  return (unsigned)(((a->k8 ? a->k8[i] : (uint64_t)a->k4[i]) >> a->shift) & 255u);
+}
+static void rs_count_task(int tid, int nt, void *p) {
+  struct rs_arg *a = (struct rs_arg *)p;
+  int64_t lo, hi;
+  split(a->n, tid, nt, &lo, &hi);
+  int64_t *c = a->counts + (int64_t)tid * 256;
+  memset(c, 0, 256 * sizeof(int64_t));
+  for (int64_t i = lo; i < hi; i++) c[rs_digit(a, i)]++;
+}
+static void rs_scatter_task(int tid, int nt, void *p) {
+  struct rs_arg *a = (struct rs_arg *)p;
+  int64_t lo, hi;
+  split(a->n, tid, nt, &lo, &hi);
+  int64_t *c = a->counts + (int64_t)tid * 256; /* now: first destination per digit */
+  for (int64_t i = lo; i < hi; i++) {
+    const int64_t d = c[rs_digit(a, i)]++;
+    if (a->k8) a->ok8[d] = a->k8[i]; else a->ok4[d] = a->k4[i];
+    if (a->v) a->ov[d] = a->v[i];
+  }
+}
+void mc_radix_sort(void *keys, int32_t *vals, int64_t n, int kb, void *keys_tmp, int32_t *vals_tmp,
+                   int threads) {
+  int64_t *counts = (int64_t *)malloc(sizeof(int64_t) * 256 * (size_t)threads);
+  void *src = keys, *dst = keys_tmp;
+  int32_t *vsrc = vals, *vdst = vals_tmp;
+  for (int pass = 0; pass < kb; pass++) {
+    struct rs_arg a = {kb == 8 ? (const uint64_t *)src : NULL, kb == 4 ? (const uint32_t *)src : NULL,
+                       vsrc, (uint64_t *)dst, (uint32_t *)dst, vdst, n, 8 * pass, counts};
+    par_loop(threads, rs_count_task, &a);
+    int64_t run = 0; /* exclusive scan in (digit, task) order */
+    for (int d = 0; d < 256; d++)
+      for (int t = 0; t < threads; t++) {
+        const int64_t c = counts[(int64_t)t * 256 + d];
+        counts[(int64_t)t * 256 + d] = run;
+        run += c;
+      }
+    par_loop(threads, rs_scatter_task, &a);
+    void *tk = src; src = dst; dst = tk;
+    int32_t *tv = vsrc; vsrc = vdst; vdst = tv;
+  }
+  /* kb passes: an even number, so the result is back in `keys` / `vals` */
+  free(counts);
 }

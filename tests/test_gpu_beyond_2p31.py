@@ -54,3 +54,37 @@ def test_reduce_and_scans_over_more_than_2p31_elements(ctx):
     # sum of xs[start..idx] = S(idx) - S(start - 1), S = the unsegmented scan
     before = np.where(start > 0, P[(start - 1) % 7], 0)
     assert np.array_equal(got[idx], P[idx % 7] - before)
+
+
+def test_transpose_with_more_blocks_than_one_launch_holds(ctx):
+    """[2][2^32 + 4099] bytes -> [2^32 + 4099][2]: the strips of 256 columns are more blocks than a
+    launch of 256-thread blocks may have along x (2^32 threads), so the library sends them in
+    pieces.  x[r][c] = (3 c + 7 r) mod 251, checked block by block on the host."""
+    import ctypes as C
+    from futhark_amd import lib_path
+    k = C.CDLL(str(lib_path("libfuthark_amd_kernels.so")))
+    k.fa_map_transpose.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
+                                   C.c_int64]
+    cols = (1 << 32) + 4099
+    period = 251 * (1 << 14)
+    base = ((np.arange(period, dtype=np.int64) * 3) % 251).astype(np.uint8)
+
+    def row(r, lo, hi):  # x[r][lo:hi] for lo a multiple of the period
+        return ((base[: hi - lo].astype(np.int16) + 7 * r) % 251).astype(np.uint8)
+
+    x = np.empty(2 * cols, np.uint8)
+    for r in range(2):
+        for lo in range(0, cols, period):
+            hi = min(lo + period, cols)
+            x[r * cols + lo: r * cols + hi] = row(r, lo, hi)
+    s = ctx.new("u8_1d", x)
+    del x
+    d = ctx.new("u8_1d", np.zeros(2 * cols, np.uint8))
+    print("fa_map_transpose u8 batch=1 rows=2 cols=2^32+4099", flush=True)
+    assert k.fa_map_transpose(ctx.stream, 1, d.device_ptr, s.device_ptr, 1, 2, cols) == 0
+    got = d.values().reshape(cols, 2)
+    s.free(); d.free()
+    for lo in range(0, cols, period):
+        hi = min(lo + period, cols)
+        for r in range(2):
+            assert np.array_equal(got[lo:hi, r], row(r, lo, hi)), (r, lo)

@@ -69,8 +69,10 @@ def test_maps_fused_into_reduce_and_scan(ctx):
 
 def test_hist_with_a_tuple_operator_locks_its_bins(ctx):
     rng = np.random.default_rng(4)
+    # up to 8192 bins a block keeps its own in LDS; beyond, every update locks its bin in the
+    # destination (the reference's pass over global memory with locks, SegHist.hs:377-467)
     for n, H in [(0, 5), (1, 1), (1000, 7), (100003, 256), ((1 << 22) + 5, 256), ((1 << 22) + 5, 8192),
-                 (300000, 1), (5, 0)]:
+                 (300000, 1), (5, 0), (200003, 8193), ((1 << 21) + 3, 100000), (500000, 3_000_000)]:
         xs = rng.integers(-50, 50, n).astype(np.int32)           # ties in every bin
         is_ = dg.hist_indices(24, n, max(H, 1), "zipf") if n else np.zeros(0, np.int32)
         out = ctx.call("hist_argmax_i32", ["i32_2d"], H, ctx.new("i32_1d", is_), ctx.new("i32_1d", xs))
@@ -78,7 +80,7 @@ def test_hist_with_a_tuple_operator_locks_its_bins(ctx):
         assert np.array_equal(out.values(), oracle.hist_argmax_i32(H, is_, xs)), (n, H)
         out.free()
     with pytest.raises(FutharkError):
-        ctx.call("hist_argmax_i32", ["i32_2d"], 8193, ctx.new("i32_1d", np.zeros(4, np.int32)),
+        ctx.call("hist_argmax_i32", ["i32_2d"], -1, ctx.new("i32_1d", np.zeros(4, np.int32)),
                  ctx.new("i32_1d", np.zeros(4, np.int32)))
 
 

@@ -127,3 +127,22 @@ def test_padded_operands_with_more_than_65535_rows(ctx):
     Ain, Bin, Af, Bf, kind = _inputs("f32", b, M, N, K, 69)
     got = ctx.call("bmm_f32", ["f32_3d"], ctx.new(kind, Ain), ctx.new(kind, Bin)).values()
     _check(got, Af, Bf, 1e-5)
+
+
+def test_more_tile_rows_than_a_launch_grid_holds(ctx):
+    """M / 128 above 65535 tile rows (f16, one matrix): the product goes out in bands of rows.
+    The rows of A repeat with period 384, so every row of C repeats too: the first period is
+    checked against the oracle and the rest against the first period."""
+    M, N, K, period = 65537 * 128, 128, 64, 384
+    Ain, Bin, Af, Bf, kind = _inputs("f16", 1, period, N, K, 70)
+    reps = M // period + 1
+    A_all = np.tile(Ain[0], (reps, 1))[:M][None]
+    out = ctx.call("bmm_f16", ["f32_3d"], ctx.new(kind, np.ascontiguousarray(A_all)), ctx.new(kind, Bin))
+    got = out.values()[0]
+    out.free()
+    assert got.shape == (M, N)
+    _check(got[:period][None], Af, Bf, 1e-2)
+    first = got[:period]
+    whole = (M // period) * period
+    assert np.array_equal(got[:whole].reshape(-1, period, N), np.broadcast_to(first, (M // period, period, N)))
+    assert np.array_equal(got[whole:], first[: M - whole])

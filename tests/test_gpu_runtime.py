@@ -175,3 +175,39 @@ def test_tuning_parameters_select_other_code_paths_with_the_same_results(segops_
             assert len(ev) == 2 and all(e["details"]["padded"] is padded for e in ev)
     with pytest.raises(KeyError):
         Context(segops_lib, tuning={"segops.no_such_parameter": 1})
+
+
+def test_scalar_results_arrive_at_the_synchronisation(segops_lib):
+    """A scalar result may be used after futhark_context_sync (docs/c-api.rst:578-581).  Entry
+    points that return one do not wait for the device: many calls are queued back to back, each
+    with its own destination, and one synchronisation delivers all of them - also more calls than
+    the runtime has pinned slots for (64), which it must drain by itself on the way."""
+    import ctypes as C
+    import oracle
+    from futhark_amd import datagen as dg
+    with Context(segops_lib) as c:
+        L = c.L
+        arrays, want = [], []
+        for i in range(150):
+            xs = dg.uniform_int(100 + i, 1000 + 37 * i, -1000, 1000, np.int32)
+            arrays.append(c.new("i32_1d", xs))
+            want.append(int(oracle.reduce("add", "i32", xs)))
+        outs = (C.c_int32 * len(arrays))(*([-1] * len(arrays)))
+        for i, a in enumerate(arrays):
+            rc = L.futhark_entry_reduce_add_i32(c.ptr, C.byref(outs, 4 * i), a.ptr)
+            assert rc == 0
+        c.sync()
+        assert list(outs) == want
+        # the same destination twice before one synchronisation: the later call wins
+        one = C.c_int32(-1)
+        assert L.futhark_entry_reduce_add_i32(c.ptr, C.byref(one), arrays[3].ptr) == 0
+        assert L.futhark_entry_reduce_add_i32(c.ptr, C.byref(one), arrays[4].ptr) == 0
+        c.sync()
+        assert one.value == want[4]
+        f = c.new("f32_1d", np.arange(1, 5, dtype=np.float32))
+        sq = C.c_float(-1.0)
+        assert L.futhark_entry_sumsq_f32(c.ptr, C.byref(sq), f.ptr) == 0
+        c.sync()
+        assert sq.value == 30.0
+        for a in arrays + [f]:
+            a.free()

@@ -388,3 +388,47 @@ def test_hist_with_2d_indices_goldens_and_shapes(ctx, goldens):
     assert int(out.values().sum(dtype=np.int64)) % 2**32 == (k * (k - 1) // 2) % 2**32  # bins wrap
     for h in (out, d, i, j, v):
         h.free()
+
+
+@pytest.mark.parametrize("t,op", [("i32", "add"), ("i64", "max"), ("f32", "add"), ("f32", "max"), ("f64", "min")])
+def test_i64_indices_small_and_ragged(ctx, t, op):
+    """hist_OP_T_i64 / rbi_OP_T_i64: the []i64 indices `hist` and `reduce_by_index` are defined
+    over (prelude/soacs.fut:132-146), with indices far outside the bins that a 32-bit view would
+    fold back into range (2^32 + 3 must be ignored, not counted in bin 3)."""
+    for n, H in [(0, 5), (5, 0), (100, 7), (4097, 256), (300001, 32769), (150000, 100001),
+                 (100000, 200000), (400000, 2_000_000)]:
+        is_ = dg.hist_indices(40, n, max(H, 1), "uniform", 3).astype(np.int64)
+        if n > 50:
+            is_[::17] += np.int64(1) << 32          # out of range only as 64-bit numbers
+            is_[5::29] = -(np.int64(1) << 40) + 2
+        vs = _vals(t, n, 41)
+        i, v = ctx.new("i64_1d", is_), ctx.new(f"{t}_1d", vs)
+        ok = (is_ >= 0) & (is_ < H)
+        narrow = np.where(ok, is_, -1).astype(np.int32)   # the oracle takes 32-bit indices
+        out = ctx.call(f"hist_{op}_{t}_i64", [f"{t}_1d"], H, i, v)
+        got = out.values()
+        assert got.shape == (H,)
+        acc = oracle.hist(op, t, H, narrow, vs, "f64acc") if (op, t) == ("add", "f32") else None
+        _check(t, op, got, oracle.hist(op, t, H, narrow, vs), acc)
+        out.free()
+        dest = _vals(t, H, 43)
+        d = ctx.new(f"{t}_1d", dest)
+        out = ctx.call(f"rbi_{op}_{t}_i64", [f"{t}_1d"], d, i, v)
+        acc = oracle.rbi(op, t, dest, narrow, vs, "f64acc") if (op, t) == ("add", "f32") else None
+        _check(t, op, out.values(), oracle.rbi(op, t, dest, narrow, vs), acc)
+        for h in (i, v, d, out):
+            h.free()
+
+
+@pytest.mark.parametrize("H", [65536, 1 << 22])
+def test_config3_full_size_i64_indices(ctx, H):
+    """The i32 (+) histogram of the configuration at 2^27 with its indices widened to i64."""
+    n = 1 << 27
+    is32 = dg.hist_indices(48, n, H, "uniform")
+    vs = dg.uniform_int(49, n, -1000, 1000)
+    i, v = ctx.new("i64_1d", is32.astype(np.int64)), ctx.new("i32_1d", vs)
+    out = ctx.call("hist_add_i32_i64", ["i32_1d"], H, i, v)
+    got = out.values()
+    assert np.array_equal(got, oracle.hist("add", "i32", H, is32, vs))
+    for h in (i, v, out):
+        h.free()

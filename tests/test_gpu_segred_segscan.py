@@ -317,14 +317,29 @@ def test_scan_of_rows(ctx, t, op):
         out.free(); a.free()
 
 
+FA_DTYPE = {"i32": 0, "i64": 1, "f32": 2, "f64": 3}
+
+
+def _tile_elems(t):
+    """Elements per look-back tile, as the kernel library states it."""
+    import ctypes as C
+    from futhark_amd import lib_path
+    k = C.CDLL(str(lib_path("libfuthark_amd_kernels.so")))
+    k.fa_segscan_tile_elems.restype = C.c_int64
+    k.fa_segscan_tile_elems.argtypes = [C.c_int]
+    tile = int(k.fa_segscan_tile_elems(FA_DTYPE[t]))
+    assert tile > 0 and tile * NP[t]().itemsize == int(k.fa_segscan_tile_elems(FA_DTYPE["i32"])) * 4
+    return tile
+
+
 @pytest.mark.parametrize("t", ["i32", "i64"])
 def test_segscan_long_look_back_chains(ctx, t):
     """Flag patterns chosen for the look-back: segment starts hundreds of tiles apart (chains that
     cross several 64-tile windows before they meet a start), starts exactly on tile boundaries and
-    on their neighbours, and runs of tiles with and without starts in turn.  2^23 elements are
-    256 tiles of 4-byte and 512 tiles of 8-byte elements."""
-    n = 1 << 23
-    tile = 32768 if t == "i32" else 8192
+    on their neighbours, and runs of tiles with and without starts in turn.  The tile size is the
+    kernel's own; 600 tiles and a ragged end."""
+    tile = _tile_elems(t)
+    n = 600 * tile + 4099
     xs = _data(t, n, 21)
     a = ctx.new(f"{t}_1d", xs)
     patterns = {
@@ -353,7 +368,7 @@ def test_scan_with_a_non_commutative_operator(ctx):
     look-back over tiles - must keep the operands in order, or some element differs.  Sizes from
     one element to many tiles, ragged ends, segment starts dense and hundreds of tiles apart."""
     rng = np.random.default_rng(17)
-    tile = 1024 * 8 * 2
+    tile = _tile_elems("i64")  # an affine map is a pair of i32: eight bytes
     for n in [0, 1, 2, 63, 64, 65, 4097, tile - 1, tile, tile + 1, 5 * tile + 3, 700 * tile + 11]:
         abs_ = rng.integers(-2**31, 2**31, (n, 2), dtype=np.int64).astype(np.int32)
         a = ctx.new("i32_2d", abs_)
@@ -376,6 +391,48 @@ def test_scan_with_a_non_commutative_operator(ctx):
     with pytest.raises(Exception, match="invalid sizes"):
         ctx.call("scan_compose_i32", ["i32_2d"], bad)
     bad.free()
+
+
+@pytest.mark.parametrize("t", ["i32", "i64", "f32"])
+def test_scans_of_whole_tiles_and_their_neighbours(ctx, t):
+    """n = k tiles exactly and one element either side, for the plain scan, the scan with flags
+    and the scan of rows: the last tile is whole, one element long, or one element short, and
+    with k = 257 and 513 the persistent blocks take more than one and more than two tiles each."""
+    tile = _tile_elems(t)
+    for k in (1, 2, 3, 257, 513):
+        for d in (-1, 0, 1):
+            n = k * tile + d
+            xs = _data(t, n, 40 + k)
+            a = ctx.new(f"{t}_1d", xs)
+            for excl in (False, True):
+                out = ctx.call(f"{'ex' if excl else ''}scan_add_{t}", [f"{t}_1d"], a)
+                if t == "f32":
+                    _close(out.values(), oracle.scan("add", t, xs, "f64acc", exclusive=excl))
+                else:
+                    assert np.array_equal(out.values(), oracle.scan("add", t, xs, exclusive=excl)), (n, excl)
+                out.free()
+            flags = np.zeros(n, np.uint8)
+            starts = [s for s in (0, tile - 1, tile, tile + 1, (k // 2) * tile, n - tile, n - 1) if 0 <= s < n]
+            flags[np.array(starts)] = 1
+            f = ctx.new("u8_1d", flags)
+            for op in ("add", "max"):
+                out = ctx.call(f"segscan_{op}_{t}", [f"{t}_1d"], f, a)
+                if t == "f32" and op == "add":
+                    _close(out.values(), oracle.segscan(op, t, flags, xs, "f64acc"))
+                else:
+                    assert np.array_equal(out.values(), oracle.segscan(op, t, flags, xs)), (n, op)
+                out.free()
+            f.free(); a.free()
+    # rows whose length divides the tile, equals it, and exceeds it by one
+    for m, k in ((8, tile), (9, tile // 2), (5, tile + 1), (3, 2 * tile - 1), (tile, 3)):
+        xss = _data(t, m * k, 47).reshape(m, k)
+        a = ctx.new(f"{t}_2d", xss)
+        out = ctx.call(f"scanrows_add_{t}", [f"{t}_2d"], a)
+        if t == "f32":
+            _close(out.values().reshape(-1), np.cumsum(xss.astype(np.float64), axis=1).reshape(-1))
+        else:
+            assert np.array_equal(out.values(), oracle.scanrows("add", t, xss)), (m, k)
+        out.free(); a.free()
 
 
 def test_more_than_2p31_elements(ctx):

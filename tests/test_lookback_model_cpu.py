@@ -183,3 +183,87 @@ def test_the_model_notices_a_broken_protocol():
         for flags in itertools.product([0, 1], repeat=3):
             explore([(flags[i], VALUES[i]) for i in range(3)], 2, 3, 2, stale_words(2),
                     accept_torn=True)
+
+
+# ---------------------------------------------------------------------------
+# Which ticket counter a persistent block draws from.
+#
+# The scan's blocks stay resident and draw tiles from several counters (counter
+# c hands out the tiles congruent to c).  A block keeps one counter for its
+# whole life and leaves when that counter has run out.  The model below
+# explores every order in which the hardware may start blocks and in which the
+# resident blocks take their steps, with at most R blocks resident, and asks
+# whether a state is reachable from which nothing can move before all tiles are
+# done.  Two rules for choosing the counter:
+#   "arrival": the k-th block to START uses counter k mod C (what the kernel does);
+#   "index":   block b uses counter b mod C, whatever the order of starts.
+def _ticket_model_deadlocks(rule, G, C, R, tiles):
+    """True when some schedule gets stuck.  A block: draw a tile from its counter;
+    publish the tile's aggregate; look back (needs the aggregates of all earlier
+    tiles); draw again.  It leaves on a ticket beyond the last tile."""
+    # state: (counters, started mask, blocks) with blocks = tuple over block ids of
+    # None (not started / left) or (counter, tile or None, published?)
+    def moves(state):
+        counters, started, left, blocks, done = state
+        out = []
+        resident = sum(b is not None for b in blocks)
+        if resident < R:
+            for b in range(G):
+                if not (started >> b) & 1:
+                    k = bin(started).count("1")
+                    c = (k if rule == "arrival" else b) % C
+                    nb = list(blocks)
+                    nb[b] = (c, None, False)
+                    out.append((counters, started | (1 << b), left, tuple(nb), done))
+                    if rule == "arrival":
+                        break  # blocks are interchangeable until they have a counter
+        for b, blk in enumerate(blocks):
+            if blk is None:
+                continue
+            c, tile, published = blk
+            nb = list(blocks)
+            if tile is None:  # draw
+                t = counters[c] * C + c
+                nc = list(counters)
+                nc[c] += 1
+                if t >= tiles:
+                    nb[b] = None
+                    out.append((tuple(nc), started, left | (1 << b), tuple(nb), done))
+                else:
+                    nb[b] = (c, t, False)
+                    out.append((tuple(nc), started, left, tuple(nb), done))
+            elif not published:
+                nb[b] = (c, tile, True)
+                out.append((counters, started, left, tuple(nb), done | (1 << tile)))
+            elif done & ((1 << tile) - 1) == (1 << tile) - 1:  # every earlier aggregate is there
+                nb[b] = (c, None, False)
+                out.append((counters, started, left, tuple(nb), done))
+        return out
+
+    start = ((0,) * C, 0, 0, (None,) * G, 0)
+    seen, stack = {start}, [start]
+    while stack:
+        st = stack.pop()
+        nxt = moves(st)
+        finished = st[2] == (1 << G) - 1
+        if not nxt and not finished:
+            return True
+        for s in nxt:
+            if s not in seen:
+                seen.add(s)
+                stack.append(s)
+    return False
+
+
+def test_counters_chosen_by_arrival_never_get_stuck():
+    """With the counter chosen by arrival number, C resident blocks (or the whole grid) are
+    enough for every schedule to finish; with the counter chosen by block index a grid that
+    is not wholly resident can get stuck (the blocks that happen to run leave a counter
+    without a drawer), and fewer than C resident blocks get stuck under either rule."""
+    for G, C, tiles in ((4, 2, 7), (5, 2, 6), (6, 3, 8), (3, 3, 5)):
+        for R in range(min(C, G), G + 1):
+            assert not _ticket_model_deadlocks("arrival", G, C, R, tiles), (G, C, R)
+        assert not _ticket_model_deadlocks("index", G, C, G, tiles)
+    assert _ticket_model_deadlocks("index", 4, 2, 2, 7)     # blocks 0 and 2 run: counter 1 starves
+    assert _ticket_model_deadlocks("index", 6, 3, 4, 8)
+    assert _ticket_model_deadlocks("arrival", 4, 2, 1, 7)   # the stated requirement is needed

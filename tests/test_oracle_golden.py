@@ -2,6 +2,7 @@
 routines.  Each check is chosen so that a plausible slip in the oracle (wrong
 neutral element, dropped wrap-around, off-by-one exclusive scan, unstable sort,
 transposed operand) fails it."""
+import math
 import numpy as np
 import pytest
 
@@ -264,6 +265,58 @@ def test_f64acc_variants_are_close_to_exact_and_lit_drifts():
     assert ex[0] == 0.0 and np.array_equal(ex[1:], got[:-1])
 
 
+def test_f64acc_reduce_segscan_segred_against_numpy_in_double():
+    """The f64-accumulated yardsticks of reduce, segmented scan and segmented
+    reduce are sums in double rounded once to f32: numpy's double sums and
+    cumulative sums over each segment say the same, bit for bit."""
+    rng = np.random.default_rng(14)
+    n = 200_003
+    xs = rng.random(n).astype(np.float32)
+    x64 = xs.astype(np.float64)
+    # reduce: one sum in double (math.fsum is the exact sum; both round to the same f32 here)
+    got = oracle.reduce("add", "f32", xs, "f64acc")
+    assert got == np.float32(np.add.reduce(x64))
+    assert abs(float(got) - math.fsum(x64.tolist())) <= 2.0 ** -24 * float(got)
+    assert oracle.reduce("add", "f32", xs[:0], "f64acc") == 0.0
+    assert oracle.reduce("add", "f32", xs[:1], "f64acc") == xs[0]
+    # A dropped element, a sum in f32 or a sum of squares would all fail this.
+    assert got != np.float32(np.add.reduce(x64[:-1]))
+
+    # segmented scan: restart at every flag; flags[0] == 0 (the neutral element
+    # is folded in front, which changes nothing) and a start on the last element.
+    flags = (rng.random(n) < 1 / 700).astype(np.uint8)
+    flags[0] = 0
+    flags[n - 1] = 1
+    flags[1000:1003] = 1  # segments of one element
+    starts = np.flatnonzero(flags).tolist()
+    bounds = [0] + [s for s in starts if s != 0] + [n]
+    want = np.empty(n, np.float32)
+    for a, b in zip(bounds[:-1], bounds[1:]):
+        want[a:b] = np.cumsum(x64[a:b]).astype(np.float32)
+    got = oracle.segscan("add", "f32", flags, xs, "f64acc")
+    assert np.array_equal(got, want)
+    assert got[n - 1] == xs[n - 1] and got[1001] == xs[1001]
+    # no flags at all: the plain scan in double
+    assert np.array_equal(oracle.segscan("add", "f32", np.zeros(n, np.uint8), xs, "f64acc"),
+                          np.cumsum(x64).astype(np.float32))
+
+    # segmented reduce over (offset, length) pairs: an empty segment gives the
+    # neutral element, and elements in a gap between segments belong to nobody.
+    lens = np.array([5, 0, 1, 70_000, 0, 3, 100_000], np.int64)
+    offsets = np.array([0, 5, 5, 6, 70_006, 70_100, 70_103], np.int64)  # gap: [70006, 70100)
+    assert offsets[-1] + lens[-1] <= n
+    want = np.array([np.add.reduce(x64[o:o + l]) for o, l in zip(offsets, lens)]).astype(np.float32)
+    got = oracle.segred("add", "f32", offsets, lens, xs, "f64acc")
+    assert np.array_equal(got, want)
+    assert got[1] == 0.0 and got[4] == 0.0 and got[2] == xs[5]
+    # segments that tile the array: the reduction of a segment is the scanned
+    # value at its last element (Builtins.hs:582-602)
+    ends = np.array(bounds[1:], np.int64)
+    begs = np.array(bounds[:-1], np.int64)
+    tiled = oracle.segred("add", "f32", begs, ends - begs, xs, "f64acc")
+    assert np.array_equal(tiled, oracle.segscan("add", "f32", flags, xs, "f64acc")[ends - 1])
+
+
 def test_transpose():
     x = np.arange(12, dtype=np.float32).reshape(3, 4)
     assert np.array_equal(oracle.transpose_f32(x), x.T)
@@ -285,6 +338,37 @@ def test_multicore_baseline_agrees_with_oracle():
                           oracle.rbi("add", "i32", np.zeros(256, np.int32), is_, xs))
     big = oracle.mc_rbi_add_i32(np.zeros(200000, np.int32), is_, xs, 4)  # atomic path
     assert np.array_equal(big, oracle.rbi("add", "i32", np.zeros(200000, np.int32), is_, xs))
+    # f32 histograms: max is order-independent (bit-exact); sums differ from the sequential
+    # fold only in the order of the additions
+    ws = rng.random(n).astype(np.float32)
+    dest = rng.random(300).astype(np.float32)
+    assert np.array_equal(oracle.mc_rbi_f32("max", dest, is_, ws, 5), oracle.rbi("max", "f32", dest, is_, ws))
+    np.testing.assert_allclose(oracle.mc_rbi_f32("add", dest, is_, ws, 5),
+                               oracle.rbi("add", "f32", dest, is_, ws, "f64acc"), rtol=1e-5)
+    # irregular segmented reduce: scan with flags from the offsets, then a gather
+    lens = np.array([5, 0, 1, 70_000, 0, 3, 100_000], np.int64)
+    offsets = np.concatenate(([0], np.cumsum(lens)[:-1])).astype(np.int64)
+    np.testing.assert_allclose(oracle.mc_segred_add_f32(offsets, lens, ws[: lens.sum()], 3),
+                               oracle.segred("add", "f32", offsets, lens, ws[: lens.sum()], "f64acc"),
+                               rtol=1e-5)
+    # matmul: the same sequential dot product per output as the oracle's literal fold
+    A = rng.standard_normal((3, 17, 29)).astype(np.float32)
+    B = rng.standard_normal((3, 29, 13)).astype(np.float32)
+    Bt = oracle.mc_transpose_f32(B, 3)
+    assert np.array_equal(Bt, B.transpose(0, 2, 1))
+    Cm = np.full((3, 17, 13), np.nan, np.float32)
+    oracle.mc_bmm_rows_f32(A, Bt, Cm, 0, 20, 4)     # a range of rows that crosses a batch boundary
+    oracle.mc_bmm_rows_f32(A, Bt, Cm, 20, 51, 4)
+    assert np.array_equal(Cm, oracle.bmm_f32(A, B, "lit"))
+    # radix sort: stable, keys and (key, value) pairs, against the sequential oracle
+    for dt in (np.uint32, np.uint64):
+        keys = rng.integers(0, np.iinfo(dt).max, 50_000, dtype=dt)
+        keys[::7] = keys[3]  # ties
+        idx = np.arange(keys.size, dtype=np.int32)
+        assert np.array_equal(oracle.mc_radix_sort(keys, None, 3), oracle.radix_sort(keys))
+        ko, vo = oracle.mc_radix_sort(keys, idx, 5)
+        kr, vr = oracle.radix_sort(keys, idx)
+        assert np.array_equal(ko, kr) and np.array_equal(vo, vr)
 
 
 def test_vectorised_reduce_is_a_reduce_per_column():

@@ -1,14 +1,16 @@
 """fa_segscan_static, the scan entry point that allocates nothing (its look-back
-scratch is a fixed array inside the library), against fa_segscan through the
-generated-library API on the same inputs: integers and max bit-exact, f32 sums
-within 1e-5 (the look-back folds tile aggregates in an order that depends on
-timing).  Two calls in a row per case, the second on a smaller input, so that
-what the first left in the shared scratch is in the way of the second."""
+scratch is a fixed array inside the library), against the CPU oracle and against
+fa_segscan through the generated-library API on the same inputs: integers and
+max bit-exact, f32 sums within 1e-5 of the f64-accumulated oracle (the look-back
+folds tile aggregates in an order that depends on timing).  Two calls in a row
+per case, the second on a smaller input, so that what the first left in the
+shared scratch is in the way of the second."""
 import ctypes as C
 
 import numpy as np
 import pytest
 
+import oracle
 from futhark_amd import datagen as dg, lib_path
 
 pytestmark = pytest.mark.gpu
@@ -25,6 +27,8 @@ def _lib():
                                     C.c_int, C.c_void_p]
     k.fa_segscan_static_max_n.restype = C.c_int64
     k.fa_segscan_static_max_n.argtypes = [C.c_int]
+    k.fa_segscan_tile_elems.restype = C.c_int64
+    k.fa_segscan_tile_elems.argtypes = [C.c_int]
     return k
 
 
@@ -56,9 +60,16 @@ def test_static_scan_matches_pooled_scan(ctx, t, op):
                                          f.device_ptr if seg else None, n, excl, out.device_ptr)
                 assert rc == 0
                 got, ref = out.values(), want.values()
-                if t == "f32" and op == "add":
-                    assert np.all(np.abs(got.astype(np.float64) - ref) <= 1e-5 * np.abs(ref))
+                variant = "f64acc" if (t, op) == ("f32", "add") else "lit"
+                if seg:
+                    truth = oracle.segscan(op, t, flags, xs, variant)
                 else:
+                    truth = oracle.scan(op, t, xs, variant, exclusive=bool(excl))
+                if t == "f32" and op == "add":
+                    for other in (truth, ref):
+                        assert np.all(np.abs(got.astype(np.float64) - other) <= 1e-5 * np.abs(other))
+                else:
+                    assert np.array_equal(got, truth)
                     assert np.array_equal(got, ref)
                 for h in (a, f, out, want):
                     h.free()
@@ -68,7 +79,8 @@ def test_static_scan_rejects_what_its_scratch_cannot_hold(ctx):
     k = _lib()
     for t in ("i32", "i64"):
         limit = k.fa_segscan_static_max_n(FA[t])
-        assert limit >= 1 << 26
+        # the documented figure: 256 KiB of descriptors, one per tile
+        assert limit == 16384 * k.fa_segscan_tile_elems(FA[t]) == {"i32": 234881024, "i64": 117440512}[t]
         a = ctx.new(f"{t}_1d", np.zeros(16, NP[t]))
         # rejected before anything is launched, so the short buffers are never touched
         assert k.fa_segscan_static(ctx.stream, FA[t], 0, a.device_ptr, None, limit + 1, 0,
