@@ -140,6 +140,10 @@ class Segops:
         L.futhark_entry_scan_norm_f32.argtypes = [vp, pp, vp]
         L.futhark_entry_reduce_summax_f32.argtypes = [vp, pp, vp]
         L.futhark_entry_rows_fraction_f32.argtypes = [vp, pp, vp]
+        L.futhark_entry_segreduce_argmax_i32.argtypes = [vp, pp, vp]
+        L.futhark_entry_segreduce_compose_i32.argtypes = [vp, pp, i64, vp]
+        L.futhark_entry_scanrows_argmax_i32.argtypes = [vp, pp, i64, vp]
+        L.futhark_entry_segred_argmax_i32.argtypes = [vp, pp, vp, vp, vp]
         L.futhark_entry_radix_sort_u32.argtypes = [vp, pp, vp]
         L.futhark_entry_radix_sort_u64.argtypes = [vp, pp, vp]
         for name, (k, v) in OPAQUE_PAIRS.items():

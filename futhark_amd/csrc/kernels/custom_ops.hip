@@ -12,7 +12,10 @@
 //   * a reduction whose operator does not commute (SegRed.hs:836-921) --
 //     composition of affine maps;
 //   * reduce_by_index with a tuple operator, which has to lock its bins
-//     (ImpGen/GPU/Base.hs:769-842) -- argmax per bin.
+//     (ImpGen/GPU/Base.hs:769-842) -- argmax per bin;
+//   * the same operators in the segmented forms -- argmax and composition per
+//     row (SegRed.hs:396-636), argmax scanned per row, argmax per irregular
+//     segment (Pass/Flatten/Builtins.hs:570-602).
 #include "futhark_amd_segops.hpp"
 
 namespace {
@@ -143,6 +146,56 @@ extern "C" int fa_scan_norm_f32(fa_stream_t stream, const float *xs, int64_t n, 
   return launch_scan<float, OpAdd<float>, SquareF32, SqrtF32>((hipStream_t)stream, xs, nullptr,
                                                               (int64_t)0, n, 0, out, scratch,
                                                               scratch_bytes, epoch);
+}
+
+// ---- the segmented forms with the same operators
+// map (\row -> reduce argmax ne (zip row (iota k))) xss: a regular segmented
+// reduction (SegRed.hs:396-636) with a tuple operator and the pair made on the
+// way in; out: [m][2]i32.
+extern "C" int fa_segreduce_argmax_i32(fa_stream_t stream, const int32_t *xss, int64_t m, int64_t k,
+                                       int32_t *out) {
+  return launch_segreduce<int32_t, ValIdx, ZipIndex, OpArgmax>((hipStream_t)stream, xss, m, k,
+                                                               (ValIdx *)out);
+}
+
+// map (reduce compose (1, 0)) over rows of k affine maps: the operator does not
+// commute, every row is folded in element order (SegRed.hs:836-921 per segment).
+extern "C" int fa_segreduce_compose_i32(fa_stream_t stream, const int32_t *abss, int64_t m, int64_t k,
+                                        int32_t *out) {
+  if (!is_aligned(abss, 8) || !is_aligned(out, 8)) return FA_EALIGN;
+  return launch_segreduce<AffineI32, AffineI32, AffineAsIs, OpCompose>(
+      (hipStream_t)stream, (const AffineI32 *)abss, m, k, (AffineI32 *)out);
+}
+
+// map (scan argmax ne) over rows of k (value, index) pairs: the single-pass scan
+// with segment starts computed from the row length (SegScan with segment
+// dimensions, SegScan/SinglePass.hs:327-361).
+extern "C" int fa_scanrows_argmax_i32(fa_stream_t stream, const int32_t *pairs, int64_t m, int64_t k,
+                                      int32_t *out, void *scratch, size_t scratch_bytes,
+                                      uint32_t epoch) {
+  if (m < 0 || k < 0 || (m > 0 && k > INT64_MAX / m)) return FA_EINVAL;
+  const int64_t n = m * k;
+  if (n == 0) return 0;
+  if (pairs == nullptr || out == nullptr || scratch == nullptr) return FA_EINVAL;
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
+  return launch_scan<ValIdx, OpArgmax>((hipStream_t)stream, pairs, nullptr, k, n, 0, out, scratch,
+                                       scratch_bytes, epoch);
+}
+
+// Irregular segments (Pass/Flatten/Builtins.hs:570-602) with the tuple operator:
+// out[i] = argmax over the pairs of segment i, the neutral pair when it is empty.
+extern "C" size_t fa_segred_argmax_workspace_bytes(int64_t n) {
+  return n < 0 ? 0 : segreduce_irregular_workspace_bytes<ValIdx>(n);
+}
+extern "C" int fa_segred_argmax_i32(fa_stream_t stream, const int64_t *offsets, const int64_t *lens,
+                                    int64_t m, const int32_t *pairs, int64_t n, int32_t *out,
+                                    void *workspace, size_t workspace_bytes, void *scratch,
+                                    size_t scratch_bytes, uint32_t epoch) {
+  if (epoch == 0 || epoch >= (1u << 28)) return FA_EINVAL;
+  if (n > 0 && scratch == nullptr) return FA_EINVAL;
+  return launch_segreduce_irregular<ValIdx, OpArgmax>(
+      (hipStream_t)stream, offsets, lens, m, (const ValIdx *)pairs, n, (ValIdx *)out, workspace,
+      workspace_bytes, scratch, scratch_bytes, epoch);
 }
 
 extern "C" size_t fa_hist_argmax_workspace_bytes(int64_t H) {

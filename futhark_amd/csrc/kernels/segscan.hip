@@ -30,6 +30,13 @@
 
 namespace fa {
 
+// How blocks pick their ticket counter: what the calling thread's tuning says.
+static ScanTickets scan_tickets() {
+  fa_tuning t;
+  fa_get_tuning(&t);
+  return t.scan_tickets_by_block ? ScanTickets::BY_BLOCK : ScanTickets::BY_ARRIVAL;
+}
+
 // ---- scratch for the entry point that allocates nothing
 // The header and 256 KiB of tile descriptors (16384 tiles).
 constexpr size_t SCAN_STATIC_BYTES = SCAN_HEADER_BYTES + 256 * 1024;
@@ -87,7 +94,7 @@ static int launch_scan_static(hipStream_t s, const void *xs, const uint8_t *flag
   const int rc = launch_status();
   if (rc != 0) return rc;
   return launch_scan<T, Op>(s, xs, flags, (int64_t)0, n, exclusive, out, base, SCAN_STATIC_BYTES, 1u,
-                            header + SCAN_STATIC_EPOCH_WORD);
+                            header + SCAN_STATIC_EPOCH_WORD, scan_tickets());
 }
 
 }  // namespace fa
@@ -146,10 +153,11 @@ extern "C" int fa_segscan(fa_stream_t stream, fa_dtype t, fa_op op, const void *
   hipStream_t s = (hipStream_t)stream;
   if (t == FA_I32X2)
     return op == FA_COMPOSE ? launch_scan<AffineI32, OpCompose>(s, xs, flags, (int64_t)0, n, exclusive,
-                                                                out, scratch, scratch_bytes, epoch)
+                                                                out, scratch, scratch_bytes, epoch,
+                                                                nullptr, scan_tickets())
                             : FA_ENOTSUP;
   FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xs, flags, (int64_t)0, n, exclusive, out, scratch,
-                      scratch_bytes, epoch);
+                      scratch_bytes, epoch, (const uint32_t *)nullptr, scan_tickets());
 }
 
 extern "C" int fa_segscan_rows(fa_stream_t stream, fa_dtype t, fa_op op, const void *xss,
@@ -164,8 +172,9 @@ extern "C" int fa_segscan_rows(fa_stream_t stream, fa_dtype t, fa_op op, const v
   if (t == FA_I32X2)
     return op == FA_COMPOSE
                ? launch_scan<AffineI32, OpCompose>(s, xss, (const uint8_t *)nullptr, k, n, exclusive,
-                                                   out, scratch, scratch_bytes, epoch)
+                                                   out, scratch, scratch_bytes, epoch, nullptr,
+                                                   scan_tickets())
                : FA_ENOTSUP;
   FA_DISPATCH_TYPE_OP(launch_scan, t, op, s, xss, (const uint8_t *)nullptr, k, n, exclusive, out,
-                      scratch, scratch_bytes, epoch);
+                      scratch, scratch_bytes, epoch, (const uint32_t *)nullptr, scan_tickets());
 }

@@ -21,21 +21,33 @@ static const char *const tuning_names[] = {
     "segops.hist_lds_bins_max",
     "segops.segred_small_threshold",
     "segops.matmul_pad_min_work",
+    "segops.scan_arrival_tickets",
 };
-static const char *const tuning_classes[] = {"shared_memory", "threshold", "threshold"};
-static const int64_t tuning_defaults[] = {0, 0, 0}; /* 0: the kernel library's default */
+static const char *const tuning_classes[] = {"shared_memory", "threshold", "threshold", "threshold"};
+static const int64_t tuning_defaults[] = {0, 0, 0, 0}; /* 0: the kernel library's default */
 
-/* The parameters choose code paths inside the kernel library (fa_tuning). */
+/* The parameters choose code paths inside the kernel library (fa_tuning).
+ *
+ * segops.scan_arrival_tickets: how the blocks of the single-pass scan pick
+ * their ticket counter (fa_tuning.scan_tickets_by_block).  0 lets the runtime
+ * decide: by block index, the cheaper way, while this context is the only one
+ * alive in the process and no CU mask is set in the environment (a scan of a
+ * single stream then has the device to itself, as far as this process can
+ * tell), by order of arrival otherwise.  1 always takes the order of arrival:
+ * for a process that shares the GPU with other processes' long-running
+ * kernels, or runs under a CU mask it applies by other means. */
 static void apply_tuning(struct futhark_context *ctx) {
   fa_tuning t;
   t.hist_lds_bins_max = rts_tuning_param(ctx, tuning_names[0], 0);
   t.segred_small_threshold = rts_tuning_param(ctx, tuning_names[1], 0);
   t.matmul_pad_min_work = rts_tuning_param(ctx, tuning_names[2], 0);
+  t.scan_tickets_by_block =
+      rts_tuning_param(ctx, tuning_names[3], 0) == 0 && rts_device_is_ours(ctx) ? 1 : 0;
   fa_set_tuning(&t);
 }
 
 const struct rts_program futhark_program = {
-    "segops", 3, tuning_names, tuning_classes, tuning_defaults, apply_tuning,
+    "segops", 4, tuning_names, tuning_classes, tuning_defaults, apply_tuning,
 };
 
 /* ------------------------------------------------------------------ arrays */
@@ -928,6 +940,134 @@ int futhark_entry_scan_norm_f32(struct futhark_context *ctx, struct futhark_f32_
                                 const struct futhark_f32_1d *in0) {
   ENTER(ctx);
   int ret = do_custom_scan(ctx, (struct fut_array **)out0, &in0->a, 1, "scan_norm_f32");
+  LEAVE(ctx);
+  return ret;
+}
+
+/* The tuple and the non-commutative operator in the segmented forms. */
+int futhark_entry_segreduce_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                       const struct futhark_i32_2d *in0) {
+  ENTER(ctx);
+  const int64_t m = in0->a.shape[0], k = in0->a.shape[1];
+  const int64_t dims[2] = {m, 2};
+  int ret = 0;
+  struct fut_array *res = out_array(ctx, m * 8, 2, dims, "segreduce.out");
+  if (res == NULL) {
+    ret = FUTHARK_OUT_OF_MEMORY;
+  } else {
+    struct rts_event *ev = rts_kernel_begin(
+        ctx, "segred_regular",
+        rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)k));
+    int code = fa_segreduce_argmax_i32(ctx->stream, (const int32_t *)in0->a.mem.mem, m, k,
+                                       (int32_t *)res->mem.mem);
+    ret = rts_kernel_end(ctx, ev, "segred_regular", code);
+    if (ret != 0) drop_array(ctx, res);
+    else *out0 = (struct futhark_i32_2d *)res;
+  }
+  LEAVE(ctx);
+  return ret;
+}
+
+/* Rows of k elements of a flat [m * k][2]i32 array; 0 on success with m in *m_out. */
+static int rows_of(struct futhark_context *ctx, const struct fut_array *in, int64_t k,
+                   const char *entry, int64_t *m_out) {
+  const int64_t n = in->shape[0];
+  if (in->shape[1] != 2 || k < 0 || (k == 0 && n != 0) || (k > 0 && n % k != 0))
+    return bad_sizes(ctx, entry);
+  *m_out = k == 0 ? 0 : n / k;
+  return 0;
+}
+
+int futhark_entry_segreduce_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                        const int64_t in0, const struct futhark_i32_2d *in1) {
+  ENTER(ctx);
+  int64_t m = 0;
+  int ret = rows_of(ctx, &in1->a, in0, "segreduce_compose_i32", &m);
+  if (ret == 0) {
+    const int64_t dims[2] = {m, 2};
+    struct fut_array *res = out_array(ctx, m * 8, 2, dims, "segreduce.out");
+    if (res == NULL) {
+      ret = FUTHARK_OUT_OF_MEMORY;
+    } else {
+      struct rts_event *ev = rts_kernel_begin(
+          ctx, "segred_regular",
+          rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)in0));
+      int code = fa_segreduce_compose_i32(ctx->stream, (const int32_t *)in1->a.mem.mem, m, in0,
+                                          (int32_t *)res->mem.mem);
+      ret = rts_kernel_end(ctx, ev, "segred_regular", code);
+      if (ret != 0) drop_array(ctx, res);
+      else *out0 = (struct futhark_i32_2d *)res;
+    }
+  }
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_scanrows_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                      const int64_t in0, const struct futhark_i32_2d *in1) {
+  ENTER(ctx);
+  int64_t m = 0;
+  int ret = rows_of(ctx, &in1->a, in0, "scanrows_argmax_i32", &m);
+  if (ret == 0) {
+    const int64_t n = in1->a.shape[0];
+    uint32_t epoch = 0;
+    void *scratch = rts_scan_scratch(ctx, fa_segscan_scratch_bytes(FA_I64, n), &epoch);
+    struct fut_array *res = scratch == NULL ? NULL : out_array(ctx, n * 8, 2, in1->a.shape, "scan.out");
+    if (res == NULL) {
+      ret = ctx->error || scratch != NULL ? FUTHARK_OUT_OF_MEMORY : 1;
+    } else {
+      struct rts_event *ev = rts_kernel_begin(
+          ctx, "segscan_rows",
+          rts_msgprintf("{\"segments\":%lld,\"segment_size\":%lld}", (long long)m, (long long)in0));
+      int code = fa_scanrows_argmax_i32(ctx->stream, (const int32_t *)in1->a.mem.mem, m, in0,
+                                        (int32_t *)res->mem.mem, scratch, ctx->scan_scratch_bytes,
+                                        epoch);
+      ret = rts_kernel_end(ctx, ev, "segscan_rows", code);
+      if (ret != 0) drop_array(ctx, res);
+      else *out0 = (struct futhark_i32_2d *)res;
+    }
+  }
+  LEAVE(ctx);
+  return ret;
+}
+
+int futhark_entry_segred_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                    const struct futhark_i64_1d *in0,
+                                    const struct futhark_i64_1d *in1,
+                                    const struct futhark_i32_2d *in2) {
+  ENTER(ctx);
+  const int64_t m = in0->a.shape[0], n = in2->a.shape[0];
+  int ret = 0;
+  if (in1->a.shape[0] != m || in2->a.shape[1] != 2) {
+    ret = bad_sizes(ctx, "segred_argmax_i32");
+  } else {
+    const int64_t dims[2] = {m, 2};
+    uint32_t epoch = 0;
+    void *scratch = rts_scan_scratch(ctx, fa_segscan_scratch_bytes(FA_I64, n), &epoch);
+    struct fut_array *res = scratch == NULL ? NULL : out_array(ctx, m * 8, 2, dims, "segred.out");
+    struct memblock_device ws = {0};
+    if (res == NULL) {
+      ret = ctx->error || scratch != NULL ? FUTHARK_OUT_OF_MEMORY : 1;
+    } else if ((ret = rts_memblock_alloc(ctx, &ws, (int64_t)fa_segred_argmax_workspace_bytes(n),
+                                         "segred.workspace")) == 0) {
+      /* The segments are checked like those of the library's own segmented
+       * reduction: a violation is reported at the next synchronisation. */
+      struct rts_event *ev = rts_kernel_begin(
+          ctx, "segred_irregular", rts_msgprintf("{\"n\":%lld,\"segments\":%lld}", (long long)n, (long long)m));
+      int code = fa_segments_check(ctx->stream, (const int64_t *)in0->a.mem.mem,
+                                   (const int64_t *)in1->a.mem.mem, m, n, RTS_FAILURE_WORD(ctx),
+                                   RTS_FAILURE_SEGMENTS);
+      if (code == 0)
+        code = fa_segred_argmax_i32(ctx->stream, (const int64_t *)in0->a.mem.mem,
+                                    (const int64_t *)in1->a.mem.mem, m,
+                                    (const int32_t *)in2->a.mem.mem, n, (int32_t *)res->mem.mem, ws.mem,
+                                    (size_t)ws.size, scratch, ctx->scan_scratch_bytes, epoch);
+      ret = rts_kernel_end(ctx, ev, "segred_irregular", code);
+    }
+    rts_memblock_unref(ctx, &ws, "segred.workspace");
+    if (ret != 0) drop_array(ctx, res);
+    else *out0 = (struct futhark_i32_2d *)res;
+  }
   LEAVE(ctx);
   return ret;
 }

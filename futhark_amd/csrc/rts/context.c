@@ -620,6 +620,24 @@ int futhark_context_clear_caches(struct futhark_context *ctx) {
   return ctx->error != NULL;
 }
 
+/* Contexts alive in this process (counted from backend set-up to free). */
+static int live_contexts = 0;
+static pthread_mutex_t live_contexts_lock = PTHREAD_MUTEX_INITIALIZER;
+static void count_context(int delta) {
+  pthread_mutex_lock(&live_contexts_lock);
+  live_contexts += delta;
+  pthread_mutex_unlock(&live_contexts_lock);
+}
+int rts_device_is_ours(struct futhark_context *ctx) {
+  (void)ctx;
+  pthread_mutex_lock(&live_contexts_lock);
+  const int alone = live_contexts <= 1;
+  pthread_mutex_unlock(&live_contexts_lock);
+  if (!alone) return 0;
+  const char *m1 = getenv("HSA_CU_MASK"), *m2 = getenv("ROC_GLOBAL_CU_MASK");
+  return (m1 == NULL || m1[0] == '\0') && (m2 == NULL || m2[0] == '\0');
+}
+
 struct futhark_context *futhark_context_new(struct futhark_context_config *cfg) {
   struct futhark_context *ctx =
       (struct futhark_context *)calloc(1, sizeof(struct futhark_context));
@@ -638,6 +656,7 @@ struct futhark_context *futhark_context_new(struct futhark_context_config *cfg) 
   ctx->log = stderr;
   if (backend_setup(ctx) == 0) {
     ctx->program_initialised = true;
+    count_context(1);
     (void)futhark_context_clear_caches(ctx);
     (void)futhark_context_sync(ctx);
   }
@@ -646,6 +665,7 @@ struct futhark_context *futhark_context_new(struct futhark_context_config *cfg) 
 }
 
 void futhark_context_free(struct futhark_context *ctx) {
+  if (ctx->program_initialised) count_context(-1);
   if (ctx->stream != NULL) {
     (void)hipStreamSynchronize((hipStream_t)ctx->stream);
     if (ctx->scan_scratch) (void)hipFree(ctx->scan_scratch);

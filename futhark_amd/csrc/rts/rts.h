@@ -233,4 +233,9 @@ int rts_kernel_end(struct futhark_context *ctx, struct rts_event *ev, const char
 
 int64_t rts_tuning_param(struct futhark_context *ctx, const char *name, int64_t fallback);
 
+/* Nonzero while, as far as this process can tell, a kernel of this context has
+ * the device to itself: no other context is alive in the process and the
+ * environment sets no CU mask (HSA_CU_MASK, ROC_GLOBAL_CU_MASK). */
+int rts_device_is_ours(struct futhark_context *ctx);
+
 #endif /* FUTHARK_AMD_RTS_H */

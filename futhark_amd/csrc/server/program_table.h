@@ -257,6 +257,21 @@ static int e_reduce_compose_i32(struct futhark_context *c, struct value *o, stru
 static int e_sumsq_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_sumsq_f32(c, &o->u.f32, ARRP(i[0]));
 }
+static int e_segreduce_argmax_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_segreduce_argmax_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]));
+}
+static int e_segreduce_compose_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_segreduce_compose_i32(c, (struct futhark_i32_2d **)&o->u.arr, i[0]->u.i64,
+                                             ARRP(i[1]));
+}
+static int e_scanrows_argmax_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_scanrows_argmax_i32(c, (struct futhark_i32_2d **)&o->u.arr, i[0]->u.i64,
+                                           ARRP(i[1]));
+}
+static int e_segred_argmax_i32(struct futhark_context *c, struct value *o, struct value **i) {
+  return futhark_entry_segred_argmax_i32(c, (struct futhark_i32_2d **)&o->u.arr, ARRP(i[0]),
+                                         ARRP(i[1]), ARRP(i[2]));
+}
 static int e_rows_fraction_f32(struct futhark_context *c, struct value *o, struct value **i) {
   return futhark_entry_rows_fraction_f32(c, (struct futhark_f32_2d **)&o->u.arr, ARRP(i[0]));
 }
@@ -315,17 +330,21 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
 #define HIST_PARAM "segops.hist_lds_bins_max"
 #define SEGRED_PARAM "segops.segred_small_threshold"
 #define MATMUL_PARAM "segops.matmul_pad_min_work"
+#define SCAN_PARAM "segops.scan_arrival_tickets"
 #define SEGOP_ENTRY_ROWS(OP, T, CT)                                                             \
   {"reduce_" #OP "_" #T, e_reduce_##OP##_##T, #T, 0, 1, {"[]" #T}, {0}, {NULL}},                \
-  {"scan_" #OP "_" #T, e_scan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {NULL}},               \
-  {"exscan_" #OP "_" #T, e_exscan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {NULL}},           \
-  {"segscan_" #OP "_" #T, e_segscan_##OP##_##T, "[]" #T, 1, 2, {"[]u8", "[]" #T}, {0}, {NULL}}, \
+  {"scan_" #OP "_" #T, e_scan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {SCAN_PARAM, NULL}},   \
+  {"exscan_" #OP "_" #T, e_exscan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0},                    \
+   {SCAN_PARAM, NULL}},                                                                         \
+  {"segscan_" #OP "_" #T, e_segscan_##OP##_##T, "[]" #T, 1, 2, {"[]u8", "[]" #T}, {0},          \
+   {SCAN_PARAM, NULL}},                                                                         \
   {"segred_" #OP "_" #T, e_segred_##OP##_##T, "[]" #T, 1, 3, {"[]i64", "[]i64", "[]" #T},       \
    {0}, {NULL}},                                                                                \
   {"segreduce_" #OP "_" #T, e_segreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0},            \
    {SEGRED_PARAM, NULL}},                                                                       \
   {"vecreduce_" #OP "_" #T, e_vecreduce_##OP##_##T, "[]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},   \
-  {"scanrows_" #OP "_" #T, e_scanrows_##OP##_##T, "[][]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},   \
+  {"scanrows_" #OP "_" #T, e_scanrows_##OP##_##T, "[][]" #T, 1, 1, {"[][]" #T}, {0},            \
+   {SCAN_PARAM, NULL}},                                                                         \
   {"vecscan_" #OP "_" #T, e_vecscan_##OP##_##T, "[][]" #T, 1, 1, {"[][]" #T}, {0}, {NULL}},     \
   {"seghist_" #OP "_" #T, e_seghist_##OP##_##T, "[][]" #T, 1, 3,                                \
    {"i64", "[][]i32", "[][]" #T}, {0}, {HIST_PARAM, NULL}},                                     \
@@ -353,10 +372,11 @@ static const struct entry entries[] = {
     FUTHARK_FOR_EACH_OP(HIST_ENTRY_ROWS, f16, uint16_t)
     {"bmm_f32", e_bmm_f32, "[][][]f32", 1, 2, {"[][][]f32", "[][][]f32"}, {0}, {MATMUL_PARAM, NULL}},
     {"bmm_f16", e_bmm_f16, "[][][]f32", 1, 2, {"[][][]f16", "[][][]f16"}, {0}, {MATMUL_PARAM, NULL}},
-    {"scan_compose_i32", e_scan_compose_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
-    {"exscan_compose_i32", e_exscan_compose_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
+    {"scan_compose_i32", e_scan_compose_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {SCAN_PARAM, NULL}},
+    {"exscan_compose_i32", e_exscan_compose_i32, "[][]i32", 1, 1, {"[][]i32"}, {0},
+     {SCAN_PARAM, NULL}},
     {"segscan_compose_i32", e_segscan_compose_i32, "[][]i32", 1, 2, {"[]u8", "[][]i32"}, {0},
-     {NULL}},
+     {SCAN_PARAM, NULL}},
     {"reduce_argmax_i32", e_reduce_argmax_i32, "[]i32", 1, 1, {"[]i32"}, {0}, {NULL}},
     {"scan_argmax_i32", e_scan_argmax_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
     {"hist_argmax_i32", e_hist_argmax_i32, "[][]i32", 1, 3, {"i64", "[]i32", "[]i32"}, {0}, {NULL}},
@@ -365,6 +385,12 @@ static const struct entry entries[] = {
     {"scan_norm_f32", e_scan_norm_f32, "[]f32", 1, 1, {"[]f32"}, {0}, {NULL}},
     {"reduce_summax_f32", e_reduce_summax_f32, "[]f32", 1, 1, {"[]f32"}, {0}, {NULL}},
     {"rows_fraction_f32", e_rows_fraction_f32, "[][]f32", 1, 1, {"[][]f32"}, {0}, {NULL}},
+    {"segreduce_argmax_i32", e_segreduce_argmax_i32, "[][]i32", 1, 1, {"[][]i32"}, {0}, {NULL}},
+    {"segreduce_compose_i32", e_segreduce_compose_i32, "[][]i32", 1, 2, {"i64", "[][]i32"}, {0},
+     {NULL}},
+    {"scanrows_argmax_i32", e_scanrows_argmax_i32, "[][]i32", 1, 2, {"i64", "[][]i32"}, {0}, {NULL}},
+    {"segred_argmax_i32", e_segred_argmax_i32, "[][]i32", 1, 3, {"[]i64", "[]i64", "[][]i32"}, {0},
+     {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {MATMUL_PARAM, NULL}},
     {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {MATMUL_PARAM, NULL}},
     {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {NULL}},

@@ -21,6 +21,7 @@ VERSION = "segops for gfx950, C API of Futhark 0.28.0"
 HIST_PARAM = "segops.hist_lds_bins_max"
 SEGRED_PARAM = "segops.segred_small_threshold"
 MATMUL_PARAM = "segops.matmul_pad_min_work"
+SCAN_PARAM = "segops.scan_arrival_tickets"
 
 
 def _array_type_name(kind: str) -> str:
@@ -45,13 +46,13 @@ def entry_points() -> dict:
             a = f"[]{t}"
             eps += [
                 _entry(f"reduce_{op}_{t}", t, [("xs", a)]),
-                _entry(f"scan_{op}_{t}", a, [("xs", a)]),
-                _entry(f"exscan_{op}_{t}", a, [("xs", a)]),
-                _entry(f"segscan_{op}_{t}", a, [("flags", "[]u8"), ("vs", a)]),
+                _entry(f"scan_{op}_{t}", a, [("xs", a)], [SCAN_PARAM]),
+                _entry(f"exscan_{op}_{t}", a, [("xs", a)], [SCAN_PARAM]),
+                _entry(f"segscan_{op}_{t}", a, [("flags", "[]u8"), ("vs", a)], [SCAN_PARAM]),
                 _entry(f"segred_{op}_{t}", a, [("offsets", "[]i64"), ("lens", "[]i64"), ("vs", a)]),
                 _entry(f"segreduce_{op}_{t}", a, [("xss", "[]" + a)], [SEGRED_PARAM]),
                 _entry(f"vecreduce_{op}_{t}", a, [("xss", "[]" + a)]),
-                _entry(f"scanrows_{op}_{t}", "[]" + a, [("xss", "[]" + a)]),
+                _entry(f"scanrows_{op}_{t}", "[]" + a, [("xss", "[]" + a)], [SCAN_PARAM]),
                 _entry(f"vecscan_{op}_{t}", "[]" + a, [("xss", "[]" + a)]),
                 _entry(f"seghist_{op}_{t}", "[]" + a,
                        [("k", "i64"), ("iss", "[][]i32"), ("vss", "[]" + a)], [HIST_PARAM]),
@@ -72,9 +73,9 @@ def entry_points() -> dict:
     eps += [
         _entry("bmm_f32", "[][][]f32", [("A", "[][][]f32"), ("B", "[][][]f32")], [MATMUL_PARAM]),
         _entry("bmm_f16", "[][][]f32", [("A", "[][][]f16"), ("B", "[][][]f16")], [MATMUL_PARAM]),
-        _entry("scan_compose_i32", "[][]i32", [("abs", "[][]i32")]),
-        _entry("exscan_compose_i32", "[][]i32", [("abs", "[][]i32")]),
-        _entry("segscan_compose_i32", "[][]i32", [("flags", "[]u8"), ("abs", "[][]i32")]),
+        _entry("scan_compose_i32", "[][]i32", [("abs", "[][]i32")], [SCAN_PARAM]),
+        _entry("exscan_compose_i32", "[][]i32", [("abs", "[][]i32")], [SCAN_PARAM]),
+        _entry("segscan_compose_i32", "[][]i32", [("flags", "[]u8"), ("abs", "[][]i32")], [SCAN_PARAM]),
         _entry("reduce_argmax_i32", "[]i32", [("xs", "[]i32")]),
         _entry("scan_argmax_i32", "[][]i32", [("vis", "[][]i32")]),
         _entry("hist_argmax_i32", "[][]i32", [("k", "i64"), ("is", "[]i32"), ("xs", "[]i32")]),
@@ -83,6 +84,10 @@ def entry_points() -> dict:
         _entry("scan_norm_f32", "[]f32", [("xs", "[]f32")]),
         _entry("reduce_summax_f32", "[]f32", [("xs", "[]f32")]),
         _entry("rows_fraction_f32", "[][]f32", [("xss", "[][]f32")]),
+        _entry("segreduce_argmax_i32", "[][]i32", [("xss", "[][]i32")]),
+        _entry("segreduce_compose_i32", "[][]i32", [("k", "i64"), ("abs", "[][]i32")]),
+        _entry("scanrows_argmax_i32", "[][]i32", [("k", "i64"), ("vis", "[][]i32")]),
+        _entry("segred_argmax_i32", "[][]i32", [("offsets", "[]i64"), ("lens", "[]i64"), ("vis", "[][]i32")]),
         _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")], [MATMUL_PARAM]),
         _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")], [MATMUL_PARAM]),
         _entry("radix_sort_u32", "[]u32", [("keys", "[]u32")]),

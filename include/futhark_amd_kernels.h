@@ -95,11 +95,24 @@ int fa_version(void);
  *                           limit 32768); four ranges fit one launch, more
  *                           bins go through the partitioned path
  *   matmul_pad_min_work     least M*N*K*batch for which shapes off the tile
- *                           grid run on padded copies (default 2^24) */
+ *                           grid run on padded copies (default 2^24)
+ *   scan_tickets_by_block   how a block of the single-pass scan picks the ticket
+ *                           counter it draws tiles from.  0 (default): by the
+ *                           order in which blocks start; the scan finishes
+ *                           whenever eight of its blocks can be resident at the
+ *                           same time, on any CUs.  Nonzero: by block index,
+ *                           which saves an atomic on one address per block and
+ *                           the wait for the first ticket (2-3 us per launch)
+ *                           and needs all blocks of the launch (one per CU at
+ *                           most) resident at the same time: for callers that
+ *                           know the launch has the device to itself (no CU
+ *                           mask, no other kernels that wait for something
+ *                           while they hold CUs) */
 typedef struct fa_tuning {
   int64_t segred_small_threshold;
   int64_t hist_lds_bins_max;
   int64_t matmul_pad_min_work;
+  int64_t scan_tickets_by_block;
 } fa_tuning;
 void fa_set_tuning(const fa_tuning *t); /* NULL: all defaults */
 void fa_get_tuning(fa_tuning *out);     /* the values in effect */
@@ -373,6 +386,31 @@ int fa_iota(fa_stream_t stream, fa_dtype t, void *dst, int64_t n,
  *                         in global memory (SegHist.hs:377-467);
  *                         H <= fa_hist_argmax_max_bins(); workspace of
  *                         fa_hist_argmax_workspace_bytes(H) bytes, contents irrelevant. */
+/* The same operators in the segmented forms (a program's own operator in
+ * `map (reduce op ne)`, `map (scan op ne)` and in a reduction over irregular
+ * segments; SegRed.hs:396-636, SegScan/SinglePass.hs:327-361,
+ * Pass/Flatten/Builtins.hs:570-602):
+ *   fa_segreduce_argmax_i32:  xss [m][k]i32 -> out [m][2]i32, (max, first column of it)
+ *                             per row, (i32.lowest, i32.highest) for k = 0
+ *   fa_segreduce_compose_i32: abss [m][k][2]i32 -> out [m][2]i32, the maps of a row
+ *                             composed in element order
+ *   fa_scanrows_argmax_i32:   pairs [m][k][2]i32 -> out of the same shape, scanned per
+ *                             row; scratch and epoch as for fa_segscan with n = m * k
+ *   fa_segred_argmax_i32:     pairs [n][2]i32, segments (offsets[i], lens[i]) that tile
+ *                             a prefix of the pairs in order -> out [m][2]i32;
+ *                             workspace of fa_segred_argmax_workspace_bytes(n) bytes,
+ *                             16-byte aligned, contents irrelevant */
+int fa_segreduce_argmax_i32(fa_stream_t stream, const int32_t *xss, int64_t m, int64_t k,
+                            int32_t *out);
+int fa_segreduce_compose_i32(fa_stream_t stream, const int32_t *abss, int64_t m, int64_t k,
+                             int32_t *out);
+int fa_scanrows_argmax_i32(fa_stream_t stream, const int32_t *pairs, int64_t m, int64_t k,
+                           int32_t *out, void *scratch, size_t scratch_bytes, uint32_t epoch);
+size_t fa_segred_argmax_workspace_bytes(int64_t n);
+int fa_segred_argmax_i32(fa_stream_t stream, const int64_t *offsets, const int64_t *lens, int64_t m,
+                         const int32_t *pairs, int64_t n, int32_t *out, void *workspace,
+                         size_t workspace_bytes, void *scratch, size_t scratch_bytes,
+                         uint32_t epoch);
 int fa_reduce_argmax_i32(fa_stream_t stream, const int32_t *xs, int64_t n, int32_t *out2,
                          void *scratch, size_t scratch_bytes, uint32_t epoch);
 int fa_scan_argmax_i32(fa_stream_t stream, const int32_t *pairs, const uint8_t *flags, int64_t n,

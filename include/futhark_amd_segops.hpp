@@ -23,6 +23,10 @@
 //   launch_reduce<Tin, T, Pre, Op>     reduction; Pre maps (element, its index) to T;
 //                                      operators that do not commute are folded in
 //                                      element order (SegRed.hs:836-921)
+//   launch_segreduce<Tin, T, Pre, Op>  the same per row of a [m][k] array (regular
+//                                      segments, SegRed.hs:396-636)
+//   launch_segreduce_irregular<T, Op>  per (offset, length) segment: a scan with flags
+//                                      from the offsets and a gather (Builtins.hs:570-602)
 //   launch_hist_locked<...>            reduce_by_index for an operator over a pair of
 //                                      values kept in two arrays, which no single
 //                                      atomic can update: bins are locked
@@ -55,13 +59,27 @@ constexpr uint32_t ST_P = 2;  // inclusive prefix up to the end of the tile
 // channels) is a ticket counter: same-address atomics are performed one at a
 // time, about 12 ns each on MI355X, and a channel that does little else slows
 // every stream that crosses it.  Counter c hands out the tiles congruent to c
-// modulo the number of counters in use.  A block draws from the counter its
-// arrival number selects (arrival number mod the number of counters), not
-// from one its block index selects: whichever blocks the hardware starts
-// first, the first eight of them cover all eight counters, so every tile is
-// handed out as long as eight blocks (or the whole grid, if it is smaller)
-// can be resident at the same time -- on any CUs, of any die.  Blocks that
-// start later join the counters in turn.
+// modulo the number of counters in use, and a block draws from one counter for
+// as long as it runs (its tiles then come in increasing order, which the
+// pipeline of three tiles inside a block relies on).  Every tile is handed out
+// only if every counter has a block drawing from it.  Which counter a block
+// takes is the launch's choice (ScanTickets):
+//   * BY_ARRIVAL: the block's arrival number (one more atomic, on one address
+//     for all blocks) modulo the number of counters.  Whichever blocks the
+//     hardware starts first, the first eight cover all eight counters, so the
+//     launch finishes as long as eight blocks (or the whole grid, if it is
+//     smaller) can be resident at the same time -- on any CUs, of any die.
+//     The arrival atomic costs 1.5-2.5 us per launch (256 atomics on one
+//     address, and a round trip more before the first ticket): 2^26 f32 with
+//     flags 92.9 -> 94.4 us, 2^24 i32 28.8 -> 30.4 us.
+//   * BY_BLOCK: block index modulo the number of counters, no arrival atomic,
+//     and the first two tiles of a block follow from its index as well, so its
+//     first loads wait for nothing.  This needs every block of the launch
+//     resident at the same time (the grid has at most one block per CU): true
+//     for a launch that has the GPU to itself, not guaranteed under a CU mask,
+//     nor when other kernels that themselves wait for something hold CUs.
+//     Callers choose it when they know that the launch is alone on the device.
+enum class ScanTickets { BY_ARRIVAL = 0, BY_BLOCK = 1 };
 constexpr size_t SCAN_HEADER_BYTES = 8192;
 constexpr int SCAN_MAX_COUNTERS = 8;
 constexpr int SCAN_COUNTER_STRIDE = 64;  // in 32-bit words
@@ -257,7 +275,7 @@ template <class T, class Op, int SEGKIND, bool EXCL, class Pre = MapIdentity, cl
 __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
     const T *__restrict__ xs, const uint8_t *__restrict__ flags, int64_t n, T *__restrict__ out,
     uint32_t *header, uint64_t *desc, uint32_t epoch, const uint32_t *epoch_dev, int64_t num_tiles,
-    int64_t seg_len) {
+    int64_t seg_len, uint32_t by_arrival) {
   // The epoch of this launch: an argument, or (for callers whose launches may
   // be replayed with the same arguments) a word a preceding kernel advanced.
   if (epoch_dev != nullptr) epoch = *epoch_dev;
@@ -292,7 +310,7 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
   // The protocol wave takes the block's arrival number first of all: its round
   // trip runs while the rest of the block sets up.
   uint32_t arrival = 0u;
-  if (tid == SS_DATA_THREADS) arrival = atomicAdd(header + SCAN_ARRIVAL_WORD, 1u);
+  if (by_arrival && tid == SS_DATA_THREADS) arrival = atomicAdd(header + SCAN_ARRIVAL_WORD, 1u);
   if (tid < SS_WAVES) s_scanned[tid] = 0u;
   if (tid == 0) {
     s_tiles_known = 0u;
@@ -309,7 +327,8 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
 
   if (wave == SS_WAVES) {
     // ------------------------------------------------------------ protocol wave
-    const uint32_t my_counter = (uint32_t)__builtin_amdgcn_readfirstlane((int)arrival) % counters;
+    const uint32_t my_counter =
+        (by_arrival ? (uint32_t)__builtin_amdgcn_readfirstlane((int)arrival) : blockIdx.x) % counters;
     uint32_t *ticket = header + my_counter * SCAN_COUNTER_STRIDE;
     // Exclusive prefix of `tile` (> 0): folds the descriptors of the tiles
     // before it, newest window first, back to one that has published its prefix
@@ -371,25 +390,36 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
       return acc;
     };
 
-    // Hands ticket `t` out as tile `q`.
+    // Hands tile number `t` out as the block's tile `q`.
     auto hand_out = [&](int q, uint32_t t) {
       if (lane == 0) {
-        s_tile[q % SS_RING] = t * counters + my_counter;
+        s_tile[q % SS_RING] = t;
         ss_signal(&s_tiles_known, (uint32_t)q + 1u);
       }
     };
+    // By block index, the first two tiles of block b are b and b + gridDim.x,
+    // without a ticket (every block of such a launch is resident, so each of
+    // these tiles has its block): the first loads leave before any atomic has
+    // come back.  The counters hand out what follows.
+    const uint32_t first_ticketed = by_arrival ? 0u : 2u * gridDim.x;
+    auto tile_of_ticket = [&](uint32_t t) { return first_ticketed + t * counters + my_counter; };
     // The first three tickets are drawn one after the other, each after the one
     // before has come back: three tickets drawn at once would be consecutive
     // tiles, and the block next in line would wait two rounds for the aggregate
     // of this block's third tile.  Drawn a round trip apart, the first tickets
     // of all blocks come first, then their second ones, as in every later round.
     uint32_t t0 = 0u, t1 = 0u, t2 = 0u, pending = 0u;
-    if (lane == 0) t0 = atomicAdd(ticket, 1u);
-    hand_out(0, t0);
-    if (lane == 0) t1 = atomicAdd(ticket, 1u + (t0 >> 31));  // (+0) issued after t0 is back
-    hand_out(1, t1);
+    if (by_arrival) {
+      if (lane == 0) t0 = atomicAdd(ticket, 1u);
+      hand_out(0, tile_of_ticket(t0));
+      if (lane == 0) t1 = atomicAdd(ticket, 1u + (t0 >> 31));  // (+0) issued after t0 is back
+      hand_out(1, tile_of_ticket(t1));
+    } else {
+      hand_out(0, blockIdx.x);
+      hand_out(1, blockIdx.x + gridDim.x);
+    }
     if (lane == 0) t2 = atomicAdd(ticket, 1u + (t1 >> 31));
-    hand_out(2, t2);
+    hand_out(2, tile_of_ticket(t2));
     // From here on a ticket is drawn in one round and handed out at the end of
     // the next: by then it has long been back, and nothing waits for the
     // atomic's round trip.  Round q hands out tile q+3, which the data waves
@@ -441,7 +471,7 @@ __global__ __launch_bounds__(SS_BLOCK) void segscan_kernel(
         }
       }
       if (!ticket_drawn && lane == 0) drawn = atomicAdd(ticket, 1u);
-      hand_out(q + 3, pending);
+      hand_out(q + 3, tile_of_ticket(pending));
       pending = drawn;
       have_p1 = have_cur;
       p1 = cur;
@@ -733,7 +763,8 @@ template <class T> static int64_t scan_num_tiles(int64_t n) {
 template <class T, class Op, class Pre = MapIdentity, class Post = MapIdentity>
 static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int64_t seg_len,
                        int64_t n, int exclusive, void *out, void *scratch, size_t scratch_bytes,
-                       uint32_t epoch, const uint32_t *epoch_dev = nullptr) {
+                       uint32_t epoch, const uint32_t *epoch_dev = nullptr,
+                       ScanTickets tickets = ScanTickets::BY_ARRIVAL) {
   if (n == 0) return 0;
   const int64_t tiles = scan_num_tiles<T>(n);
   if (scratch_bytes < SCAN_HEADER_BYTES + (size_t)tiles * SCAN_DESC_BYTES) return FA_ESCRATCH;
@@ -755,7 +786,8 @@ static int launch_scan(hipStream_t s, const void *xs, const uint8_t *flags, int6
         (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);          \
     if (raised != hipSuccess) return (int)raised;                                              \
     hipLaunchKernelGGL(kernel, grid, block, lds_bytes, s, (const T *)xs, flags, n, (T *)out,   \
-                       header, desc, epoch, epoch_dev, tiles, seg_len);                        \
+                       header, desc, epoch, epoch_dev, tiles, seg_len,                         \
+                       tickets == ScanTickets::BY_ARRIVAL ? 1u : 0u);                          \
   } while (0)
   if (seg_len > 0) {
     if (exclusive) FA_LAUNCH(SEG_ROWS, true);
@@ -840,7 +872,8 @@ __device__ __forceinline__ T block_fold_ordered(T v, T *lds /* BLOCK/64 slots */
 template <class Tin, class T, class Pre, class Op>
 __global__ __launch_bounds__(RED_BLOCK) void reduce_kernel(const Tin *__restrict__ xs, int64_t n,
                                                            T *__restrict__ out, uint32_t *ticket,
-                                                           uint64_t *desc, uint32_t epoch) {
+                                                           uint64_t *desc, uint32_t epoch,
+                                                           bool vectors) {
   constexpr int PER = 4;
   __shared__ T lds[RED_BLOCK / WAVE];
   __shared__ uint32_t s_ticket;
@@ -849,8 +882,45 @@ __global__ __launch_bounds__(RED_BLOCK) void reduce_kernel(const Tin *__restrict
 
   T v = Op::identity();
   if constexpr (Op::commutative) {
+    // As the library's own reduction reads (segred_nonseg_kernel): 16 bytes per
+    // load with the non-temporal policy, two loads in flight per thread, the
+    // map applied to every element with its own index.  Inputs whose base is not
+    // 16-byte aligned, and element types that do not divide 16 bytes, are read
+    // element by element.
+    constexpr bool VECTORS = 16 % sizeof(Tin) == 0 && sizeof(Tin) <= 8;
     const int64_t stride = (int64_t)gridDim.x * RED_BLOCK;
     int64_t i = (int64_t)blockIdx.x * RED_BLOCK + threadIdx.x;
+    int64_t done = 0;  // elements [0, done) are covered by vector loads
+    if constexpr (VECTORS) {
+      if (vectors) {
+        constexpr int VEC = 16 / (int)sizeof(Tin);
+        constexpr int UNROLL = 2;
+        const int64_t nvec = n / VEC;
+        T acc[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] = Op::identity();
+        int64_t j = i;
+        for (; j + (UNROLL - 1) * stride < nvec; j += UNROLL * stride) {
+          Vec16<Tin> x[UNROLL];
+#pragma unroll
+          for (int u = 0; u < UNROLL; u++) x[u] = load_vec16_nt(xs + (j + u * stride) * VEC);
+#pragma unroll
+          for (int u = 0; u < UNROLL; u++)
+#pragma unroll
+            for (int e = 0; e < VEC; e++)
+              acc[e] = Op::apply(acc[e], Pre::apply(x[u].e[e], (j + u * stride) * VEC + e));
+        }
+        for (; j < nvec; j += stride) {
+          const Vec16<Tin> x = load_vec16_nt(xs + j * VEC);
+#pragma unroll
+          for (int e = 0; e < VEC; e++) acc[e] = Op::apply(acc[e], Pre::apply(x.e[e], j * VEC + e));
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; e++) v = Op::apply(v, acc[e]);
+        done = nvec * VEC;
+      }
+    }
+    i += done;
     for (; i + (PER - 1) * stride < n; i += PER * stride) {
       Tin x[PER];
 #pragma unroll
@@ -919,7 +989,208 @@ static int launch_reduce(hipStream_t s, const Tin *xs, int64_t n, T *out, void *
   uint32_t *ticket = (uint32_t *)scratch;
   uint64_t *desc = (uint64_t *)((char *)scratch + RED_HEADER_BYTES);
   hipLaunchKernelGGL((reduce_kernel<Tin, T, Pre, Op>), dim3(grid), dim3(RED_BLOCK), 0, s, xs, n, out,
-                     ticket, desc, epoch);
+                     ticket, desc, epoch, is_aligned(xs, 16));
+  return launch_status();
+}
+
+// ===========================================================================
+// Segmented reductions with a fused map, for operators over 4- or 8-byte
+// elements.
+//
+// Regular segments, `map (\row -> reduce op ne (map f row)) xss` with
+// xss : [m][k] (SegRed.hs:396-636): a row is folded by a group of G lanes
+// (1 to 64, a power of two, chosen from k) or, when it is long, by a block.
+// Element j of a row enters as Pre::apply(x, j), j its position in the row.
+// Operands keep their order whatever the operator: a round of a group is G
+// consecutive elements, folded across the lanes in lane order (an inclusive
+// scan over the wave restricted to the group), and rounds are folded in turn;
+// operators that commute skip the per-round fold and fold the lanes once at
+// the end.
+constexpr int SEGRED_T_BLOCK = 256;
+constexpr int64_t SEGRED_T_LONG = 16384;  // rows longer than this get a block each
+
+// Fold over the G lanes of a group (groups are aligned, G a power of two),
+// result valid in the group's last lane; lane order kept.
+template <class T, class Op, int G> __device__ __forceinline__ T group_fold_ordered(T v) {
+  const T id = Op::identity();
+  if constexpr (G >= 2) v = Op::apply(dpp_move<DPP_ROW_SHR1, 0xf>(id, v), v);
+  if constexpr (G >= 4) v = Op::apply(dpp_move<DPP_ROW_SHR2, 0xf>(id, v), v);
+  if constexpr (G >= 8) v = Op::apply(dpp_move<DPP_ROW_SHR4, 0xf>(id, v), v);
+  if constexpr (G >= 16) v = Op::apply(dpp_move<DPP_ROW_SHR8, 0xf>(id, v), v);
+  if constexpr (G >= 32) v = Op::apply(dpp_move<DPP_ROW_BCAST15, 0xa>(id, v), v);
+  if constexpr (G >= 64) v = Op::apply(dpp_move<DPP_ROW_BCAST31, 0xc>(id, v), v);
+  return v;
+}
+// The row shifts above pull in the lanes of the group only when the group is a
+// whole row of 16 lanes or more; inside a row a shift crosses group borders,
+// so smaller groups mask what comes from outside.
+template <class T, class Op, int G> __device__ __forceinline__ T small_group_fold_ordered(T v) {
+  static_assert(G < 16, "groups below a DPP row");
+  const int sub = lane_id() % G;
+#pragma unroll
+  for (int d = 1; d < G; d *= 2) {
+    T other;
+    if constexpr (sizeof(T) == 4) {
+      other = bit_cast<T>(__shfl_up(bit_cast<int>(v), d, WAVE));
+    } else {
+      other = bit_cast<T>((unsigned long long)__shfl_up((unsigned long long)bit_cast<uint64_t>(v), d, WAVE));
+    }
+    if (sub >= d) v = Op::apply(other, v);
+  }
+  return v;
+}
+
+template <class Tin, class T, class Pre, class Op, int G>
+__global__ __launch_bounds__(SEGRED_T_BLOCK) void segreduce_group_kernel(const Tin *__restrict__ xss,
+                                                                         int64_t m, int64_t k,
+                                                                         T *__restrict__ out) {
+  const int64_t gthread = (int64_t)blockIdx.x * SEGRED_T_BLOCK + threadIdx.x;
+  const int64_t seg = gthread / G;
+  const int sub = (int)(gthread % G);
+  const bool live = seg < m;
+  const Tin *row = xss + (live ? seg : 0) * k;
+  T acc = Op::identity();
+  auto fold = [](T v) {
+    if constexpr (G >= 16) return group_fold_ordered<T, Op, G>(v);
+    else if constexpr (G > 1) return small_group_fold_ordered<T, Op, G>(v);
+    else return v;
+  };
+  if constexpr (Op::commutative) {
+    if (live)
+      for (int64_t j = sub; j < k; j += G) acc = Op::apply(acc, Pre::apply(row[j], j));
+    acc = fold(acc);
+  } else {
+    // Every lane of the wave takes part in every round (the folds move data
+    // across lanes), so the trip count is that of the longest row: k for all.
+    for (int64_t j0 = 0; j0 < k; j0 += G) {
+      const int64_t j = j0 + sub;
+      const T mine = live && j < k ? Pre::apply(row[j], j) : Op::identity();
+      const T round = fold(mine);  // in the group's last lane: elements j0 .. j0 + G - 1
+      acc = Op::apply(acc, round);
+    }
+  }
+  if (live && sub == G - 1) out[seg] = acc;
+}
+
+template <class Tin, class T, class Pre, class Op>
+__global__ __launch_bounds__(RED_BLOCK) void segreduce_block_kernel(const Tin *__restrict__ xss,
+                                                                    int64_t m, int64_t k,
+                                                                    T *__restrict__ out) {
+  __shared__ T lds[RED_BLOCK / WAVE];
+  for (int64_t seg = blockIdx.x; seg < m; seg += gridDim.x) {
+    const Tin *row = xss + seg * k;
+    T acc = Op::identity();
+    if constexpr (Op::commutative) {
+      for (int64_t j = threadIdx.x; j < k; j += RED_BLOCK) acc = Op::apply(acc, Pre::apply(row[j], j));
+      acc = block_fold_ordered<T, Op, RED_BLOCK>(acc, lds);
+    } else {
+      for (int64_t j0 = 0; j0 < k; j0 += RED_BLOCK) {
+        const int64_t j = j0 + threadIdx.x;
+        const T mine = j < k ? Pre::apply(row[j], j) : Op::identity();
+        acc = Op::apply(acc, block_fold_ordered<T, Op, RED_BLOCK>(mine, lds));
+      }
+    }
+    if (threadIdx.x == 0) out[seg] = acc;
+  }
+}
+
+// out[i] = fold of Pre::apply(xss[i][j], j) over j < k, for i < m.  k == 0
+// gives m neutral elements.
+template <class Tin, class T, class Pre, class Op>
+static int launch_segreduce(hipStream_t s, const Tin *xss, int64_t m, int64_t k, T *out) {
+  static_assert(sizeof(T) == 4 || sizeof(T) == 8, "4- or 8-byte elements");
+  if (m < 0 || k < 0) return FA_EINVAL;
+  if (m == 0) return 0;
+  if (out == nullptr || (k > 0 && xss == nullptr)) return FA_EINVAL;
+  if (k > SEGRED_T_LONG) {
+    int dev = 0, cus = NUM_CUS_HINT;
+    if (hipGetDevice(&dev) == hipSuccess)
+      (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    const int64_t most = (int64_t)cus * 2;
+    hipLaunchKernelGGL((segreduce_block_kernel<Tin, T, Pre, Op>), dim3((unsigned)(m < most ? m : most)),
+                       dim3(RED_BLOCK), 0, s, xss, m, k, out);
+    return launch_status();
+  }
+#define FA_GROUPS(G)                                                                              \
+  do {                                                                                            \
+    const int64_t blocks = ceil_div(m * (G), (int64_t)SEGRED_T_BLOCK);                            \
+    if (blocks > INT32_MAX) return FA_EINVAL;                                                     \
+    hipLaunchKernelGGL((segreduce_group_kernel<Tin, T, Pre, Op, G>), dim3((unsigned)blocks),      \
+                       dim3(SEGRED_T_BLOCK), 0, s, xss, m, k, out);                               \
+  } while (0)
+  if (k <= 2) FA_GROUPS(1);
+  else if (k <= 8) FA_GROUPS(4);
+  else if (k <= 64) FA_GROUPS(16);
+  else FA_GROUPS(64);
+#undef FA_GROUPS
+  return launch_status();
+}
+
+// Irregular segments given as (offset, length) pairs, the way flattening
+// expresses them (Pass/Flatten/Builtins.hs:570-602): flags are written from
+// the offsets, the values are scanned with the flag-tuple operator, and
+// segment i takes the scanned value at its last element, or the neutral
+// element when it is empty.  Segments must tile a prefix of the input in order
+// (offsets[i] + lens[i] == offsets[i+1]); elements behind the last segment are
+// ignored.  workspace: n * (sizeof(T) + 1) bytes rounded up to 16, 16-byte
+// aligned; scratch and epoch as for launch_scan.
+// Clears `units` 16-byte units (a kernel rather than a memset, so that callers
+// may record the launches in a graph).
+static __global__ void clear_units_kernel(uint4 *p, int64_t units) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < units; i += stride)
+    p[i] = uint4{0u, 0u, 0u, 0u};
+}
+template <class T>
+__global__ void segments_to_flags_kernel(const int64_t *__restrict__ offsets,
+                                         const int64_t *__restrict__ lens, int64_t m, int64_t n,
+                                         uint8_t *flags) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < m && lens[i] > 0 && offsets[i] >= 0 && offsets[i] < n) flags[offsets[i]] = 1;
+}
+template <class T, class Op>
+__global__ void segments_gather_kernel(const int64_t *__restrict__ offsets,
+                                       const int64_t *__restrict__ lens, int64_t m, int64_t n,
+                                       const T *__restrict__ scanned, T *__restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= m) return;
+  const int64_t last = offsets[i] + lens[i] - 1;
+  out[i] = lens[i] > 0 && last >= 0 && last < n ? scanned[last] : Op::identity();
+}
+template <class T> static size_t segreduce_irregular_workspace_bytes(int64_t n) {
+  return (((size_t)n * sizeof(T) + 15) & ~(size_t)15) + (((size_t)n + 15) & ~(size_t)15);
+}
+template <class T, class Op, class Pre = MapIdentity>
+static int launch_segreduce_irregular(hipStream_t s, const int64_t *offsets, const int64_t *lens,
+                                      int64_t m, const T *xs, int64_t n, T *out, void *workspace,
+                                      size_t workspace_bytes, void *scratch, size_t scratch_bytes,
+                                      uint32_t epoch) {
+  if (m < 0 || n < 0) return FA_EINVAL;
+  if (m == 0) return 0;
+  if (offsets == nullptr || lens == nullptr || out == nullptr) return FA_EINVAL;
+  if (m > (int64_t)INT32_MAX * 256) return FA_EINVAL;
+  const dim3 per_segment((unsigned)ceil_div(m, (int64_t)256));
+  if (n > 0) {
+    if (xs == nullptr || workspace == nullptr) return FA_EINVAL;
+    if (workspace_bytes < segreduce_irregular_workspace_bytes<T>(n)) return FA_ESCRATCH;
+    if (!is_aligned(workspace, 16)) return FA_EALIGN;
+    T *scanned = (T *)workspace;
+    uint8_t *flags = (uint8_t *)workspace + (((size_t)n * sizeof(T) + 15) & ~(size_t)15);
+    const int64_t units = ceil_div(n, (int64_t)16);
+    const int64_t clear_blocks = ceil_div(units, (int64_t)256);
+    hipLaunchKernelGGL(clear_units_kernel, dim3((unsigned)(clear_blocks < 4096 ? clear_blocks : 4096)),
+                       dim3(256), 0, s, (uint4 *)flags, units);
+    int rc0 = launch_status();
+    if (rc0 != 0) return rc0;
+    hipLaunchKernelGGL(segments_to_flags_kernel<T>, per_segment, dim3(256), 0, s, offsets, lens, m, n,
+                       flags);
+    int rc = launch_status();
+    if (rc != 0) return rc;
+    rc = launch_scan<T, Op, Pre>(s, xs, flags, (int64_t)0, n, 0, scanned, scratch, scratch_bytes, epoch);
+    if (rc != 0) return rc;
+  }
+  hipLaunchKernelGGL((segments_gather_kernel<T, Op>), per_segment, dim3(256), 0, s, offsets, lens, m, n,
+                     (const T *)workspace, out);
   return launch_status();
 }
 
@@ -946,16 +1217,26 @@ constexpr int HL_MAX_BINS = 8192;
 // loop body, in the same trip; written as "spin until the lock is mine, then
 // update", the compiler places the update behind the spin loop, where lanes
 // that hold a lock wait for the lanes of their own wave that spin on it.
-template <class P, class Op, class F> __device__ __forceinline__ void hl_with_lock(uint32_t *lock, F &&update) {
+// BACKOFF (locks in global memory): a trip in which no lane of the wave got its
+// lock is followed by a pause, so that the waves that wait do not keep the
+// lock's memory channel busy with attempts while its holder needs it to
+// release.
+template <class P, class Op, bool BACKOFF = false, class F>
+__device__ __forceinline__ void hl_with_lock(uint32_t *lock, F &&update) {
   bool waiting = true;
   while (__ballot(waiting) != 0) {
+    bool got = false;
     if (waiting) {
       if (atomicCAS(lock, 0u, 1u) == 0u) {
         update();
         __threadfence();
         atomicExch(lock, 0u);
         waiting = false;
+        got = true;
       }
+    }
+    if constexpr (BACKOFF) {
+      if (__ballot(got) == 0) __builtin_amdgcn_s_sleep(32);
     }
   }
 }
@@ -1011,20 +1292,40 @@ __global__ __launch_bounds__(HL_BLOCK) void hist_locked_kernel(const I *__restri
   }
 }
 
-// More bins than a block's LDS holds: every update locks its bin in the
-// destination itself (the reference's pass over global memory with locks,
-// SegHist.hs:377-467 with Base.hs:769-842; one sub-histogram, hist_M = 1).
+// More bins than a block's LDS holds (the reference's pass over global memory
+// with locks, SegHist.hs:377-467 with Base.hs:769-842).  Locking a bin of the
+// destination for every update is only bearable while updates to a bin are
+// rare: under skewed indices thousands of waves queue on the locks of a few
+// bins, and same-address atomics are performed one at a time.  So a block keeps
+// HL_MAX_BINS slots in LDS as a cache of the bins it meets: slot bin mod
+// HL_MAX_BINS belongs to the first bin that claims it (a tag word, claimed by
+// compare-and-swap, never given up), updates of that bin are made in the slot
+// under the slot's LDS lock, and only updates of other bins that map to a taken
+// slot go to the destination under the bin's global lock.  Frequent bins get
+// their slots early and stay out of global memory; at the end the block merges
+// its slots into the destination.
 template <class Tin, class A, class B, class P, class Pre, class Op, class I>
-__global__ __launch_bounds__(HL_BLOCK) void hist_locked_global_kernel(const I *__restrict__ is,
+__global__ __launch_bounds__(HL_BLOCK) void hist_locked_cached_kernel(const I *__restrict__ is,
                                                                       const Tin *__restrict__ xs,
                                                                       int64_t n, A *dest_a, B *dest_b,
                                                                       uint32_t *locks, int64_t H) {
-  const int64_t stride = (int64_t)gridDim.x * HL_BLOCK;
-  for (int64_t i = (int64_t)blockIdx.x * HL_BLOCK + threadIdx.x; i < n; i += stride) {
-    const int64_t bin = (int64_t)is[i];
-    if ((uint64_t)bin >= (uint64_t)H) continue;  // out of range: ignored
-    const P mine = Pre::apply(xs[i], i);
-    hl_with_lock<P, Op>(&locks[bin], [&] {
+  extern __shared__ __align__(16) unsigned char hl_lds[];
+  constexpr int SLOTS = HL_MAX_BINS;
+  static_assert((SLOTS & (SLOTS - 1)) == 0, "slot = bin mod a power of two");
+  volatile A *sa = reinterpret_cast<volatile A *>(hl_lds);
+  volatile B *sb = reinterpret_cast<volatile B *>(hl_lds + (size_t)SLOTS * sizeof(A));
+  uint32_t *sl = reinterpret_cast<uint32_t *>(hl_lds + (size_t)SLOTS * (sizeof(A) + sizeof(B)));
+  uint32_t *tag = sl + SLOTS;  // bin + 1 of the slot's owner, 0 while free
+  const P ne = Op::identity();
+  for (int i = threadIdx.x; i < SLOTS; i += HL_BLOCK) {
+    sa[i] = ne.a;
+    sb[i] = ne.b;
+    sl[i] = 0u;
+    tag[i] = 0u;
+  }
+  __syncthreads();
+  auto update_global = [&](int64_t bin, const P &mine) {
+    hl_with_lock<P, Op, true>(&locks[bin], [&] {
       P cur;
       cur.a = __hip_atomic_load(dest_a + bin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       cur.b = __hip_atomic_load(dest_b + bin, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1032,13 +1333,49 @@ __global__ __launch_bounds__(HL_BLOCK) void hist_locked_global_kernel(const I *_
       __hip_atomic_store(dest_a + bin, r.a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(dest_b + bin, r.b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     });
+  };
+  const int64_t stride = (int64_t)gridDim.x * HL_BLOCK;
+  for (int64_t i = (int64_t)blockIdx.x * HL_BLOCK + threadIdx.x; i < n; i += stride) {
+    const int64_t bin = (int64_t)is[i];
+    if ((uint64_t)bin >= (uint64_t)H) continue;  // out of range: ignored
+    const P mine = Pre::apply(xs[i], i);
+    const int slot = (int)(bin & (SLOTS - 1));
+    const uint32_t want = (uint32_t)bin + 1u;
+    uint32_t owner = __hip_atomic_load(&tag[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (owner == 0u) {
+      const uint32_t seen = atomicCAS(&tag[slot], 0u, want);
+      owner = seen == 0u ? want : seen;
+    }
+    if (owner == want) {
+      hl_with_lock<P, Op>(&sl[slot], [&] {
+        P cur;
+        cur.a = sa[slot];
+        cur.b = sb[slot];
+        const P r = Op::apply(cur, mine);
+        sa[slot] = r.a;
+        sb[slot] = r.b;
+      });
+    } else {
+      update_global(bin, mine);
+    }
+  }
+  __syncthreads();
+  for (int slot = threadIdx.x; slot < SLOTS; slot += HL_BLOCK) {
+    const uint32_t owner = tag[slot];
+    if (owner == 0u) continue;
+    P mine;
+    mine.a = sa[slot];
+    mine.b = sb[slot];
+    if (bits_equal_pair(mine, ne)) continue;
+    update_global((int64_t)owner - 1, mine);
   }
 }
 
 // dest_a, dest_b: H bins each, holding the values to combine with (as
 // reduce_by_index takes them); locks: H 32-bit words, all zero, zero again
-// afterwards.  Up to HL_MAX_BINS bins are accumulated per block in LDS; more
-// are updated in place under the locks.
+// afterwards.  Up to HL_MAX_BINS bins are accumulated per block in LDS; with
+// more, a block caches the bins it meets first in LDS and updates the others
+// in place under the locks.
 template <class Tin, class A, class B, class P, class Pre, class Op, class I>
 static int launch_hist_locked(hipStream_t s, const I *is, const Tin *xs, int64_t n, A *dest_a,
                               B *dest_b, uint32_t *locks, int64_t H) {
@@ -1051,11 +1388,16 @@ static int launch_hist_locked(hipStream_t s, const I *is, const Tin *xs, int64_t
   if (hipGetDevice(&dev) == hipSuccess)
     (void)hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   if (H > HL_MAX_BINS) {
-    const int64_t want = ceil_div(n, (int64_t)HL_BLOCK * 4);
-    const int64_t most = (int64_t)cus * 8;
-    const int grid = (int)(want < 1 ? 1 : (want > most ? most : want));
-    hipLaunchKernelGGL((hist_locked_global_kernel<Tin, A, B, P, Pre, Op, I>), dim3(grid), dim3(HL_BLOCK),
-                       0, s, is, xs, n, dest_a, dest_b, locks, H);
+    if (H > ((int64_t)1 << 31)) return FA_EINVAL;  // a slot's tag is bin + 1 in 32 bits
+    auto cached = hist_locked_cached_kernel<Tin, A, B, P, Pre, Op, I>;
+    constexpr int cached_lds = HL_MAX_BINS * (int)(sizeof(A) + sizeof(B) + 8);
+    static const hipError_t raised_cached = hipFuncSetAttribute(
+        (const void *)cached, hipFuncAttributeMaxDynamicSharedMemorySize, cached_lds);
+    if (raised_cached != hipSuccess) return (int)raised_cached;
+    const int64_t want = ceil_div(n, (int64_t)HL_BLOCK * 8);
+    const int grid = (int)(want < 1 ? 1 : (want > cus ? cus : want));
+    hipLaunchKernelGGL(cached, dim3(grid), dim3(HL_BLOCK), cached_lds, s, is, xs, n, dest_a, dest_b,
+                       locks, H);
     return launch_status();
   }
   const size_t lds = (size_t)H * (sizeof(A) + sizeof(B) + 4);

@@ -353,7 +353,18 @@ int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhar
  *   entry scan_norm_f32 (xs: []f32) : []f32 = map f32.sqrt (scan (+) 0 (map (\x -> x * x) xs))
  *   entry rows_fraction_f32 (xss: [][]f32) : [][]f32 =
  *     map (\r -> let t = reduce (+) 0 r in map (/ t) (scan (+) 0 r)) xss
- *                                   -- SegOps at block level, ImpGen/GPU/Block.hs:357-615 */
+ *                                   -- SegOps at block level, ImpGen/GPU/Block.hs:357-615
+ * The same operators in the segmented forms (SegRed.hs:396-636,
+ * SegScan/SinglePass.hs:327-361, Pass/Flatten/Builtins.hs:570-602):
+ *   entry segreduce_argmax_i32 [m][k] (xss: [m][k]i32) : [m][2]i32 =
+ *     map (\row -> reduce_comm argmax (i32.lowest, i32.highest) (zip row (map i32.i64 (iota k)))) xss
+ *     |> map (\(v, i) -> [v, i])
+ *   entry segreduce_compose_i32 (k: i64) (abs: [][2]i32) : [][2]i32 =   -- rows of k maps each
+ *     map (reduce compose (1, 0)) (unflatten (map (\r -> (r[0], r[1])) abs)) |> map (\(a, b) -> [a, b])
+ *   entry scanrows_argmax_i32 (k: i64) (vis: [][2]i32) : [][2]i32 =     -- rows of k pairs each
+ *     map (scan argmax (i32.lowest, i32.highest)) (unflatten ...) |> flatten
+ *   entry segred_argmax_i32 [m] (offsets: [m]i64) (lens: [m]i64) (vis: [][2]i32) : [m][2]i32
+ *     -- segred_OP_T above with argmax over the pairs */
 int futhark_entry_reduce_argmax_i32(struct futhark_context *ctx, struct futhark_i32_1d **out0,
                                     const struct futhark_i32_1d *in0);
 int futhark_entry_scan_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
@@ -371,6 +382,16 @@ int futhark_entry_scan_norm_f32(struct futhark_context *ctx, struct futhark_f32_
                                 const struct futhark_f32_1d *in0);
 int futhark_entry_rows_fraction_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,
                                     const struct futhark_f32_2d *in0);
+int futhark_entry_segreduce_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                       const struct futhark_i32_2d *in0);
+int futhark_entry_segreduce_compose_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                        const int64_t in0, const struct futhark_i32_2d *in1);
+int futhark_entry_scanrows_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                      const int64_t in0, const struct futhark_i32_2d *in1);
+int futhark_entry_segred_argmax_i32(struct futhark_context *ctx, struct futhark_i32_2d **out0,
+                                    const struct futhark_i64_1d *in0,
+                                    const struct futhark_i64_1d *in1,
+                                    const struct futhark_i32_2d *in2);
 int futhark_entry_bmm_bf16(struct futhark_context *ctx, struct futhark_f32_3d **out0,
                            const struct futhark_u16_3d *in0, const struct futhark_u16_3d *in1);
 int futhark_entry_matmul_f32(struct futhark_context *ctx, struct futhark_f32_2d **out0,

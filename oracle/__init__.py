@@ -187,6 +187,58 @@ def hist_argmax_i32(k: int, is_, xs):
     return dest
 
 
+def segreduce_argmax_i32(xss):
+    """map (\\row -> argmax over zip row (iota k)) xss -> [m][2]: the largest value of a row
+    and the first column that holds it; (i32.lowest, i32.highest) for rows of no elements."""
+    xss = _arr(xss, np.int32)
+    m, k = xss.shape
+    out = np.empty((m, 2), np.int32)
+    if k == 0:
+        out[:] = (np.iinfo(np.int32).min, np.iinfo(np.int32).max)
+        return out
+    first = np.argmax(xss, axis=1)          # numpy returns the first of equal maxima
+    out[:, 0] = xss[np.arange(m), first]
+    out[:, 1] = first
+    return out
+
+
+def segreduce_compose_i32(k: int, abs_):
+    """Rows of k affine maps composed in element order -> [m][2] (the sequential scan of
+    orc_scan_compose_i32_lit restarted at every row, read at the rows' last elements)."""
+    abs_ = _arr(abs_, np.int32).reshape(-1, 2)
+    if k == 0:
+        return np.zeros((0, 2), np.int32)
+    flags = np.zeros(abs_.shape[0], np.uint8)
+    flags[::k] = 1
+    return scan_compose_i32(abs_, flags)[k - 1::k].copy()
+
+
+def scanrows_argmax_i32(k: int, vis):
+    vis = _arr(vis, np.int32).reshape(-1, 2)
+    if k == 0:
+        return vis.copy()
+    flags = np.zeros(vis.shape[0], np.uint8)
+    flags[::k] = 1
+    return scan_argmax_i32(vis, flags)
+
+
+def segred_argmax_i32(offsets, lens, vis):
+    """Builtins.hs:570-602 with the argmax operator: flags from the offsets, segmented scan,
+    the scanned pair at the last element of every segment, the neutral pair for empty ones."""
+    vis = _arr(vis, np.int32).reshape(-1, 2)
+    offsets, lens = _arr(offsets, np.int64), _arr(lens, np.int64)
+    out = np.empty((offsets.size, 2), np.int32)
+    out[:] = (np.iinfo(np.int32).min, np.iinfo(np.int32).max)
+    if vis.shape[0] == 0:
+        return out
+    flags = np.zeros(vis.shape[0], np.uint8)
+    flags[offsets[lens > 0]] = 1
+    sc = scan_argmax_i32(vis, flags)
+    live = lens > 0
+    out[live] = sc[offsets[live] + lens[live] - 1]
+    return out
+
+
 def reduce_compose_i32(abs_):
     """reduce compose (1, 0) abs: the last element of the scan, (1, 0) for no elements."""
     abs_ = _arr(abs_, np.int32).reshape(-1, 2)

@@ -117,3 +117,50 @@ def test_two_operators_in_one_reduction(ctx):
         assert got.shape == (2,)
         assert abs(float(got[0]) - float(want[0])) <= 1e-5 * float(np.abs(xs).sum(dtype=np.float64)) + 1e-30, n
         assert float(got[1]) == float(want[1]) or (n == 0 and np.isneginf(got[1])), n
+
+
+def test_custom_operators_in_the_segmented_forms(ctx):
+    """The program's own operators in `map (reduce op ne)`, `map (scan op ne)` and over irregular
+    segments: argmax (a tuple, made from the row by a fused map) and composition of affine maps
+    (not commutative, so every row must be folded in element order).  Row lengths on both sides
+    of every change of lane-group size and of the change to one block per row; bit-exact."""
+    rng = np.random.default_rng(8)
+    for m, k in [(0, 5), (3, 0), (1, 1), (1000, 2), (999, 3), (513, 8), (300, 9), (77, 64), (50, 65),
+                 (9, 1000), (5, 16384), (3, 16385), (2, 100003), (70000, 5)]:
+        xss = rng.integers(-50, 50, (m, k)).astype(np.int32)     # ties in every row
+        a = ctx.new("i32_2d", xss)
+        out = ctx.call("segreduce_argmax_i32", ["i32_2d"], a)
+        assert out.shape == (m, 2)
+        assert np.array_equal(out.values(), oracle.segreduce_argmax_i32(xss)), (m, k)
+        out.free(); a.free()
+        abs_ = rng.integers(-2**31, 2**31, (m * k, 2), dtype=np.int64).astype(np.int32)
+        a = ctx.new("i32_2d", abs_)
+        if k > 0:
+            out = ctx.call("segreduce_compose_i32", ["i32_2d"], k, a)
+            assert out.shape == (m, 2)
+            assert np.array_equal(out.values(), oracle.segreduce_compose_i32(k, abs_)), (m, k)
+            out.free()
+            vis = np.stack([rng.integers(-50, 50, m * k), np.arange(m * k) % k], axis=1).astype(np.int32)
+            v = ctx.new("i32_2d", vis)
+            out = ctx.call("scanrows_argmax_i32", ["i32_2d"], k, v)
+            assert np.array_equal(out.values(), oracle.scanrows_argmax_i32(k, vis)), (m, k)
+            out.free(); v.free()
+        a.free()
+    bad = ctx.new("i32_2d", np.zeros((10, 2), np.int32))
+    for entry in ("segreduce_compose_i32", "scanrows_argmax_i32"):
+        with pytest.raises(FutharkError, match="invalid sizes"):
+            ctx.call(entry, ["i32_2d"], 3, bad)          # 10 pairs are no rows of 3
+    bad.free()
+    # irregular segments: geometric lengths with empty segments in between, and pairs behind
+    # the last segment that belong to nobody
+    for n, mean in [(0, 4), (1, 1), (5000, 3), (300007, 50), ((1 << 21) + 11, 1000)]:
+        lens = rng.geometric(1.0 / mean, max(1, n // mean) + 5).astype(np.int64) - 1 if n else np.zeros(3, np.int64)
+        lens = lens[np.cumsum(lens) <= n]
+        offsets = np.concatenate(([0], np.cumsum(lens)[:-1])).astype(np.int64) if lens.size else np.zeros(0, np.int64)
+        vis = np.stack([rng.integers(-50, 50, n), np.arange(n)], axis=1).astype(np.int32)
+        o, l, v = ctx.new("i64_1d", offsets), ctx.new("i64_1d", lens), ctx.new("i32_2d", vis)
+        out = ctx.call("segred_argmax_i32", ["i32_2d"], o, l, v)
+        assert out.shape == (lens.size, 2)
+        assert np.array_equal(out.values(), oracle.segred_argmax_i32(offsets, lens, vis)), (n, mean)
+        for h in (o, l, v, out):
+            h.free()

@@ -34,6 +34,11 @@ def make_inputs(name, e, rng):
     types = [i["type"] for i in e["inputs"]]
     el = lambda ty: ty.lstrip("[]")
     fam = name.split("_")[0]
+    if name in ("segreduce_compose_i32", "scanrows_argmax_i32"):
+        return [np.array(4, np.int64), _vals(rng, "i32", (36, 2))]       # nine rows of four
+    if name == "segred_argmax_i32":
+        return [np.array([0, 10, 10, 30], np.int64), np.array([10, 0, 20, 7], np.int64),
+                _vals(rng, "i32", (N, 2))]
     if name.startswith("rbi_vec"):
         t = el(types[0])
         return [_vals(rng, t, (5, 3)), rng.integers(-1, 6, N).astype(np.int64), _vals(rng, t, (N, 3))]
@@ -60,10 +65,11 @@ def make_inputs(name, e, rng):
     if fam in ("segreduce", "scanrows", "vecreduce", "vecscan"):
         return [_vals(rng, el(types[0]), (6, 7))]
     if fam == "hist":
-        return [np.array(5, np.int64), rng.integers(-1, 7, N).astype(np.int32), _vals(rng, el(types[2]), N)]
+        return [np.array(5, np.int64), rng.integers(-1, 7, N).astype(NP[el(types[1])]),
+                _vals(rng, el(types[2]), N)]
     if fam == "rbi":
         t = el(types[0])
-        return [_vals(rng, t, 5), rng.integers(-1, 7, N).astype(np.int32), _vals(rng, t, N)]
+        return [_vals(rng, t, 5), rng.integers(-1, 7, N).astype(NP[el(types[1])]), _vals(rng, t, N)]
     if fam == "seghist":
         return [np.array(5, np.int64), rng.integers(-1, 7, (3, N)).astype(np.int32),
                 _vals(rng, el(types[2]), (3, N))]
@@ -163,12 +169,24 @@ def test_every_entry_point_through_the_c_api_and_the_server(ctx, server, tmp_pat
             assert a.shape == b.shape and a.tobytes() == b.tobytes(), name
         # -- a few families against the oracle as well (exact: whole numbers)
         fam, parts = name.split("_")[0], name.split("_")
-        if fam in ("vecreduce", "segreduce") and parts[2] in ("i32", "i64", "f32", "f64"):
+        if fam in ("vecreduce", "segreduce") and parts[1] not in ("argmax", "compose") \
+                and parts[2] in ("i32", "i64", "f32", "f64"):
             want = getattr(oracle, fam)(parts[1], parts[2], ins[0])
             assert np.array_equal(via_api[0], want), name
         if name.startswith("rbi_2d"):
             assert np.array_equal(via_api[0], oracle.rbi_2d(parts[2], parts[3], *ins)), name
         if name.startswith("rbi_vec"):
             assert np.array_equal(via_api[0], oracle.rbi_vec(parts[2], parts[3], *ins)), name
+        if fam in ("hist", "rbi") and parts[1] != "argmax" and parts[-1] == "i64" and len(parts) == 4 \
+                and parts[2] in ("i32", "i64", "f32", "f64"):
+            # the []i64 forms against the oracle, which takes 32-bit indices
+            narrow = [ins[0], ins[1].astype(np.int32), ins[2]]
+            want = oracle.hist(parts[1], parts[2], int(ins[0]), *narrow[1:]) if fam == "hist" \
+                else oracle.rbi(parts[1], parts[2], *narrow)
+            assert np.array_equal(via_api[0], want), name
+        if name in ("segreduce_argmax_i32", "segreduce_compose_i32", "scanrows_argmax_i32",
+                    "segred_argmax_i32"):
+            assert np.array_equal(via_api[0], getattr(oracle, name)(*[x.item() if x.ndim == 0 else x
+                                                                      for x in ins])), name
         checked += 1
     assert checked == len(MANIFEST["entry_points"]) > 300

@@ -211,3 +211,34 @@ def test_scalar_results_arrive_at_the_synchronisation(segops_lib):
         assert sq.value == 30.0
         for a in arrays + [f]:
             a.free()
+
+
+def test_scans_under_both_ways_of_picking_ticket_counters(segops_lib):
+    """The blocks of the single-pass scan pick their ticket counter by block index while the
+    context is alone in the process (no arrival atomic), by order of arrival otherwise or when
+    `segops.scan_arrival_tickets` says so.  Same results either way: a context of its own with
+    the parameter set, a second context alive beside it (both then take the order of arrival),
+    and hundreds of tiles, a few tiles and fewer tiles than counters."""
+    import oracle
+    from futhark_amd import datagen as dg
+
+    def check(c):
+        for n in (5, 40000, 100003, (1 << 22) + 77):
+            xs = dg.uniform_int(7, n, -1000, 1000, np.int32)
+            flags = (dg.raw_u64(9, n) % np.uint64(900) == 0).astype(np.uint8)
+            a, f = c.new("i32_1d", xs), c.new("u8_1d", flags)
+            out = c.call("scan_add_i32", ["i32_1d"], a)
+            assert np.array_equal(out.values(), oracle.scan("add", "i32", xs)), n
+            out.free()
+            out = c.call("segscan_max_i32", ["i32_1d"], f, a)
+            assert np.array_equal(out.values(), oracle.segscan("max", "i32", flags, xs)), n
+            for h in (out, a, f):
+                h.free()
+
+    with Context(segops_lib, tuning={"segops.scan_arrival_tickets": 1}) as c1:
+        check(c1)
+        with Context(segops_lib) as c2:      # two contexts alive: neither assumes the device is its own
+            check(c2)
+            check(c1)
+    with Context(segops_lib) as c3:
+        check(c3)

@@ -510,7 +510,15 @@ def test_scan_with_a_vector_operator(ctx, t, op):
     for n, k in [(1, 1), (1000, 1), (7, 3), (1, 300), (1000, 4), (333, 33), (40001, 5), (70, 1000),
                  (20000, 64), (0, 4), (4, 0),
                  # rows of whole 1 KiB strips take the kernels without a transposed copy
-                 (5, 256), (1000, 256), (40001, 512), (17, 1024), (1, 768), (3000, 128), (16385, 256)]:
+                 (5, 256), (1000, 256), (40001, 512), (17, 1024), (1, 768), (3000, 128), (16385, 256),
+                 # ... and so do rows of whole 16-byte units: a last strip that is not full,
+                 (1000, 100), (40001, 68), (333, 260), (50, 1028), (9, 300000),
+                 # rows of 16 to 128 bytes, several to a wave-wide load (ragged last loads,
+                 # fewer rows than a load holds, many chunks),
+                 (1, 4), (63, 4), (64, 4), (65, 4), (100003, 4), (5000, 8), (70001, 16), (33, 32),
+                 (1 << 20, 4), (300000, 2),
+                 # and enough strips to fill the chip with one chunk: the input is read once
+                 (100, 1 << 18), (17, (1 << 18) + 4)]:
         xss = _data(t, n * k, 17).reshape(n, k)
         out = ctx.call(f"vecscan_{op}_{t}", [f"{t}_2d"], ctx.new(f"{t}_2d", xss))
         got = out.values()

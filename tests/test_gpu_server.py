@@ -45,7 +45,7 @@ def test_introspection(srv):
     types = srv.cmd("types")
     assert {"i32", "[]f32", "[][]f32", "[][][]f16", "([]u32, []i32)"} <= set(types)
     entries = srv.cmd("entry_points")
-    assert len(entries) == (4 * 3 + 2 * 3) * 14 + (6 * 6 + 3) * 2 + 22 and "segscan_add_f32" in entries
+    assert len(entries) == (4 * 3 + 2 * 3) * 16 + (6 * 6 + 3) * 4 + 26 and "segscan_add_f32" in entries
     from futhark_amd import manifest
     m = manifest.manifest()            # the server and the manifest describe the same API
     assert set(entries) == set(m["entry_points"])

@@ -195,14 +195,21 @@ def test_the_model_notices_a_broken_protocol():
 # resident blocks take their steps, with at most R blocks resident, and asks
 # whether a state is reachable from which nothing can move before all tiles are
 # done.  Two rules for choosing the counter:
-#   "arrival": the k-th block to START uses counter k mod C (what the kernel does);
-#   "index":   block b uses counter b mod C, whatever the order of starts.
+#   "arrival": the k-th block to START uses counter k mod C (the kernel's default);
+#   "index":   block b uses counter b mod C, whatever the order of starts;
+#   "static":  as "index", and the first two tiles of block b are b and b + G
+#              without a ticket, the counters handing out tiles 2 G and up (what
+#              the kernel does for callers that say the launch has the device to
+#              itself).
 def _ticket_model_deadlocks(rule, G, C, R, tiles):
-    """True when some schedule gets stuck.  A block: draw a tile from its counter;
-    publish the tile's aggregate; look back (needs the aggregates of all earlier
-    tiles); draw again.  It leaves on a ticket beyond the last tile."""
-    # state: (counters, started mask, blocks) with blocks = tuple over block ids of
-    # None (not started / left) or (counter, tile or None, published?)
+    """True when some schedule gets stuck.  A block: take its next tile (by ticket from its
+    counter, or by its index for the first two tiles under "static"); publish the tile's
+    aggregate; look back (needs the aggregates of all earlier tiles); take the next.  It
+    leaves on a tile beyond the last one."""
+    base = 2 * G if rule == "static" else 0   # first tile the counters hand out
+
+    # state: (counters, started mask, left mask, blocks, done mask) with blocks = tuple over
+    # block ids of None (not started / left) or (counter, tiles taken, tile or None, published?)
     def moves(state):
         counters, started, left, blocks, done = state
         out = []
@@ -213,30 +220,37 @@ def _ticket_model_deadlocks(rule, G, C, R, tiles):
                     k = bin(started).count("1")
                     c = (k if rule == "arrival" else b) % C
                     nb = list(blocks)
-                    nb[b] = (c, None, False)
+                    nb[b] = (c, 0, None, False)
                     out.append((counters, started | (1 << b), left, tuple(nb), done))
                     if rule == "arrival":
                         break  # blocks are interchangeable until they have a counter
         for b, blk in enumerate(blocks):
             if blk is None:
                 continue
-            c, tile, published = blk
+            c, taken, tile, published = blk
             nb = list(blocks)
-            if tile is None:  # draw
-                t = counters[c] * C + c
+            if tile is None:  # take the next tile
                 nc = list(counters)
-                nc[c] += 1
+                if rule == "static" and taken < 2:
+                    t = b + taken * G
+                    if t >= tiles:       # nothing here; the block goes on to its counter
+                        nb[b] = (c, taken + 1, None, False)
+                        out.append((counters, started, left, tuple(nb), done))
+                        continue
+                else:
+                    t = base + counters[c] * C + c
+                    nc[c] += 1
                 if t >= tiles:
                     nb[b] = None
                     out.append((tuple(nc), started, left | (1 << b), tuple(nb), done))
                 else:
-                    nb[b] = (c, t, False)
+                    nb[b] = (c, taken + 1, t, False)
                     out.append((tuple(nc), started, left, tuple(nb), done))
             elif not published:
-                nb[b] = (c, tile, True)
+                nb[b] = (c, taken, tile, True)
                 out.append((counters, started, left, tuple(nb), done | (1 << tile)))
             elif done & ((1 << tile) - 1) == (1 << tile) - 1:  # every earlier aggregate is there
-                nb[b] = (c, None, False)
+                nb[b] = (c, taken, None, False)
                 out.append((counters, started, left, tuple(nb), done))
         return out
 
@@ -248,6 +262,8 @@ def _ticket_model_deadlocks(rule, G, C, R, tiles):
         finished = st[2] == (1 << G) - 1
         if not nxt and not finished:
             return True
+        if finished:
+            assert st[4] == (1 << tiles) - 1, "every tile was processed"
         for s in nxt:
             if s not in seen:
                 seen.add(s)
@@ -264,6 +280,10 @@ def test_counters_chosen_by_arrival_never_get_stuck():
         for R in range(min(C, G), G + 1):
             assert not _ticket_model_deadlocks("arrival", G, C, R, tiles), (G, C, R)
         assert not _ticket_model_deadlocks("index", G, C, G, tiles)
+        # the whole grid resident: the first two tiles may follow from the block index
+        assert not _ticket_model_deadlocks("static", G, C, G, tiles)
+        assert not _ticket_model_deadlocks("static", G, C, G, 2 * G + 3)
+    assert _ticket_model_deadlocks("static", 4, 2, 3, 7)    # ... and only then
     assert _ticket_model_deadlocks("index", 4, 2, 2, 7)     # blocks 0 and 2 run: counter 1 starves
     assert _ticket_model_deadlocks("index", 6, 3, 4, 8)
     assert _ticket_model_deadlocks("arrival", 4, 2, 1, 7)   # the stated requirement is needed

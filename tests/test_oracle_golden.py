@@ -541,3 +541,52 @@ def test_two_operator_reduction_oracle_is_pinned():
     assert oracle.reduce_summax_f32(xs[:2]).tolist() == [-0.5, 1.5]
     e = oracle.reduce_summax_f32(np.zeros(0, np.float32))
     assert e[0] == 0 and np.isneginf(e[1])
+
+
+def test_custom_operators_in_the_segmented_forms():
+    """segreduce_argmax_i32, segreduce_compose_i32, scanrows_argmax_i32 and segred_argmax_i32
+    against brute force in plain Python (ties go to the smaller index; maps are applied one
+    after the other to a probe value) and against the unsegmented functions pinned above."""
+    rng = np.random.default_rng(33)
+    lo, hi = -2 ** 31, 2 ** 31 - 1
+    xss = rng.integers(-5, 5, (23, 17)).astype(np.int32)   # many ties
+    got = oracle.segreduce_argmax_i32(xss)
+    for r in range(23):
+        best = max(range(17), key=lambda j: (int(xss[r, j]), -j))
+        assert got[r].tolist() == [int(xss[r, best]), best]
+        assert got[r].tolist() == oracle.reduce_argmax_i32(xss[r]).tolist()
+    assert oracle.segreduce_argmax_i32(np.zeros((3, 0), np.int32)).tolist() == [[lo, hi]] * 3
+    assert oracle.segreduce_argmax_i32(np.zeros((0, 4), np.int32)).shape == (0, 2)
+
+    k = 9
+    abs_ = rng.integers(-9, 9, (7 * k, 2)).astype(np.int32)
+    got = oracle.segreduce_compose_i32(k, abs_)
+    assert got.shape == (7, 2)
+    for r in range(7):
+        x = 4321
+        for fa, fb in abs_[r * k:(r + 1) * k].tolist():
+            x = (fa * x + fb) % (1 << 32)
+        a, b = (int(v) for v in got[r])
+        assert (a * 4321 + b) % (1 << 32) == x
+        assert got[r].tolist() == oracle.reduce_compose_i32(abs_[r * k:(r + 1) * k]).tolist()
+
+    vis = np.stack([rng.integers(-4, 4, 6 * k), np.arange(6 * k)], axis=1).astype(np.int32)
+    got = oracle.scanrows_argmax_i32(k, vis)
+    for r in range(6):
+        row = vis[r * k:(r + 1) * k]
+        assert np.array_equal(got[r * k:(r + 1) * k], oracle.scan_argmax_i32(row))
+        best = (lo, hi)
+        for j in range(k):   # the running argmax, by hand
+            v, i = int(row[j, 0]), int(row[j, 1])
+            if v > best[0] or (v == best[0] and i < best[1]):
+                best = (v, i)
+            assert got[r * k + j].tolist() == list(best)
+
+    lens = np.array([4, 0, 1, 20, 0, 3], np.int64)
+    offsets = np.concatenate(([0], np.cumsum(lens)[:-1])).astype(np.int64)
+    vis = np.stack([rng.integers(-4, 4, 40), np.arange(40)], axis=1).astype(np.int32)  # 12 pairs unused
+    got = oracle.segred_argmax_i32(offsets, lens, vis)
+    for s in range(6):
+        seg = vis[offsets[s]:offsets[s] + lens[s]]
+        want = [lo, hi] if lens[s] == 0 else oracle.scan_argmax_i32(seg)[-1].tolist()
+        assert got[s].tolist() == want
