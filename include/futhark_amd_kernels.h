@@ -396,8 +396,8 @@ int fa_iota(fa_stream_t stream, fa_dtype t, void *dst, int64_t n,
  *                             composed in element order
  *   fa_scanrows_argmax_i32:   pairs [m][k][2]i32 -> out of the same shape, scanned per
  *                             row; scratch and epoch as for fa_segscan with n = m * k
- *   fa_segred_argmax_i32:     pairs [n][2]i32, segments (offsets[i], lens[i]) that tile
- *                             a prefix of the pairs in order -> out [m][2]i32;
+ *   fa_segred_argmax_i32:     pairs [n][2]i32, segments (offsets[i], lens[i]) in order
+ *                             and not overlapping -> out [m][2]i32;
  *                             workspace of fa_segred_argmax_workspace_bytes(n) bytes,
  *                             16-byte aligned, contents irrelevant */
 int fa_segreduce_argmax_i32(fa_stream_t stream, const int32_t *xss, int64_t m, int64_t k,

@@ -1130,9 +1130,10 @@ static int launch_segreduce(hipStream_t s, const Tin *xss, int64_t m, int64_t k,
 // expresses them (Pass/Flatten/Builtins.hs:570-602): flags are written from
 // the offsets, the values are scanned with the flag-tuple operator, and
 // segment i takes the scanned value at its last element, or the neutral
-// element when it is empty.  Segments must tile a prefix of the input in order
-// (offsets[i] + lens[i] == offsets[i+1]); elements behind the last segment are
-// ignored.  workspace: n * (sizeof(T) + 1) bytes rounded up to 16, 16-byte
+// element when it is empty.  Segments must be in order and must not overlap
+// (offsets[i] + lens[i] <= offsets[i+1] <= n); elements between two segments
+// and behind the last one belong to nobody (they are scanned on as a tail of
+// the segment before them, which nobody reads).  workspace: n * (sizeof(T) + 1) bytes rounded up to 16, 16-byte
 // aligned; scratch and epoch as for launch_scan.
 // Clears `units` 16-byte units (a kernel rather than a memset, so that callers
 // may record the launches in a graph).
