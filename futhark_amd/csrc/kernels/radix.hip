@@ -23,7 +23,8 @@ template <class K, int VB>
 static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const void *vin, void *vout,
                        void *vtmp, int64_t n, int begin_bit, int end_bit, void *scratch) {
   const int passes = (end_bit - begin_bit) / 8;
-  RsScratch sc = rs_carve(scratch, rs_num_tiles(n));
+  const bool wide = n >= RS_WIDE_N;
+  RsScratch sc = rs_carve(scratch, rs_num_tiles(n), wide);
   DigitBits<K> fn{begin_bit};
   int rc = rs_prepare(st, sc);
   if (rc != 0) return rc;
@@ -35,7 +36,10 @@ static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const voi
     const bool to_out = ((passes - 1 - p) % 2) == 0;
     K *dst_k = to_out ? kout : ktmp;
     void *dst_v = to_out ? vout : vtmp;
-    rc = rs_pass<K, VB>(st, src_k, dst_k, src_v, dst_v, n, fn, p, (uint32_t)(p + 1), sc);
+    rc = wide ? rs_pass<K, VB, DigitBits<K>, uint64_t>(st, src_k, dst_k, src_v, dst_v, n, fn, p,
+                                                       (uint32_t)(p + 1), sc)
+              : rs_pass<K, VB, DigitBits<K>, uint32_t>(st, src_k, dst_k, src_v, dst_v, n, fn, p,
+                                                       (uint32_t)(p + 1), sc);
     if (rc != 0) return rc;
     src_k = dst_k;
     src_v = dst_v;
@@ -47,14 +51,14 @@ static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const voi
 
 extern "C" size_t fa_radix_sort_scratch_bytes(int64_t n) {
   if (n < 0) n = 0;
-  return rs_scratch_bytes(rs_num_tiles(n));
+  return rs_scratch_bytes(rs_num_tiles(n), n >= RS_WIDE_N);
 }
 
 extern "C" int fa_radix_sort(fa_stream_t stream, int key_bytes, int val_bytes, const void *keys_in,
                              void *keys_out, void *keys_tmp, const void *vals_in, void *vals_out,
                              void *vals_tmp, int64_t n, int begin_bit, int end_bit, void *scratch,
                              size_t scratch_bytes) {
-  if (n < 0 || n >= RS_MAX_N) return FA_EINVAL;
+  if (n < 0) return FA_EINVAL;
   if (key_bytes != 4 && key_bytes != 8) return FA_ENOTSUP;
   if (val_bytes != 0 && val_bytes != 4 && val_bytes != 8) return FA_ENOTSUP;
   if (begin_bit < 0 || end_bit > key_bytes * 8 || end_bit < begin_bit ||

@@ -18,36 +18,39 @@ constexpr int RS_WAVES = RS_BLOCK / WAVE;
 constexpr int RS_KPT = 16;  // keys per thread
 constexpr int RS_TILE = RS_BLOCK * RS_KPT;
 constexpr int RS_RADIX = 256;
-// Positions in the output are unsigned 32-bit numbers (offsets, counts, the
-// scatter's destinations); everything that scales with the tile count is 64-bit.
-constexpr int64_t RS_MAX_N = ((int64_t)1 << 32) - 1;
+// Positions in the output (counts, offsets, the scatter's destinations) are of
+// type Off: unsigned 32-bit numbers for fewer than RS_WIDE_N keys, 64-bit ones
+// from there on.  Everything that scales with the tile count is 64-bit.
+constexpr int64_t RS_WIDE_N = ((int64_t)1 << 32) - 1;
 constexpr int RS_DIES = 8;  // a block runs on die blockIdx.x % 8
 
 struct RsScratch {
-  uint32_t *counts;   // [256][tiles]
-  uint32_t *offsets;  // [256][tiles] exclusive scan of counts, digit-major
-  void *lookback;     // scratch of the scan kernel, cleared once per call
+  void *counts;    // [256][tiles] of Off
+  void *offsets;   // [256][tiles] exclusive scan of counts, digit-major
+  void *lookback;  // scratch of the scan kernel, cleared once per call
   size_t lookback_bytes;
   int64_t tiles;
+  bool wide;  // Off is 64-bit
 };
 
 static inline int64_t rs_num_tiles(int64_t n) { return ceil_div(n, (int64_t)RS_TILE); }
 static inline size_t rs_align(size_t x) { return (x + 255) & ~(size_t)255; }
 
-static inline size_t rs_scratch_bytes(int64_t tiles) {
+static inline size_t rs_scratch_bytes(int64_t tiles, bool wide) {
   if (tiles < 1) tiles = 1;
-  return 2 * rs_align((size_t)tiles * RS_RADIX * 4) +
-         rs_align(fa_segscan_scratch_bytes(FA_U32, tiles * RS_RADIX));
+  return 2 * rs_align((size_t)tiles * RS_RADIX * (wide ? 8 : 4)) +
+         rs_align(fa_segscan_scratch_bytes(wide ? FA_U64 : FA_U32, tiles * RS_RADIX));
 }
 
-static inline RsScratch rs_carve(void *scratch, int64_t tiles) {
+static inline RsScratch rs_carve(void *scratch, int64_t tiles, bool wide) {
   RsScratch sc;
-  const size_t counts = rs_align((size_t)tiles * RS_RADIX * 4);
-  sc.counts = (uint32_t *)scratch;
-  sc.offsets = (uint32_t *)((char *)scratch + counts);
+  const size_t counts = rs_align((size_t)tiles * RS_RADIX * (wide ? 8 : 4));
+  sc.counts = scratch;
+  sc.offsets = (char *)scratch + counts;
   sc.lookback = (char *)scratch + 2 * counts;
-  sc.lookback_bytes = rs_align(fa_segscan_scratch_bytes(FA_U32, tiles * RS_RADIX));
+  sc.lookback_bytes = rs_align(fa_segscan_scratch_bytes(wide ? FA_U64 : FA_U32, tiles * RS_RADIX));
   sc.tiles = tiles;
+  sc.wide = wide;
   return sc;
 }
 
@@ -90,15 +93,27 @@ __device__ __forceinline__ void rs_count(uint32_t *h, uint32_t d, uint32_t one) 
     atomicAdd(&h[d0], one * (uint32_t)__builtin_popcountll(same));
 }
 
-template <class K, class DigitFn>
+template <class K, class DigitFn, class Off>
 __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__ keys, int64_t n,
-                                                           DigitFn fn, int pass, uint32_t *counts,
+                                                           DigitFn fn, int pass, Off *counts,
                                                            int64_t num_tiles) {
   constexpr int VEC = 16 / sizeof(K);
   constexpr int ROWS = RS_KPT / VEC;
   __shared__ __align__(16) uint32_t h[RS_HIST_TILES][RS_RADIX];
   for (int i = threadIdx.x; i < RS_HIST_TILES * RS_RADIX; i += RS_BLOCK) (&h[0][0])[i] = 0u;
-  const int64_t tile0 = (int64_t)blockIdx.x * RS_HIST_TILES;
+  // The scatter kernel that follows takes the tiles die by die (block b: tile
+  // (b % 8) * tiles_per_die + b / 8).  Counting the keys in the reverse of that
+  // order leaves in the memory-side cache what the scatter reads first; the
+  // non-temporal loads bypass L2 only.  Sort of 2^26 4-byte keys: 770 -> 747 us;
+  // with 8-byte keys, where a pass reads twice the cache's size, the order
+  // costs 1 % instead (3521 -> 3552 us), so those keep the plain order.
+  // (gridDim.x is a multiple of RS_DIES.)
+  int64_t group = blockIdx.x;
+  if constexpr (sizeof(K) == 4) {
+    const int64_t rb = (int64_t)gridDim.x - 1 - blockIdx.x;
+    group = (rb % RS_DIES) * (gridDim.x / RS_DIES) + rb / RS_DIES;
+  }
+  const int64_t tile0 = group * RS_HIST_TILES;
   // The tiles of a block are taken in an order rotated by the block's number:
   // blocks run in step, and with every block at the same place of its own run
   // of tiles the reads of one moment would lie 8 tiles apart from each other
@@ -145,10 +160,10 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_hist_kernel(const K *__restrict__
     uint32_t mine[RS_HIST_TILES];
 #pragma unroll
     for (int i = 0; i < RS_HIST_TILES; i++) mine[(i + rot) % RS_HIST_TILES] = h[i][threadIdx.x];
-    uint32_t *dst = counts + (int64_t)threadIdx.x * num_tiles + tile0;
+    Off *dst = counts + (int64_t)threadIdx.x * num_tiles + tile0;
     const int tiles_here =
         (int)(num_tiles - tile0 < RS_HIST_TILES ? num_tiles - tile0 : RS_HIST_TILES);
-    if (tiles_here == RS_HIST_TILES && (num_tiles & 3) == 0) {
+    if (sizeof(Off) == 4 && tiles_here == RS_HIST_TILES && (num_tiles & 3) == 0) {
       static_assert(RS_HIST_TILES == 8, "two 16-byte stores per digit");
       reinterpret_cast<uint4 *>(dst)[0] = make_uint4(mine[0], mine[1], mine[2], mine[3]);
       reinterpret_cast<uint4 *>(dst)[1] = make_uint4(mine[4], mine[5], mine[6], mine[7]);
@@ -269,18 +284,20 @@ constexpr size_t RS_LDS_FIXED = RS_WAVES * RS_RADIX * 4 + 2 * RS_RADIX * 4 + 64;
 // run of a digit in tile t ends in the cache line where the run of the same
 // digit in tile t + 1 begins, and the two halves of that line meet in one L2
 // only if both tiles are scattered on the same die.
-template <class K, int VB, bool FULL, class DigitFn>
+template <class K, int VB, bool FULL, class DigitFn, class Off>
 __device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__restrict__ kout,
                                                 const typename ValType<VB>::T *__restrict__ vin,
                                                 typename ValType<VB>::T *__restrict__ vout,
                                                 int64_t n, DigitFn fn, int pass,
-                                                const uint32_t *__restrict__ offs,
+                                                const Off *__restrict__ offs,
                                                 int64_t num_tiles, int64_t tile,
                                                 unsigned char *s_raw) {
   using V = typename ValType<VB>::T;
   uint32_t(*cnt)[RS_RADIX] = reinterpret_cast<uint32_t(*)[RS_RADIX]>(s_raw);
-  uint32_t *s_tab = reinterpret_cast<uint32_t *>(s_raw + RS_WAVES * RS_RADIX * 4);
-  uint32_t *s_wsum = s_tab + 2 * RS_RADIX;  // 4 used
+  static_assert(sizeof(Off) <= 8, "the table of a tile is 2 * RS_RADIX words");
+  Off *s_tab = reinterpret_cast<Off *>(s_raw + RS_WAVES * RS_RADIX * 4);
+  uint32_t *s_wsum =
+      reinterpret_cast<uint32_t *>(s_raw + RS_WAVES * RS_RADIX * 4 + 2 * RS_RADIX * 4);  // 4 used
   unsigned char *buf = s_raw + RS_LDS_FIXED;
 
   const int tid = threadIdx.x;
@@ -309,7 +326,7 @@ __device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__
   }
   for (int i = tid; i < RS_WAVES * RS_RADIX; i += RS_BLOCK) (&cnt[0][0])[i] = 0u;
   // Global offsets of this tile, one digit per thread (strided, L2-resident).
-  uint32_t goff = 0;
+  Off goff = 0;
   if (tid < RS_RADIX) goff = offs[(int64_t)tid * num_tiles + tile];
   __syncthreads();
   // The kernel is bound by vector-ALU issue; rs_match2 finds the lanes with
@@ -382,16 +399,16 @@ __device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__
   __syncthreads();
   // The offsets come from this library's own histogram and scan; should they
   // ever be wrong, a store outside the output would fault the GPU, whereas a
-  // dropped key is a wrong result the caller can see.  n < 2^32 - 1.
-  uint32_t dst[RS_KPT];
-  const uint32_t limit = (uint32_t)n;
+  // dropped key is a wrong result the caller can see.
+  Off dst[RS_KPT];
+  const Off limit = (Off)n;
 #pragma unroll
   for (int j = 0; j < RS_KPT; j++) {
     const int i = j * RS_BLOCK + tid;
     dst[j] = limit;
     if (FULL || i < tile_n) {
       const K k = kbuf[i];
-      dst[j] = s_tab[fn(k, pass)] + (uint32_t)i;
+      dst[j] = s_tab[fn(k, pass)] + (Off)i;
       if (dst[j] < limit) kout[dst[j]] = k;
     }
   }
@@ -410,10 +427,10 @@ __device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__
   }
 }
 
-template <class K, int VB, class DigitFn>
+template <class K, int VB, class DigitFn, class Off>
 __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
     const K *__restrict__ kin, K *__restrict__ kout, const void *__restrict__ vin_,
-    void *__restrict__ vout_, int64_t n, DigitFn fn, int pass, const uint32_t *__restrict__ offs,
+    void *__restrict__ vout_, int64_t n, DigitFn fn, int pass, const Off *__restrict__ offs,
     int64_t num_tiles) {
   using V = typename ValType<VB>::T;
   extern __shared__ __align__(16) unsigned char s_raw[];
@@ -422,10 +439,10 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
   const int64_t tile = (int64_t)(blockIdx.x % RS_DIES) * tiles_per_die + blockIdx.x / RS_DIES;
   if (tile >= num_tiles) return;  // uniform over the block
   if ((tile + 1) * RS_TILE <= n)
-    rs_scatter_tile<K, VB, true>(kin, kout, (const V *)vin_, (V *)vout_, n, fn, pass, offs,
+    rs_scatter_tile<K, VB, true, DigitFn, Off>(kin, kout, (const V *)vin_, (V *)vout_, n, fn, pass, offs,
                                  num_tiles, tile, s_raw);
   else
-    rs_scatter_tile<K, VB, false>(kin, kout, (const V *)vin_, (V *)vout_, n, fn, pass, offs,
+    rs_scatter_tile<K, VB, false, DigitFn, Off>(kin, kout, (const V *)vin_, (V *)vout_, n, fn, pass, offs,
                                   num_tiles, tile, s_raw);
 }
 
@@ -433,30 +450,31 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
 // equal digits keeping their order.  `epoch` must grow from call to call on
 // the same scratch (1, 2, ...).  Afterwards sc.offsets[d * tiles] is the
 // position where digit d starts in the output.
-template <class K, int VB, class DigitFn>
+template <class K, int VB, class DigitFn, class Off = uint32_t>
 static int rs_pass(hipStream_t st, const K *kin, K *kout, const void *vin, void *vout, int64_t n,
                    DigitFn fn, int pass, uint32_t epoch, const RsScratch &sc) {
   using V = typename ValType<VB>::T;
-  if (n >= RS_MAX_N) return FA_EINVAL;  // positions are unsigned 32-bit
+  constexpr bool WIDE = sizeof(Off) == 8;
+  if (sc.wide != WIDE || (!WIDE && n >= RS_WIDE_N)) return FA_EINVAL;
   const size_t lds =
       RS_LDS_FIXED + (size_t)RS_TILE * (sizeof(K) > sizeof(V) ? sizeof(K) : sizeof(V));
-  auto scatter = rs_scatter_kernel<K, VB, DigitFn>;
+  auto scatter = rs_scatter_kernel<K, VB, DigitFn, Off>;
   // Initialised once, under the lock C++ gives function-local statics.
   static const hipError_t raised = hipFuncSetAttribute(
       (const void *)scatter, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
   if (raised != hipSuccess) return (int)raised;
-  hipLaunchKernelGGL((rs_hist_kernel<K, DigitFn>),
+  hipLaunchKernelGGL((rs_hist_kernel<K, DigitFn, Off>),
                      dim3((unsigned)(ceil_div(sc.tiles, (int64_t)RS_HIST_TILES * RS_DIES) * RS_DIES)),
                      dim3(RS_BLOCK), 0, st,
-                     kin, n, fn, pass, sc.counts, sc.tiles);
+                     kin, n, fn, pass, (Off *)sc.counts, sc.tiles);
   int rc = launch_status();
   if (rc != 0) return rc;
-  rc = fa_segscan((fa_stream_t)st, FA_U32, FA_ADD, sc.counts, nullptr, sc.tiles * RS_RADIX, 1,
+  rc = fa_segscan((fa_stream_t)st, WIDE ? FA_U64 : FA_U32, FA_ADD, sc.counts, nullptr, sc.tiles * RS_RADIX, 1,
                   sc.offsets, sc.lookback, sc.lookback_bytes, epoch);
   if (rc != 0) return rc;
   const int64_t tiles_per_die = ceil_div(sc.tiles, (int64_t)RS_DIES);
   hipLaunchKernelGGL(scatter, dim3((unsigned)(tiles_per_die * RS_DIES)), dim3(RS_BLOCK), lds, st,
-                     kin, kout, vin, vout, n, fn, pass, sc.offsets, sc.tiles);
+                     kin, kout, vin, vout, n, fn, pass, (const Off *)sc.offsets, sc.tiles);
   return launch_status();
 }
 

@@ -289,8 +289,8 @@ int fa_seghist_shaped(fa_stream_t stream, fa_dtype t, fa_op op,
  * key_bytes is 4 or 8; keys compare as unsigned.  val_bytes is 0, 4 or 8.
  * keys_in/vals_in are not modified; the result lands in keys_out/vals_out.
  * keys_tmp/vals_tmp are n-element ping-pong buffers.  begin_bit/end_bit select
- * the key bits that take part (multiple of 8 apart).  n < 2^32 - 1 (positions
- * are unsigned 32-bit numbers); FA_EINVAL beyond. */
+ * the key bits that take part (multiple of 8 apart).  Positions are unsigned
+ * 32-bit numbers below 2^32 - 1 keys and 64-bit ones from there on. */
 size_t fa_radix_sort_scratch_bytes(int64_t n);
 int fa_radix_sort(fa_stream_t stream, int key_bytes, int val_bytes,
                   const void *keys_in, void *keys_out, void *keys_tmp,

@@ -343,7 +343,7 @@ int futhark_entry_segscan_compose_i32(struct futhark_context *ctx, struct futhar
  *     scan argmax (i32.lowest, i32.highest) (map (\r -> (r[0], r[1])) vis) |> map (\(v, i) -> [v, i])
  *   entry hist_argmax_i32 (k: i64) (is: []i32) (xs: []i32) : [k][2]i32 =
  *     hist argmax (i32.lowest, i32.highest) k (map i64.i32 is) (zip xs (map i32.i64 (indices xs)))
- *     |> map (\(v, i) -> [v, i])                           -- k at most 8192
+ *     |> map (\(v, i) -> [v, i])
  *   entry reduce_compose_i32 (abs: [][2]i32) : [2]i32 =    -- compose as above; does not commute
  *     let (a, b) = reduce compose (1, 0) (map (\r -> (r[0], r[1])) abs) in [a, b]
  *   entry sumsq_f32 (xs: []f32) : f32 = reduce (+) 0 (map (\x -> x * x) xs)

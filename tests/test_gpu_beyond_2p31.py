@@ -88,3 +88,67 @@ def test_transpose_with_more_blocks_than_one_launch_holds(ctx):
         hi = min(lo + period, cols)
         for r in range(2):
             assert np.array_equal(got[lo:hi, r], row(r, lo, hi)), (r, lo)
+
+
+ODD = 2654435761
+
+
+def _scrambled(lo, hi):
+    """(i * ODD) mod 2^32 for i in [lo, hi): a permutation of the 32-bit numbers over any 2^32
+    consecutive i."""
+    return ((np.arange(lo, hi, dtype=np.uint64) * np.uint64(ODD)) & np.uint64(0xFFFFFFFF)).astype(np.uint32)
+
+
+def test_sort_of_more_than_2p32_keys(ctx):
+    """From 2^32 - 1 keys on, positions in the output no longer fit 32 bits and the sort counts
+    and scatters with 64-bit ones.  keys[i] = (i * odd) mod 2^32 for i < 2^32 + 4099: every
+    32-bit number once, the first 4099 of the sequence twice, so the sorted output is known
+    position by position: 0, 1, 2, ... with those 4099 values doubled."""
+    extra = 4099
+    n = (1 << 32) + extra
+    step = 1 << 27
+    keys = np.empty(n, np.uint32)
+    for lo in range(0, n, step):
+        hi = min(lo + step, n)
+        keys[lo:hi] = _scrambled(lo, hi)
+    a = ctx.new("u32_1d", keys)
+    del keys
+    print("radix_sort_u32 n=2^32+4099", flush=True)
+    out = ctx.call("radix_sort_u32", ["u32_1d"], a)
+    a.free()
+    got = out.values()
+    out.free()
+    ctx.clear_caches()
+    assert got.shape == (n,)
+    doubled = np.sort(_scrambled(0, extra)).astype(np.int64)
+    second = doubled + np.arange(1, extra + 1)  # where the second copy of each doubled value sits
+    for lo in range(0, n, step):
+        hi = min(lo + step, n)
+        pos = np.arange(lo, hi, dtype=np.int64)
+        want = pos - np.searchsorted(second, pos, side="right")
+        assert np.array_equal(got[lo:hi], want.astype(np.uint32)), lo
+
+
+def test_histogram_with_many_bins_over_more_than_2p31_updates(ctx):
+    """reduce_by_index into 2^22 bins partitions its updates by bin range, in slices whose
+    histograms add up; 2^31 + 12345 updates are nine slices, the last a ragged one.
+    is[i] = top 22 bits of (i * odd) mod 2^32, vs[i] = (i mod 7) - 3, dest starts non-zero."""
+    H = 1 << 22
+    dest = (np.arange(H) % 5).astype(np.int32)
+    vs = _pattern(N)
+    is_ = np.empty(N, np.int32)
+    want = dest.astype(np.int64)
+    step = 1 << 27
+    for lo in range(0, N, step):
+        hi = min(lo + step, N)
+        is_[lo:hi] = (_scrambled(lo, hi) >> np.uint32(10)).astype(np.int32)
+        want += np.bincount(is_[lo:hi], weights=vs[lo:hi], minlength=H).astype(np.int64)
+    d, i, v = ctx.new("i32_1d", dest), ctx.new("i32_1d", is_), ctx.new("i32_1d", vs)
+    del is_, vs
+    print("rbi_add_i32 H=2^22 n=2^31+12345", flush=True)
+    out = ctx.call("rbi_add_i32", ["i32_1d"], d, i, v)
+    got = out.values()
+    for h in (d, i, v, out):
+        h.free()
+    ctx.clear_caches()
+    assert np.array_equal(got.astype(np.int64), want)
