@@ -370,11 +370,117 @@ __global__ __launch_bounds__(IB_BLOCK) void rows_fraction_wave_kernel(const floa
   }
 }
 
+// Inclusive scan inside every group of LPR consecutive lanes (a power of two):
+// the steps of the wave scan that stay inside a group.  Up to 16 lanes the row
+// shifts must not cross into the group before; 32 and 64 lanes are whole rows
+// of 16 joined by one or both broadcasts.
+template <class T, class Op, int LPR>
+__device__ __forceinline__ T lane_group_incl_scan(T x, int lane) {
+  static_assert(LPR >= 1 && LPR <= WAVE && (LPR & (LPR - 1)) == 0, "a power of two");
+  const T id = Op::identity();
+  if constexpr (LPR >= 32) {
+    x = Op::apply(dpp_move<DPP_ROW_SHR1, 0xf>(id, x), x);
+    x = Op::apply(dpp_move<DPP_ROW_SHR2, 0xf>(id, x), x);
+    x = Op::apply(dpp_move<DPP_ROW_SHR4, 0xf>(id, x), x);
+    x = Op::apply(dpp_move<DPP_ROW_SHR8, 0xf>(id, x), x);
+    x = Op::apply(dpp_move<DPP_ROW_BCAST15, 0xa>(id, x), x);
+    if constexpr (LPR == 64) x = Op::apply(dpp_move<DPP_ROW_BCAST31, 0xc>(id, x), x);
+  } else {
+    const int j = lane & (LPR - 1);
+    if constexpr (LPR > 1) {
+      const T t = dpp_move<DPP_ROW_SHR1, 0xf>(id, x);
+      x = j >= 1 ? Op::apply(t, x) : x;
+    }
+    if constexpr (LPR > 2) {
+      const T t = dpp_move<DPP_ROW_SHR2, 0xf>(id, x);
+      x = j >= 2 ? Op::apply(t, x) : x;
+    }
+    if constexpr (LPR > 4) {
+      const T t = dpp_move<DPP_ROW_SHR4, 0xf>(id, x);
+      x = j >= 4 ? Op::apply(t, x) : x;
+    }
+    if constexpr (LPR > 8) {
+      const T t = dpp_move<DPP_ROW_SHR8, 0xf>(id, x);
+      x = j >= 8 ? Op::apply(t, x) : x;
+    }
+  }
+  return x;
+}
+
+// Rows of 4 LPR elements, LPR = 1, 2, ... 64 lanes per row: a wave-wide 16-byte
+// load is 64 / LPR whole rows, each scanned by its group of lanes; the row's
+// sum is the last lane's scan value, so the row is read once, and a wave has
+// IB_PACKED_LOADS loads in flight.  ([2^20][64] f32 with a wave per row, the
+// row read twice: 258 us.)
+constexpr int IB_PACKED_LOADS = 4;
+template <int LPR>
+__global__ __launch_bounds__(IB_BLOCK) void rows_fraction_packed_kernel(const float *__restrict__ xss,
+                                                                        int64_t m,
+                                                                        float *__restrict__ out) {
+  constexpr int G = WAVE / LPR;  // rows per load
+  constexpr int U = IB_PACKED_LOADS;
+  const int lane = lane_id();
+  const int64_t n = m * (LPR * IB_VEC);
+  const int64_t loads = ceil_div(m, (int64_t)G);
+  const int64_t waves = (int64_t)gridDim.x * (IB_BLOCK / WAVE);
+  for (int64_t l0 = ((int64_t)blockIdx.x * (IB_BLOCK / WAVE) + threadIdx.x / WAVE) * U; l0 < loads;
+       l0 += waves * U) {
+    Vec16<float> v[U];
+    int64_t at[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      // rows are whole groups of lanes, so a group lies inside the array or
+      // beyond it; lanes beyond load the first element and store nothing
+      at[u] = ((l0 + u) * WAVE + lane) * IB_VEC;
+      v[u] = load_vec16_nt(xss + (at[u] < n ? at[u] : 0));
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      float x[IB_VEC];
+#pragma unroll
+      for (int e = 0; e < IB_VEC; e++) x[e] = v[u].e[e];
+#pragma unroll
+      for (int e = 1; e < IB_VEC; e++) x[e] += x[e - 1];
+      const float incl = lane_group_incl_scan<float, OpAdd<float>, LPR>(x[IB_VEC - 1], lane);
+      float excl = wave_shift_up1<float, OpAdd<float>>(incl);
+      if ((lane & (LPR - 1)) == 0) excl = 0.0f;
+      const float total = __shfl(incl, lane | (LPR - 1), WAVE);
+      Vec16<float> o;
+#pragma unroll
+      for (int e = 0; e < IB_VEC; e++) o.e[e] = (excl + x[e]) / total;
+      if (at[u] < n) store_vec16_nt(out + at[u], o);
+    }
+  }
+}
+
+template <int LPR>
+static int launch_rows_fraction_packed(hipStream_t st, const float *xss, int64_t m, float *out) {
+  const int64_t loads = ceil_div(m, (int64_t)(WAVE / LPR));
+  const int64_t blocks = ceil_div(loads, (int64_t)(IB_BLOCK / WAVE) * IB_PACKED_LOADS);
+  const int64_t grid = blocks < 256 * 8 ? blocks : 256 * 8;
+  hipLaunchKernelGGL(rows_fraction_packed_kernel<LPR>, dim3((unsigned)grid), dim3(IB_BLOCK), 0, st,
+                     xss, m, out);
+  return launch_status();
+}
+
 extern "C" int fa_rows_fraction_f32(fa_stream_t stream, const float *xss, int64_t m, int64_t k,
                                     float *out) {
   if (m < 0 || k < 0) return FA_EINVAL;
   if (m == 0 || k == 0) return 0;
   if (xss == nullptr || out == nullptr) return FA_EINVAL;
+  if (k % IB_VEC == 0 && k <= WAVE * IB_VEC && (k & (k - 1)) == 0 &&
+      ((uintptr_t)xss | (uintptr_t)out) % 16 == 0) {
+    hipStream_t st = (hipStream_t)stream;
+    switch ((int)(k / IB_VEC)) {
+      case 1: return launch_rows_fraction_packed<1>(st, xss, m, out);
+      case 2: return launch_rows_fraction_packed<2>(st, xss, m, out);
+      case 4: return launch_rows_fraction_packed<4>(st, xss, m, out);
+      case 8: return launch_rows_fraction_packed<8>(st, xss, m, out);
+      case 16: return launch_rows_fraction_packed<16>(st, xss, m, out);
+      case 32: return launch_rows_fraction_packed<32>(st, xss, m, out);
+      default: return launch_rows_fraction_packed<64>(st, xss, m, out);
+    }
+  }
   if (k <= IB_WAVE_ROW_MAX) {
     const int64_t blocks = ceil_div(m, (int64_t)(IB_BLOCK / WAVE));
     const int64_t grid = blocks < 256 * 8 ? blocks : 256 * 8;

@@ -90,7 +90,9 @@ def test_segops_inside_a_block(ctx):
     scan, more rows than blocks, empty in either dimension; a row that sums to zero divides
     as IEEE says.  Tolerance 1e-5 relative (positive data, f32 sums in another order)."""
     for m, k in [(1, 1), (5, 3), (7, 64), (9, 255), (6, 256), (5, 257), (3, 1023), (4, 1024), (3, 1025), (2, 40001), (5000, 17),
-                 (0, 4), (4, 0)]:
+                 (0, 4), (4, 0),
+                 # rows of 4, 8, ... 256 elements share a wave-wide load: whole and ragged last loads
+                 (1, 4), (4097, 4), (1000, 8), (33, 16), (65, 32), (5000, 64), (100, 128), (13, 256), (20000, 256)]:
         xss = (dg.uniform_f32(25, m * k) + np.float32(0.01)).reshape(m, k)
         out = ctx.call("rows_fraction_f32", ["f32_2d"], ctx.new("f32_2d", xss))
         got = out.values()
