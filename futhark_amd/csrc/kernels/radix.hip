@@ -13,7 +13,9 @@ namespace fa {
 
 // Digits of pass p are bits [begin + 8p, begin + 8p + 8) of the key.
 template <class K> struct DigitBits {
+  using Out = K;
   int begin_bit;
+  __device__ __forceinline__ K out(K key) const { return key; }
   __device__ __forceinline__ uint32_t operator()(K key, int pass) const {
     return (uint32_t)(key >> (begin_bit + 8 * pass)) & 0xffu;
   }

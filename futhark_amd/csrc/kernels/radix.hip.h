@@ -285,7 +285,8 @@ constexpr size_t RS_LDS_FIXED = RS_WAVES * RS_RADIX * 4 + 2 * RS_RADIX * 4 + 64;
 // digit in tile t + 1 begins, and the two halves of that line meet in one L2
 // only if both tiles are scattered on the same die.
 template <class K, int VB, bool FULL, class DigitFn, class Off>
-__device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__restrict__ kout,
+__device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin,
+                                                typename DigitFn::Out *__restrict__ kout,
                                                 const typename ValType<VB>::T *__restrict__ vin,
                                                 typename ValType<VB>::T *__restrict__ vout,
                                                 int64_t n, DigitFn fn, int pass,
@@ -409,7 +410,7 @@ __device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__
     if (FULL || i < tile_n) {
       const K k = kbuf[i];
       dst[j] = s_tab[fn(k, pass)] + (Off)i;
-      if (dst[j] < limit) kout[dst[j]] = k;
+      if (dst[j] < limit) kout[dst[j]] = fn.out(k);
     }
   }
   if constexpr (VB != 0) {
@@ -429,8 +430,9 @@ __device__ __forceinline__ void rs_scatter_tile(const K *__restrict__ kin, K *__
 
 template <class K, int VB, class DigitFn, class Off>
 __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
-    const K *__restrict__ kin, K *__restrict__ kout, const void *__restrict__ vin_,
-    void *__restrict__ vout_, int64_t n, DigitFn fn, int pass, const Off *__restrict__ offs,
+    const K *__restrict__ kin, typename DigitFn::Out *__restrict__ kout,
+    const void *__restrict__ vin_, void *__restrict__ vout_, int64_t n, DigitFn fn, int pass,
+    const Off *__restrict__ offs,
     int64_t num_tiles) {
   using V = typename ValType<VB>::T;
   extern __shared__ __align__(16) unsigned char s_raw[];
@@ -447,11 +449,14 @@ __global__ __launch_bounds__(RS_BLOCK) void rs_scatter_kernel(
 }
 
 // One pass: keys (and values) move from *in to *out ordered by digit `pass`,
-// equal digits keeping their order.  `epoch` must grow from call to call on
+// equal digits keeping their order.  What is written for a key is fn.out(key),
+// of type DigitFn::Out: the key itself for the sort, what is left of a bin
+// number inside its range for the partition of a histogram.  `epoch` must grow from call to call on
 // the same scratch (1, 2, ...).  Afterwards sc.offsets[d * tiles] is the
 // position where digit d starts in the output.
 template <class K, int VB, class DigitFn, class Off = uint32_t>
-static int rs_pass(hipStream_t st, const K *kin, K *kout, const void *vin, void *vout, int64_t n,
+static int rs_pass(hipStream_t st, const K *kin, typename DigitFn::Out *kout, const void *vin,
+                   void *vout, int64_t n,
                    DigitFn fn, int pass, uint32_t epoch, const RsScratch &sc) {
   using V = typename ValType<VB>::T;
   constexpr bool WIDE = sizeof(Off) == 8;

@@ -522,21 +522,28 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_lds_kernel(
 }
 
 template <class U> struct DigitBinRange {
+  using Out = uint16_t;  // the bin inside its range: shift <= 15 bits
   uint64_t H;
   int shift;
+  __device__ __forceinline__ uint16_t out(U key) const {
+    return (uint16_t)((uint64_t)key & (((uint64_t)1 << shift) - 1));
+  }
   __device__ __forceinline__ uint32_t operator()(U key, int) const {
     return (uint64_t)key < H ? (uint32_t)((uint64_t)key >> shift) : 255u;
   }
 };
 
 // Input: pairs grouped by bin range; range r starts at offs[r * num_tiles] (the
-// digit-major offsets of the partition pass).  Each block takes a contiguous
-// chunk of the valid pairs and, for every range the chunk touches, accumulates
-// in LDS and flushes.
-template <class T, class Op, class U>
+// digit-major offsets of the partition pass).  Of a pair's bin only the place
+// inside its range is left, 16 bits (the range is known from where the pair
+// lies), so a pair is 2 + sizeof(T) bytes.  Each block takes a contiguous chunk
+// of the valid pairs and, for every range the chunk touches, accumulates in LDS
+// and flushes.
+template <class T, class Op>
 __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
-    const U *__restrict__ pis, const T *__restrict__ pvs, const uint32_t *__restrict__ offs,
+    const uint16_t *__restrict__ pis, const T *__restrict__ pvs, const uint32_t *__restrict__ offs,
     int64_t num_tiles, T *dest, int64_t H, int shift) {
+  using U = uint16_t;
   using A = typename HistAcc<T>::A;
   using OpA = typename RebindOp<Op, A>::type;
   extern __shared__ __align__(16) unsigned char s_raw[];
@@ -560,7 +567,7 @@ __global__ __launch_bounds__(HIST_BLOCK) void seghist_part_kernel(
     __syncthreads();
     // f32 sums: one compare-and-swap attempt before the float atomic (no copies here)
     constexpr int CAS = std::is_same<A, float>::value && std::is_same<OpA, OpAdd<A>>::value ? HIST_CAS_FEW : 0;
-    auto update = [&](U b, T v) { lds_update<A, OpA, CAS>(&sh[(int)((int64_t)b - bin0)], (A)v); };
+    auto update = [&](U b, T v) { lds_update<A, OpA, CAS>(&sh[(int)b], (A)v); };
     // [lo, hi) = loose elements up to a multiple of four, groups of four read
     // with 16-byte non-temporal loads (two groups of a thread in flight),
     // loose elements at the end.
@@ -853,10 +860,10 @@ static int launch_part_hist(hipStream_t st, const U *is, const T *vs, int64_t n,
   constexpr int shift = hist_part_shift<T>();
   const int64_t tiles = rs_num_tiles(n);
   const size_t rs_bytes = hist_align(rs_scratch_bytes(tiles, false));
-  const size_t is_bytes = hist_align((size_t)n * sizeof(U));
+  const size_t is_bytes = hist_align((size_t)n * sizeof(uint16_t));
   if (scratch_bytes < rs_bytes + is_bytes + (size_t)n * sizeof(T)) return FA_ESCRATCH;
   if (!is_aligned(scratch, 256)) return FA_EALIGN;
-  U *pis = (U *)((char *)scratch + rs_bytes);
+  uint16_t *pis = (uint16_t *)((char *)scratch + rs_bytes);
   T *pvs = (T *)((char *)scratch + rs_bytes + is_bytes);
   RsScratch sc = rs_carve(scratch, tiles, false);
   DigitBinRange<U> fn{(uint64_t)H, shift};
@@ -864,7 +871,7 @@ static int launch_part_hist(hipStream_t st, const U *is, const T *vs, int64_t n,
   if (rc != 0) return rc;
   rc = rs_pass<U, (int)sizeof(T)>(st, is, pis, vs, pvs, n, fn, 0, 1u, sc);
   if (rc != 0) return rc;
-  auto kernel = seghist_part_kernel<T, Op, U>;
+  auto kernel = seghist_part_kernel<T, Op>;
   // Initialised once, under the lock C++ gives function-local statics.
   static const hipError_t raised = hipFuncSetAttribute(
       (const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, HIST_LDS_BYTES);
@@ -1046,8 +1053,9 @@ extern "C" size_t fa_seghist_scratch_bytes(fa_dtype t, int is64, int64_t n, int6
   const int64_t part_limit = (int64_t)255 << (as == 4 ? 15 : 14);
   if (H <= lds_limit || H > part_limit) return 256;
   if (n > HIST_PART_SLICE) n = HIST_PART_SLICE;
-  return hist_align(rs_scratch_bytes(rs_num_tiles(n), false)) +
-         hist_align((size_t)n * (is64 ? 8 : 4)) + (size_t)n * es + 256;
+  (void)is64;  // the partitioned indices are 16 bits whatever the width of the input's
+  return hist_align(rs_scratch_bytes(rs_num_tiles(n), false)) + hist_align((size_t)n * 2) +
+         (size_t)n * es + 256;
 }
 
 extern "C" int fa_seghist(fa_stream_t stream, fa_dtype t, fa_op op, const void *is, int is64,
