@@ -117,11 +117,11 @@ extern "C" const char *fa_strerror(int code) {
 // One set per calling thread: the launchers read it on the thread that calls
 // them, so callers that hold different values (contexts with different tuning
 // parameters) can run side by side without touching each other's.
-static thread_local fa_tuning g_tuning = {0, 0, 0, 0};
+static thread_local fa_tuning g_tuning = {0, 0, 0, 0, 0};
 
 extern "C" void fa_set_tuning(const fa_tuning *t) {
   if (t == nullptr) {
-    g_tuning = fa_tuning{0, 0, 0, 0};
+    g_tuning = fa_tuning{0, 0, 0, 0, 0};
     return;
   }
   g_tuning = *t;
@@ -139,4 +139,5 @@ extern "C" void fa_get_tuning(fa_tuning *out) {
   out->hist_lds_bins_max = bins;
   out->matmul_pad_min_work = g_tuning.matmul_pad_min_work > 0 ? g_tuning.matmul_pad_min_work : (int64_t)1 << 24;
   out->scan_tickets_by_block = g_tuning.scan_tickets_by_block != 0;
+  out->sort_wide_positions = g_tuning.sort_wide_positions != 0;
 }

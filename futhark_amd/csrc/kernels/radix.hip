@@ -21,11 +21,18 @@ template <class K> struct DigitBits {
   }
 };
 
+// 64-bit positions: needed from RS_WIDE_N keys on, or asked for.
+static bool sort_wide(int64_t n) {
+  fa_tuning t;
+  fa_get_tuning(&t);
+  return n >= RS_WIDE_N || t.sort_wide_positions != 0;
+}
+
 template <class K, int VB>
 static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const void *vin, void *vout,
                        void *vtmp, int64_t n, int begin_bit, int end_bit, void *scratch) {
   const int passes = (end_bit - begin_bit) / 8;
-  const bool wide = n >= RS_WIDE_N;
+  const bool wide = sort_wide(n);
   RsScratch sc = rs_carve(scratch, rs_num_tiles(n), wide);
   DigitBits<K> fn{begin_bit};
   int rc = rs_prepare(st, sc);
@@ -53,7 +60,7 @@ static int sort_passes(hipStream_t st, const K *kin, K *kout, K *ktmp, const voi
 
 extern "C" size_t fa_radix_sort_scratch_bytes(int64_t n) {
   if (n < 0) n = 0;
-  return rs_scratch_bytes(rs_num_tiles(n), n >= RS_WIDE_N);
+  return rs_scratch_bytes(rs_num_tiles(n), sort_wide(n));
 }
 
 extern "C" int fa_radix_sort(fa_stream_t stream, int key_bytes, int val_bytes, const void *keys_in,

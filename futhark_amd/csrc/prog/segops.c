@@ -22,9 +22,11 @@ static const char *const tuning_names[] = {
     "segops.segred_small_threshold",
     "segops.matmul_pad_min_work",
     "segops.scan_arrival_tickets",
+    "segops.sort_wide_positions",
 };
-static const char *const tuning_classes[] = {"shared_memory", "threshold", "threshold", "threshold"};
-static const int64_t tuning_defaults[] = {0, 0, 0, 0}; /* 0: the kernel library's default */
+static const char *const tuning_classes[] = {"shared_memory", "threshold", "threshold", "threshold",
+                                             "threshold"};
+static const int64_t tuning_defaults[] = {0, 0, 0, 0, 0}; /* 0: the kernel library's default */
 
 /* The parameters choose code paths inside the kernel library (fa_tuning).
  *
@@ -35,7 +37,10 @@ static const int64_t tuning_defaults[] = {0, 0, 0, 0}; /* 0: the kernel library'
  * single stream then has the device to itself, as far as this process can
  * tell), by order of arrival otherwise.  1 always takes the order of arrival:
  * for a process that shares the GPU with other processes' long-running
- * kernels, or runs under a CU mask it applies by other means. */
+ * kernels, or runs under a CU mask it applies by other means.
+ *
+ * segops.sort_wide_positions: 1 makes the radix sort use the 64-bit positions
+ * it otherwise switches to at 2^32 - 1 keys (fa_tuning.sort_wide_positions). */
 static void apply_tuning(struct futhark_context *ctx) {
   fa_tuning t;
   t.hist_lds_bins_max = rts_tuning_param(ctx, tuning_names[0], 0);
@@ -43,11 +48,12 @@ static void apply_tuning(struct futhark_context *ctx) {
   t.matmul_pad_min_work = rts_tuning_param(ctx, tuning_names[2], 0);
   t.scan_tickets_by_block =
       rts_tuning_param(ctx, tuning_names[3], 0) == 0 && rts_device_is_ours(ctx) ? 1 : 0;
+  t.sort_wide_positions = rts_tuning_param(ctx, tuning_names[4], 0) != 0;
   fa_set_tuning(&t);
 }
 
 const struct rts_program futhark_program = {
-    "segops", 4, tuning_names, tuning_classes, tuning_defaults, apply_tuning,
+    "segops", 5, tuning_names, tuning_classes, tuning_defaults, apply_tuning,
 };
 
 /* ------------------------------------------------------------------ arrays */

@@ -331,6 +331,7 @@ static int e_replicate_i32(struct futhark_context *c, struct value *o, struct va
 #define SEGRED_PARAM "segops.segred_small_threshold"
 #define MATMUL_PARAM "segops.matmul_pad_min_work"
 #define SCAN_PARAM "segops.scan_arrival_tickets"
+#define SORT_PARAM "segops.sort_wide_positions"
 #define SEGOP_ENTRY_ROWS(OP, T, CT)                                                             \
   {"reduce_" #OP "_" #T, e_reduce_##OP##_##T, #T, 0, 1, {"[]" #T}, {0}, {NULL}},                \
   {"scan_" #OP "_" #T, e_scan_##OP##_##T, "[]" #T, 1, 1, {"[]" #T}, {0}, {SCAN_PARAM, NULL}},   \
@@ -393,12 +394,12 @@ static const struct entry entries[] = {
      {NULL}},
     {"bmm_bf16", e_bmm_bf16, "[][][]f32", 1, 2, {"[][][]u16", "[][][]u16"}, {0}, {MATMUL_PARAM, NULL}},
     {"matmul_f32", e_matmul_f32, "[][]f32", 1, 2, {"[][]f32", "[][]f32"}, {0}, {MATMUL_PARAM, NULL}},
-    {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {NULL}},
-    {"radix_sort_u64", e_radix_sort_u64, "[]u64", 1, 1, {"[]u64"}, {0}, {NULL}},
+    {"radix_sort_u32", e_radix_sort_u32, "[]u32", 1, 1, {"[]u32"}, {0}, {SORT_PARAM, NULL}},
+    {"radix_sort_u64", e_radix_sort_u64, "[]u64", 1, 1, {"[]u64"}, {0}, {SORT_PARAM, NULL}},
     {"radix_sort_pairs_u32_i32", e_radix_sort_pairs_u32_i32, "([]u32, []i32)", 1, 2,
-     {"[]u32", "[]i32"}, {0}, {NULL}},
+     {"[]u32", "[]i32"}, {0}, {SORT_PARAM, NULL}},
     {"radix_sort_pairs_u64_i32", e_radix_sort_pairs_u64_i32, "([]u64, []i32)", 1, 2,
-     {"[]u64", "[]i32"}, {0}, {NULL}},
+     {"[]u64", "[]i32"}, {0}, {SORT_PARAM, NULL}},
     {"transpose_f32", e_transpose_f32, "[][]f32", 1, 1, {"[][]f32"}, {0}, {NULL}},
     {"iota_i64", e_iota_i64, "[]i64", 1, 1, {"i64"}, {0}, {NULL}},
     {"replicate_i32", e_replicate_i32, "[]i32", 1, 2, {"i64", "i32"}, {0}, {NULL}},

@@ -22,6 +22,7 @@ HIST_PARAM = "segops.hist_lds_bins_max"
 SEGRED_PARAM = "segops.segred_small_threshold"
 MATMUL_PARAM = "segops.matmul_pad_min_work"
 SCAN_PARAM = "segops.scan_arrival_tickets"
+SORT_PARAM = "segops.sort_wide_positions"
 
 
 def _array_type_name(kind: str) -> str:
@@ -90,12 +91,12 @@ def entry_points() -> dict:
         _entry("segred_argmax_i32", "[][]i32", [("offsets", "[]i64"), ("lens", "[]i64"), ("vis", "[][]i32")]),
         _entry("bmm_bf16", "[][][]f32", [("A", "[][][]u16"), ("B", "[][][]u16")], [MATMUL_PARAM]),
         _entry("matmul_f32", "[][]f32", [("A", "[][]f32"), ("B", "[][]f32")], [MATMUL_PARAM]),
-        _entry("radix_sort_u32", "[]u32", [("keys", "[]u32")]),
-        _entry("radix_sort_u64", "[]u64", [("keys", "[]u64")]),
+        _entry("radix_sort_u32", "[]u32", [("keys", "[]u32")], [SORT_PARAM]),
+        _entry("radix_sort_u64", "[]u64", [("keys", "[]u64")], [SORT_PARAM]),
     ]
     for k, v in OPAQUE_PAIRS.values():
         eps.append(_entry(f"radix_sort_pairs_{k}_{v}", f"([]{k}, []{v})",
-                          [("keys", f"[]{k}"), ("vals", f"[]{v}")]))
+                          [("keys", f"[]{k}"), ("vals", f"[]{v}")], [SORT_PARAM]))
     eps += [
         _entry("transpose_f32", "[][]f32", [("xss", "[][]f32")]),
         _entry("iota_i64", "[]i64", [("n", "i64")]),

@@ -107,12 +107,17 @@ int fa_version(void);
  *                           most) resident at the same time: for callers that
  *                           know the launch has the device to itself (no CU
  *                           mask, no other kernels that wait for something
- *                           while they hold CUs) */
+ *                           while they hold CUs)
+ *   sort_wide_positions     nonzero: the radix sort counts and scatters with
+ *                           64-bit positions whatever the number of keys (0:
+ *                           only from 2^32 - 1 keys on), so that this path can
+ *                           be exercised without 16 GiB of keys */
 typedef struct fa_tuning {
   int64_t segred_small_threshold;
   int64_t hist_lds_bins_max;
   int64_t matmul_pad_min_work;
   int64_t scan_tickets_by_block;
+  int64_t sort_wide_positions;
 } fa_tuning;
 void fa_set_tuning(const fa_tuning *t); /* NULL: all defaults */
 void fa_get_tuning(fa_tuning *out);     /* the values in effect */

@@ -104,7 +104,8 @@ def test_errors():
 def test_options_that_need_no_input():
     assert run(["--print-params"]).stdout.decode().splitlines() == [
         "segops.hist_lds_bins_max (shared_memory)", "segops.segred_small_threshold (threshold)",
-        "segops.matmul_pad_min_work (threshold)", "segops.scan_arrival_tickets (threshold)"]
+        "segops.matmul_pad_min_work (threshold)", "segops.scan_arrival_tickets (threshold)",
+        "segops.sort_wide_positions (threshold)"]
     assert run(["-h"]).stdout.decode().startswith("Usage: ")
     p = run(["-e", "reduce_add_i32", "-P", "--param", "segops.hist_lds_bins_max=1024"], b"[1, 2, 3]")
     assert p.stdout.decode() == "6i32\n" and b'"events"' in p.stderr

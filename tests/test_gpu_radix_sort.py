@@ -145,3 +145,25 @@ def test_more_than_two_to_the_31_keys(ctx):
     want, have = summary(keys), summary(got)
     assert np.array_equal(want[0], have[0]) and np.array_equal(want[1], have[1])
     assert want[2:] == have[2:]
+
+
+def test_sort_with_64_bit_positions(segops_lib):
+    """From 2^32 - 1 keys on the sort counts, scans and scatters with 64-bit positions; the
+    tuning parameter segops.sort_wide_positions switches to them at any size, so every key and
+    value type goes through that path at sizes the oracle sorts (tests/test_gpu_beyond_2p31.py
+    sorts 2^32 + 4099 u32 keys through it).  Bit-exact, ties in input order."""
+    from futhark_amd import Context
+    with Context(segops_lib, tuning={"segops.sort_wide_positions": 1}) as c:
+        for n in [1, 64, 8191, 8193, 100003, (1 << 21) + 5]:
+            for kt in ("u32", "u64"):
+                keys = dg.uniform_u32(72, n) if kt == "u32" else dg.uniform_u64(73, n)
+                if n > 1000:
+                    keys[::3] = keys[0]          # many ties
+                out = c.call(f"radix_sort_{kt}", [f"{kt}_1d"], c.new(f"{kt}_1d", keys))
+                assert np.array_equal(out.values(), oracle.radix_sort(keys)), (kt, n)
+                out.free()
+                vals = np.arange(n, dtype=np.int32)
+                ko, vo = _sort_pairs(c, kt, keys, vals)
+                wk, wv = oracle.radix_sort(keys, vals)
+                assert np.array_equal(ko.values(), wk) and np.array_equal(vo.values(), wv), (kt, n)
+                ko.free(); vo.free()

@@ -93,4 +93,5 @@ def test_every_function_the_manifest_names_is_exported_and_every_entry_is_listed
     assert entries == {e["cfun"] for e in m["entry_points"].values()}
     tuning = {p for e in m["entry_points"].values() for p in e["tuning_params"]}
     assert tuning == {"segops.hist_lds_bins_max", "segops.segred_small_threshold",
-                      "segops.matmul_pad_min_work", "segops.scan_arrival_tickets"}
+                      "segops.matmul_pad_min_work", "segops.scan_arrival_tickets",
+                      "segops.sort_wide_positions"}
