@@ -214,10 +214,19 @@ def make_workload(name: str, ctx):
             w["cpu_work"] = 2 * rows * m * m
             w["cpu_how"] = (f"rows 0..{rows - 1} of the {b * m} rows of C: parallel over rows, sequential "
                             f"loops over columns and k, B transposed once beforehand (not timed)")
-        elif t == "f16":
-            a, bb = ctx.new("f16_3d", dg.to_f16_bits(A)), ctx.new("f16_3d", dg.to_f16_bits(B))
         else:
-            a, bb = ctx.new("u16_3d", dg.to_bf16_bits(A)), ctx.new("u16_3d", dg.to_bf16_bits(B))
+            bits = dg.to_f16_bits if t == "f16" else dg.to_bf16_bits
+            A16, B16 = bits(A), bits(B)
+            kind = "f16_3d" if t == "f16" else "u16_3d"
+            a, bb = ctx.new(kind, A16), ctx.new(kind, B16)
+            rows = min(b * m, max(16, (1 << 29) // (m * m)))
+            Bt16 = oracle.mc_transpose_16(B16)
+            Cs = np.empty((b, m, m), np.float32)
+            w["cpu"] = lambda: oracle.mc_bmm_rows_16(A16, Bt16, Cs, 0, rows, t == "bf16")
+            w["cpu_work"] = 2 * rows * m * m
+            w["cpu_how"] = (f"rows 0..{rows - 1} of the {b * m} rows of C: parallel over rows, sequential "
+                            f"loops over columns and k, every {t} element widened to f32 where it is used, "
+                            f"B transposed once beforehand (not timed)")
 
         def step():
             ctx.call(f"bmm_{t}", ["f32_3d"], a, bb).free()

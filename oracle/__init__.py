@@ -510,6 +510,32 @@ def mc_bmm_rows_f32(A, Bt, C_out, row_lo: int, row_hi: int, threads: int | None 
     return C_out
 
 
+def mc_transpose_16(B, threads: int | None = None):
+    """[b][K][N] 16-bit payloads -> [b][N][K], in parallel over the rows of the result."""
+    B = _arr(B, np.uint16)
+    b, K, N = B.shape
+    Bt = np.empty((b, N, K), np.uint16)
+    fn = lib().mc_transpose_16
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int]
+    fn(_p(B), _p(Bt), b, K, N, threads or mc_threads())
+    return Bt
+
+
+def mc_bmm_rows_16(A, Bt, C_out, row_lo: int, row_hi: int, bf16: bool, threads: int | None = None):
+    """mc_bmm_rows_f32 for f16 (or bf16) bit patterns: widened where they are used, summed in f32."""
+    A, Bt = _arr(A, np.uint16), _arr(Bt, np.uint16)
+    b, M, K = A.shape
+    N = Bt.shape[1]
+    assert C_out.shape == (b, M, N) and C_out.dtype == np.float32 and C_out.flags.c_contiguous
+    fn = lib().mc_bmm_rows_16
+    fn.restype = None
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                   C.c_int64, C.c_int, C.c_int]
+    fn(_p(A), _p(Bt), _p(C_out), M, N, K, row_lo, row_hi, 1 if bf16 else 0, threads or mc_threads())
+    return C_out
+
+
 def mc_radix_sort(keys, vals=None, threads: int | None = None):
     keys = np.array(keys, copy=True)
     assert keys.dtype in (np.uint32, np.uint64)

@@ -340,6 +340,53 @@ void mc_bmm_rows_f32(const float *A, const float *Bt, float *C, int64_t M, int64
   par_loop(threads, mm_task_f32, &a);
 }
 
+/* The same for 16-bit inputs (f16, or bf16 when `bf16` is nonzero): A and the
+ * transposed copy of B stay 16-bit in memory and every element is widened where
+ * it is used, f32.f16 x * f32.f16 y summed in f32, as a program over f16 arrays
+ * compiles (rts/c/half.h for the conversion; for bf16 the widening is bits << 16). */
+float orc_f16_to_f32(uint16_t h);
+float orc_bf16_to_f32(uint16_t h);
+struct mm_16 { const uint16_t *A, *Bt; float *C; int64_t M, N, K, row_lo, row_hi; int bf16; };
+static void mm_task_16(int tid, int nt, void *p) {
+  struct mm_16 *a = (struct mm_16 *)p;
+  int64_t lo, hi;
+  split(a->row_hi - a->row_lo, tid, nt, &lo, &hi);
+  for (int64_t r = a->row_lo + lo; r < a->row_lo + hi; r++) {
+    const int64_t b = r / a->M;
+    const uint16_t *arow = a->A + r * a->K;
+    const uint16_t *bt = a->Bt + b * a->N * a->K;
+    float *crow = a->C + r * a->N;
+    for (int64_t j = 0; j < a->N; j++) {
+      const uint16_t *bcol = bt + j * a->K;
+      float acc = 0.0f;
+      if (a->bf16)
+        for (int64_t k = 0; k < a->K; k++) acc += orc_bf16_to_f32(arow[k]) * orc_bf16_to_f32(bcol[k]);
+      else
+        for (int64_t k = 0; k < a->K; k++) acc += orc_f16_to_f32(arow[k]) * orc_f16_to_f32(bcol[k]);
+      crow[j] = acc;
+    }
+  }
+}
+struct tr_16 { const uint16_t *B; uint16_t *Bt; int64_t batch, K, N; };
+static void tr_task_16(int tid, int nt, void *p) {
+  struct tr_16 *a = (struct tr_16 *)p;
+  int64_t lo, hi;
+  split(a->batch * a->N, tid, nt, &lo, &hi);
+  for (int64_t r = lo; r < hi; r++) {
+    const int64_t b = r / a->N, j = r % a->N;
+    for (int64_t k = 0; k < a->K; k++) a->Bt[r * a->K + k] = a->B[(b * a->K + k) * a->N + j];
+  }
+}
+void mc_transpose_16(const uint16_t *B, uint16_t *Bt, int64_t batch, int64_t K, int64_t N, int threads) {
+  struct tr_16 t = {B, Bt, batch, K, N};
+  par_loop(threads, tr_task_16, &t);
+}
+void mc_bmm_rows_16(const uint16_t *A, const uint16_t *Bt, float *C, int64_t M, int64_t N, int64_t K,
+                    int64_t row_lo, int64_t row_hi, int bf16, int threads) {
+  struct mm_16 a = {A, Bt, C, M, N, K, row_lo, row_hi, bf16};
+  par_loop(threads, mm_task_16, &a);
+}
+
 /* -------------------------------------------------------------- radix sort
  * The composition the sort is made of, per 8-bit digit from the least
  * significant one: a histogram of the digit per task, an exclusive scan of the

@@ -360,6 +360,17 @@ def test_multicore_baseline_agrees_with_oracle():
     oracle.mc_bmm_rows_f32(A, Bt, Cm, 0, 20, 4)     # a range of rows that crosses a batch boundary
     oracle.mc_bmm_rows_f32(A, Bt, Cm, 20, 51, 4)
     assert np.array_equal(Cm, oracle.bmm_f32(A, B, "lit"))
+    # 16-bit inputs: widened where they are used, so the result is the f32 matmul of the widened
+    # matrices, bit for bit
+    from futhark_amd import datagen as dg
+    for kind, bits in (("f16", dg.to_f16_bits), ("bf16", dg.to_bf16_bits)):
+        A16, B16 = bits(A), bits(B)
+        Bt16 = oracle.mc_transpose_16(B16, 3)
+        assert np.array_equal(Bt16, B16.transpose(0, 2, 1))
+        Cm = np.full((3, 17, 13), np.nan, np.float32)
+        oracle.mc_bmm_rows_16(A16, Bt16, Cm, 0, 30, kind == "bf16", 4)
+        oracle.mc_bmm_rows_16(A16, Bt16, Cm, 30, 51, kind == "bf16", 2)
+        assert np.array_equal(Cm, oracle.bmm_f32(oracle.widen(A16, kind), oracle.widen(B16, kind), "lit")), kind
     # radix sort: stable, keys and (key, value) pairs, against the sequential oracle
     for dt in (np.uint32, np.uint64):
         keys = rng.integers(0, np.iinfo(dt).max, 50_000, dtype=dt)
