@@ -510,8 +510,13 @@ struct rts_event *rts_kernel_begin(struct futhark_context *ctx, const char *name
     l->capacity = l->capacity ? l->capacity * 2 : 64;
     l->events = (struct rts_event *)realloc(l->events, (size_t)l->capacity * sizeof(*l->events));
   }
+  /* The events only measure time (the report is read after a synchronisation
+   * of the stream), so they skip the system-scope fence an event carries by
+   * default: its cache write-back and invalidation would be timed with the
+   * kernel and slow the work that follows. */
   hipEvent_t a = NULL, b = NULL;
-  if (hipEventCreate(&a) != hipSuccess || hipEventCreate(&b) != hipSuccess) {
+  if (hipEventCreateWithFlags(&a, hipEventDisableSystemFence) != hipSuccess ||
+      hipEventCreateWithFlags(&b, hipEventDisableSystemFence) != hipSuccess) {
     if (a) (void)hipEventDestroy(a);
     free(desc);
     return NULL;
