@@ -36,7 +36,58 @@ def test_row_shaped_reductions_and_scans(ctx):
         out = ctx.call(f"scanrows_{op}_{t}", [f"{t}_2d"], a)
         assert np.array_equal(out.values(), oracle.scanrows(op, t, xss)), ("scanrows", n, k, op, t)
         out.free()
+        out = ctx.call(f"vecscan_{op}_{t}", [f"{t}_2d"], a)
+        assert np.array_equal(out.values(), oracle.vecscan(op, t, xss)), ("vecscan", n, k, op, t)
+        out.free()
         a.free()
+
+
+def test_scans_with_a_vector_operator_over_rows_of_every_width(ctx):
+    """vecscan chooses by the bytes of a row: groups of lanes for 16, 32, ... 512 bytes, strips of
+    1 KiB of columns from 256 bytes on (a ragged last strip), transposes for the rest; the rows
+    are cut into chunks whose first pass runs backwards.  Row counts on both sides of a chunk
+    and of a wave-wide load, 4- and 8-byte elements."""
+    rng = np.random.default_rng(2027)
+    for case in range(48):
+        t = ("i32", "i64")[case % 2]
+        es = 4 if t == "i32" else 8
+        op = OPS[case % 4]
+        dt = np.int32 if t == "i32" else np.int64
+        row_bytes = [16, 32, 64, 128, 256, 512, 1024, 1040, 2048, 4000, 4096 + 16, 48][case % 12]
+        k = row_bytes // es
+        n = int(rng.integers(1, max(2, 2_000_000 // k)))
+        if case % 5 == 0:
+            n = (n // 64) * 64 + int(rng.integers(-1, 2))   # around whole wave-wide loads
+        n = max(n, 1)
+        xss = rng.integers(-10**6, 10**6, (n, k)).astype(dt)
+        a = ctx.new(f"{t}_2d", xss)
+        out = ctx.call(f"vecscan_{op}_{t}", [f"{t}_2d"], a)
+        assert np.array_equal(out.values(), oracle.vecscan(op, t, xss)), (n, k, op, t)
+        out.free(); a.free()
+
+
+def test_irregular_segments_of_random_lengths(ctx):
+    """segred over segments with gaps, empty segments, one-element segments and segments of many
+    tiles, laid out at random; integers, exact."""
+    rng = np.random.default_rng(2028)
+    for case in range(24):
+        t = ("i32", "i64")[case % 2]
+        op = ("add", "max", "min")[case % 3]
+        dt = np.int32 if t == "i32" else np.int64
+        m = int(2 ** rng.uniform(0, 14))
+        mean = float(2 ** rng.uniform(0, 12))
+        lens = rng.geometric(1.0 / mean, m).astype(np.int64) - 1      # zeros included
+        if case % 4 == 0:
+            lens[int(rng.integers(0, m))] = int(rng.integers(50_000, 400_000))  # one long segment
+        gaps = (rng.random(m) < 0.1) * rng.integers(0, 5, m)
+        offsets = (np.cumsum(lens + gaps) - lens).astype(np.int64)
+        n = int(offsets[-1] + lens[-1] + int(rng.integers(0, 3)))
+        vs = rng.integers(-10**6, 10**6, n).astype(dt)
+        o, l, v = ctx.new("i64_1d", offsets), ctx.new("i64_1d", lens), ctx.new(f"{t}_1d", vs)
+        out = ctx.call(f"segred_{op}_{t}", [f"{t}_1d"], o, l, v)
+        assert np.array_equal(out.values(), oracle.segred(op, t, offsets, lens, vs)), (case, m, n, op, t)
+        for h in (out, o, l, v):
+            h.free()
 
 
 def test_shaped_histograms(ctx):
