@@ -561,6 +561,9 @@ def main() -> None:
                     help="also run the plain copy kernel (fa_copy, 256 MiB) a few times, so "
                          "that a rocprofv3 --pmc run of this command holds a dispatch of known "
                          "traffic to scale FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--param", action="append", default=[], metavar="NAME=VALUE",
+                    help="a tuning parameter of the program (as futhark bench passes them), "
+                         "e.g. segops.hist_lds_bins_max=16384; may be given several times")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: this build has no multi-GPU path "
@@ -568,7 +571,8 @@ def main() -> None:
 
     from futhark_amd import Context
 
-    ctx = Context(profiling=True)
+    tuning = {k: int(v) for k, v in (p.split("=", 1) for p in args.param)}
+    ctx = Context(profiling=True, tuning=tuning or None)
     ctx.L.futhark_context_pause_profiling(ctx.ptr)
     w = make_workload(args.workload, ctx)
     w["name"] = args.workload
