@@ -99,7 +99,8 @@ extern "C" int fa_copy(fa_stream_t stream, void *dst, const void *src, size_t by
   return launch_status();
 }
 
-extern "C" int fa_version(void) { return 1000; }
+// 1.2: fa_tuning has grown by scan_tickets_by_block (1.1) and sort_wide_positions (1.2).
+extern "C" int fa_version(void) { return 1002; }
 
 extern "C" const char *fa_strerror(int code) {
   if (code == 0) return "success";
