@@ -32,23 +32,32 @@ constexpr int MM_BM = 256, MM_BN = 256;
 constexpr int MM_XCDS = 8;
 constexpr int MM_GROUP_M = 4;
 
-// Block -> C tile.  Consecutive block ids land on different XCDs (id mod 8),
-// each with its own L2.  The ids of one XCD are therefore made consecutive
-// first (id' = xcd * per_xcd + id / 8) and then walked in groups of
-// MM_GROUP_M tile rows, so that the 32 tiles an XCD works on at a time form a
-// compact 4 x 8 patch: it streams 4 row panels of A and 8 column panels of B
-// through its L2 instead of 16 + 2.
-__device__ __forceinline__ void mm_tile_of_block(int &tile_m, int &tile_n) {
+// Block -> (matrix of the batch, C tile).  Blocks are dispatched in the order
+// of their linear id (x fastest, then y, then z) and consecutive ids land on
+// different XCDs (id mod 8), each with its own L2.  The ids of one XCD are
+// therefore made consecutive first (id' = xcd * per_xcd + id / 8), over the
+// whole batch, and then walked matrix by matrix and, inside a matrix, in groups
+// of MM_GROUP_M tile rows: the 32 tiles of a large matrix that an XCD works on
+// at a time form a compact 4 x 8 patch (it streams 4 row panels of A and 8
+// column panels of B through its L2 instead of 16 + 2), and the few tiles of a
+// small matrix of a batch all run on one XCD, where the second tile that needs
+// a panel finds it in L2 (64 products of 512^3 f16, four tiles each: with the
+// tiles of a matrix on four XCDs every panel came from memory twice, 134 MB
+// fetched instead of 67, and the launch took 33 us).
+__device__ __forceinline__ void mm_tile_of_block(int64_t &batch, int &tile_m, int &tile_n) {
   const int tiles_n = gridDim.x, tiles_m = gridDim.y;
-  const int total = tiles_m * tiles_n;
-  int id = blockIdx.y * tiles_n + blockIdx.x;
+  const int64_t per_matrix = (int64_t)tiles_m * tiles_n;
+  const int64_t total = per_matrix * gridDim.z;
+  int64_t id = ((int64_t)blockIdx.z * tiles_m + blockIdx.y) * tiles_n + blockIdx.x;
   if (total % MM_XCDS == 0) id = (id % MM_XCDS) * (total / MM_XCDS) + id / MM_XCDS;
+  batch = id / per_matrix;
+  const int in_matrix = (int)(id % per_matrix);
   const int width = MM_GROUP_M * tiles_n;
-  const int group = id / width;
+  const int group = in_matrix / width;
   const int first_m = group * MM_GROUP_M;
   const int rows = tiles_m - first_m < MM_GROUP_M ? tiles_m - first_m : MM_GROUP_M;
-  tile_m = first_m + (id % width) % rows;
-  tile_n = (id % width) / rows;
+  tile_m = first_m + (in_matrix % width) % rows;
+  tile_n = (in_matrix % width) / rows;
 }
 constexpr int MM_THREADS = 256;
 constexpr int MM_A_ROW_BYTES = 64;                     // one k-step of a row of A
@@ -143,9 +152,9 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void matmul16_kernel(
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / MM16_WAVES_N, wn = wave % MM16_WAVES_N;
-  const int64_t batch = blockIdx.z;
+  int64_t batch;
   int tile_m, tile_n;
-  mm_tile_of_block(tile_m, tile_n);
+  mm_tile_of_block(batch, tile_m, tile_n);
   const int bm = tile_m * MM_BM, bn = tile_n * MM_BN;
   const uint16_t *Ab = A + batch * (int64_t)M * K;
   const uint16_t *Bb = B + batch * (int64_t)K * N;
@@ -367,9 +376,9 @@ __global__ __launch_bounds__(MM_THREADS) void matmul32_kernel(const float *__res
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int64_t batch = blockIdx.z;
+  int64_t batch;
   int tile_m, tile_n;
-  mm_tile_of_block(tile_m, tile_n);
+  mm_tile_of_block(batch, tile_m, tile_n);
   const int bm = tile_m * MM_BM, bn = tile_n * MM_BN;
   const float *Ab = A + batch * (int64_t)M * K;
   const float *Bb = B + batch * (int64_t)K * N;
